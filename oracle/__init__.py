@@ -1,0 +1,223 @@
+"""TEST INFRASTRUCTURE ONLY: numpy-facing binding of the CPU checker (oracle/liboracle.so).
+
+May be imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of bench.py,
+always as the checker and never as the thing measured or shipped.  The arithmetic and the
+reference lines it follows are documented in oracle/oracle.c.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "liboracle.so")
+
+_c = ctypes
+_f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+_f64p = np.ctypeslib.ndpointer(np.float64, flags="C_CONTIGUOUS")
+_u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
+_i64p = np.ctypeslib.ndpointer(np.int64, flags="C_CONTIGUOUS")
+
+
+def build():
+    """Compile oracle/liboracle.so with the committed Makefile."""
+    subprocess.check_call(["make", "-C", _HERE, "-s"])
+
+
+def _load():
+    if not os.path.exists(_SO):
+        build()
+    lib = ctypes.CDLL(_SO)
+    lib.cn_oracle_table.argtypes = [_f32p]
+    for name in ("cn_oracle_compress_literal", "cn_oracle_compress_closed"):
+        getattr(lib, name).argtypes = [_f32p, _c.c_float, _c.c_size_t, _u8p, _c.c_int]
+    lib.cn_oracle_decode_lut.argtypes = [_c.c_float, _f32p]
+    lib.cn_oracle_decompress.argtypes = [_u8p, _c.c_float, _c.c_size_t, _f32p]
+    lib.cn_oracle_absmax.argtypes = [_f32p, _c.c_size_t]
+    lib.cn_oracle_absmax.restype = _c.c_float
+    g = [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _f32p, _c.c_int64, _f32p,
+         _c.c_int64, _f32p, _c.c_int64]
+    lib.cn_oracle_gemm_f64acc.argtypes = g
+    lib.cn_oracle_gemm_f32_seqfma.argtypes = g
+    lib.cn_oracle_gemm_f64acc_abs.argtypes = [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64,
+                                              _c.c_int64, _f32p, _c.c_int64, _f32p, _c.c_int64,
+                                              _f64p, _f64p]
+    lib.cn_oracle_gemm_cols_f64acc.argtypes = [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _f32p,
+                                               _c.c_int64, _f32p, _c.c_int64, _i64p, _c.c_int64,
+                                               _f64p, _f64p]
+    lib.cn_oracle_gemm_w8_f64acc.argtypes = [_c.c_int64, _c.c_int64, _c.c_int64, _f32p,
+                                             _c.c_int64, _u8p, _c.c_int64, _c.c_float, _f32p,
+                                             _c.c_int64]
+    lib.cn_oracle_add_row_vector.argtypes = [_f32p, _f32p, _c.c_int64, _c.c_int64, _f32p]
+    lib.cn_oracle_maxout.argtypes = [_f32p, _c.c_int64, _c.c_int64, _c.c_int, _f32p, _f32p]
+    lib.cn_oracle_expand_to_maxout_grad.argtypes = [_f32p, _f32p, _c.c_int64, _c.c_int64,
+                                                    _c.c_int, _f32p]
+    lib.cn_oracle_softmax.argtypes = [_f32p, _c.c_int64, _c.c_int64, _f32p]
+    lib.cn_oracle_num_threads.restype = _c.c_int
+    lib.cn_oracle_set_threads.argtypes = [_c.c_int]
+    lib.cn_port_compress.argtypes = [_f32p, _c.c_float, _c.c_size_t, _u8p]
+    lib.cn_port_decompress.argtypes = [_u8p, _c.c_float, _c.c_size_t, _f32p]
+    lib.cn_port_absmax.argtypes = [_f32p, _c.c_size_t]
+    lib.cn_port_absmax.restype = _c.c_float
+    lib.cn_port_gemm_nn.argtypes = [_c.c_int64, _c.c_int64, _c.c_int64, _f32p, _c.c_int64, _f32p,
+                                    _c.c_int64, _f32p, _c.c_int64]
+    return lib
+
+
+_lib = _load()
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def table():
+    t = np.empty(126, np.float32)
+    _lib.cn_oracle_table(t)
+    return t
+
+
+def compress(x, precision, sliver_rule=0, form="literal"):
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint8)
+    fn = _lib.cn_oracle_compress_literal if form == "literal" else _lib.cn_oracle_compress_closed
+    fn(x.reshape(-1), float(precision), x.size, out.reshape(-1), int(sliver_rule))
+    return out
+
+
+def decode_lut(precision):
+    lut = np.empty(256, np.float32)
+    _lib.cn_oracle_decode_lut(float(precision), lut)
+    return lut
+
+
+def decompress(codes, precision):
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.empty(codes.shape, np.float32)
+    _lib.cn_oracle_decompress(codes.reshape(-1), float(precision), codes.size, out.reshape(-1))
+    return out
+
+
+def absmax(x):
+    x = _f32(x)
+    return float(_lib.cn_oracle_absmax(x.reshape(-1), x.size))
+
+
+def _gemm_dims(A, B, ta, tb):
+    M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+    K2, N = (B.shape[1], B.shape[0]) if tb else B.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ: %d vs %d" % (K, K2))
+    return M, N, K
+
+
+def gemm(A, B, ta=False, tb=False, mode="f64acc"):
+    """C = op(A) op(B) on row-major arrays; mode 'f64acc' (yard-stick) or 'seqfma'."""
+    A, B = _f32(A), _f32(B)
+    M, N, K = _gemm_dims(A, B, ta, tb)
+    C = np.empty((M, N), np.float32)
+    fn = _lib.cn_oracle_gemm_f64acc if mode == "f64acc" else _lib.cn_oracle_gemm_f32_seqfma
+    fn(int(ta), int(tb), M, N, K, A, A.shape[1], B, B.shape[1], C, N)
+    return C
+
+
+def gemm_with_abs(A, B, ta=False, tb=False):
+    """(C, sum_k |a||b|) in float64."""
+    A, B = _f32(A), _f32(B)
+    M, N, K = _gemm_dims(A, B, ta, tb)
+    C = np.empty((M, N), np.float64)
+    Cabs = np.empty((M, N), np.float64)
+    _lib.cn_oracle_gemm_f64acc_abs(int(ta), int(tb), M, N, K, A, A.shape[1], B, B.shape[1], C, Cabs)
+    return C, Cabs
+
+
+def gemm_cols(A, B, cols, ta=False, tb=False):
+    """Selected output columns, float64: returns (C[:, cols], sum_k|a||b|[:, cols])."""
+    A, B = _f32(A), _f32(B)
+    M, N, K = _gemm_dims(A, B, ta, tb)
+    cols = np.ascontiguousarray(cols, dtype=np.int64)
+    C = np.empty((M, cols.size), np.float64)
+    Cabs = np.empty((M, cols.size), np.float64)
+    _lib.cn_oracle_gemm_cols_f64acc(int(ta), int(tb), M, K, A, A.shape[1], B, B.shape[1], cols,
+                                    cols.size, C, Cabs)
+    return C, Cabs
+
+
+def gemm_w8(A, W, scale):
+    A = _f32(A)
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    M, K = A.shape
+    K2, N = W.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ")
+    C = np.empty((M, N), np.float32)
+    _lib.cn_oracle_gemm_w8_f64acc(M, N, K, A, K, W, N, float(scale), C, N)
+    return C
+
+
+def add_row_vector(A, v):
+    A, v = _f32(A), _f32(v).reshape(-1)
+    out = np.empty_like(A)
+    _lib.cn_oracle_add_row_vector(A, v, A.shape[0], A.shape[1], out)
+    return out
+
+
+def maxout(A, pool):
+    A = _f32(A)
+    out = np.empty((A.shape[0], A.shape[1] // pool), np.float32)
+    arg = np.empty_like(out)
+    _lib.cn_oracle_maxout(A, A.shape[0], A.shape[1], int(pool), out, arg)
+    return out, arg
+
+
+def expand_to_maxout_grad(err, argmax, pool):
+    err, argmax = _f32(err), _f32(argmax)
+    out = np.empty((err.shape[0], err.shape[1] * pool), np.float32)
+    _lib.cn_oracle_expand_to_maxout_grad(err, argmax, err.shape[0], err.shape[1], int(pool), out)
+    return out
+
+
+def softmax(A):
+    A = _f32(A)
+    out = np.empty_like(A)
+    _lib.cn_oracle_softmax(A, A.shape[0], A.shape[1], out)
+    return out
+
+
+def num_threads():
+    return int(_lib.cn_oracle_num_threads())
+
+
+def set_threads(n):
+    _lib.cn_oracle_set_threads(int(n))
+
+
+def port_compress(x, precision):
+    x = _f32(x)
+    out = np.empty(x.shape, np.uint8)
+    _lib.cn_port_compress(x.reshape(-1), float(precision), x.size, out.reshape(-1))
+    return out
+
+
+def port_decompress(codes, precision):
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.empty(codes.shape, np.float32)
+    _lib.cn_port_decompress(codes.reshape(-1), float(precision), codes.size, out.reshape(-1))
+    return out
+
+
+def port_absmax(x):
+    x = _f32(x)
+    return float(_lib.cn_port_absmax(x.reshape(-1), x.size))
+
+
+def port_gemm_nn(A, B):
+    A, B = _f32(A), _f32(B)
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ")
+    C = np.empty((M, N), np.float32)
+    _lib.cn_port_gemm_nn(M, N, K, A, K, B, N, C, N)
+    return C

@@ -1,0 +1,300 @@
+/* TEST INFRASTRUCTURE ONLY.
+ *
+ * CPU restatement of the arithmetic of clusterNet's matrix-multiply + 8-bit codec path, used as
+ * the checker by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of bench.py.
+ * Nothing in the shipped library links, loads or calls this file.
+ *
+ * What each function follows in the reference (paths under the reference tree):
+ *   cn_oracle_compress_literal   source/clusterKernels.cu:1163-1232 (kCompression_8bit), launched
+ *                                flat over A->size by source/basicOps.cu:1163-1168
+ *   cn_oracle_compress_closed    same kernel, second independent formulation (count of odd
+ *                                table entries below the input, then a two-candidate pick)
+ *   cn_oracle_decompress         source/clusterKernels.cu:1135-1160 (kDecompression_8bit)
+ *   cn_oracle_absmax             source/basicOps.cu:810-822 + source/clusterKernels.cu:429-436
+ *                                (abs) followed by source/basicOps.cu:1076-1081 (max)
+ *   cn_oracle_gemm_*             source/clusterNet.cpp:404-461: C = op(A) op(B), alpha 1, beta 0,
+ *                                shape rule of source/basicOps.cu:839-864.  The arithmetic of the
+ *                                reference lives in cuBLAS (cublasSgemm, version unpinned by
+ *                                Makefile:13-15, not in the tree); the textbook product is
+ *                                restated here and pinned by the reference's known-answer tests
+ *                                tests/clusterNet_test.cu:67-84,106-129,158-165,257-276,338-394.
+ *   cn_oracle_gemm_w8            C = A * decode(W codes, scale) with decode == cn_oracle_decompress
+ *                                (no counterpart kernel in the reference; its nearest relatives
+ *                                are kDot8bit / kDot8bit_shared, source/clusterKernels.cu:1717-1843)
+ *   helpers of the training step source/clusterKernels.cu:706-718 (bias add), :1432-1458
+ *                                (maxout), :1481-1495 (expand to maxout grad), :651-688 (softmax);
+ *                                definitions taken from the brute-force expectations in
+ *                                tests/basicOps_test.cu:580-638 and :279-300, not from the kernels
+ *                                (which skip rows / mis-index at large sizes).
+ *
+ * Pinning status.  The reference holds no test vector for the codec (nothing under its tests/
+ * touches compression_8bit / decompression_8bit), so the codec is pinned by: the table bytes of
+ * source/8bit_floats.hdf5; agreement of the two independent formulations on every table value,
+ * neighbour, midpoint, threshold and on random data; hand-traced cases; and the monotonicity /
+ * fixed-point invariants the procedure implies (tests/test_oracle_codec.py).
+ * One input range has no defined result in the reference: for 0.99140614 < |x|/precision <=
+ * 0.995703 the search reads tbl_floats[126], which the kernel never writes
+ * (source/clusterKernels.cu:1176-1178 vs :1220).  PARITY UNPINNED for that range: this file pins
+ * it by decision (sliver_rule 0: the slot holds 1.0f, giving code 125/253; sliver_rule 1: the slot
+ * holds 0.0f, giving 126/254).  The shipped library implements rule 0.
+ * cn_oracle_absmax on inputs containing NaN is likewise PARITY UNPINNED (thrust's reduction order
+ * decides whether a NaN survives); this file propagates NaN.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <string.h>
+#include <stdlib.h>
+
+#include "table_8bit.h"
+
+static float bits_to_float(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static uint32_t float_to_bits(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+void cn_oracle_table(float out[126]) {
+    for (int i = 0; i < 126; ++i) out[i] = bits_to_float(cn_oracle_table_bits[i]);
+}
+
+/* The 128-slot working copy of the table the compression kernel keeps in shared memory:
+ * slots 0..125 loaded, slot 126 per the sliver rule, slot 127 never read. */
+static void load_slots(float slot[128], int sliver_rule) {
+    cn_oracle_table(slot);
+    slot[126] = (sliver_rule == 0) ? 1.0f : 0.0f;
+    slot[127] = 0.0f;
+}
+
+/* One element of the literal search.  Volatile-free plain float arithmetic: x86-64 SSE keeps
+ * every intermediate in binary32, as the device does. */
+static uint8_t compress_one_literal(const float slot[128], float x, float precision) {
+    const float below = 0.0000015f; /* float(0.0000015) */
+    const float above = 0.995703f;  /* float(0.995703)  */
+    float a = x / precision;
+    int neg = 0;
+    if (a < 0.0f) { neg = 1; a = -a; }
+    if (a < below) return (uint8_t)254;
+    if (a > above) return neg ? (uint8_t)255 : (uint8_t)127;
+    int lo = 0, hi = 125, p = 63;
+    for (int step = 32; step > 0; step >>= 1) {
+        if (a > slot[p]) { lo = p; p += step; }
+        else             { hi = p; p -= step; }
+    }
+    int c;
+    if (lo == p) c = (fabsf(slot[p] - a) < (slot[hi] - a)) ? p : hi;
+    else         c = ((slot[p] - a) < fabsf(slot[lo] - a)) ? p : lo;
+    return (uint8_t)(neg ? (c | 0x80) : c);
+}
+
+void cn_oracle_compress_literal(const float *x, float precision, size_t n, uint8_t *codes,
+                                int sliver_rule) {
+    float slot[128];
+    load_slots(slot, sliver_rule);
+    for (size_t i = 0; i < n; ++i) codes[i] = compress_one_literal(slot, x[i], precision);
+}
+
+/* Second formulation.  q = 2 * #{odd p in 1,3,..,125 : a > t[p]}.  The search always ends with
+ * its pivot on the even slot q; the candidates are q and its lower odd neighbour (q == 0: slots
+ * 0 and 1). */
+static uint8_t compress_one_closed(const float slot[128], float x, float precision) {
+    float a = x / precision;
+    int neg = 0;
+    if (a < 0.0f) { neg = 1; a = -a; }
+    if (a < 0.0000015f) return (uint8_t)254;
+    if (a > 0.995703f) return neg ? (uint8_t)255 : (uint8_t)127;
+    int q = 0;
+    for (int p = 1; p <= 125; p += 2) q += (a > slot[p]) ? 2 : 0;
+    int c;
+    if (q == 0) c = (fabsf(slot[0] - a) < (slot[1] - a)) ? 0 : 1;
+    else        c = ((slot[q] - a) < fabsf(slot[q - 1] - a)) ? q : q - 1;
+    return (uint8_t)(neg ? (c | 0x80) : c);
+}
+
+void cn_oracle_compress_closed(const float *x, float precision, size_t n, uint8_t *codes,
+                               int sliver_rule) {
+    float slot[128];
+    load_slots(slot, sliver_rule);
+    for (size_t i = 0; i < n; ++i) codes[i] = compress_one_closed(slot, x[i], precision);
+}
+
+/* The 256-entry decode table for one precision. */
+void cn_oracle_decode_lut(float precision, float lut[256]) {
+    float t[126];
+    cn_oracle_table(t);
+    for (int i = 0; i < 126; ++i) {
+        lut[i] = t[i] * precision;
+        lut[i + 128] = -lut[i];
+    }
+    lut[126] = precision;
+    lut[254] = precision; /* the "zero" code decodes to +precision in the reference */
+    lut[127] = precision;
+    lut[255] = -precision;
+}
+
+void cn_oracle_decompress(const uint8_t *codes, float precision, size_t n, float *out) {
+    float lut[256];
+    cn_oracle_decode_lut(precision, lut);
+    for (size_t i = 0; i < n; ++i) out[i] = lut[codes[i]];
+}
+
+/* max_i |x_i|, start value -1 as in the reference's reduction; NaN propagates. */
+float cn_oracle_absmax(const float *x, size_t n) {
+    float best = -1.0f;
+    int saw_nan = 0;
+    for (size_t i = 0; i < n; ++i) {
+        float v = fabsf(x[i]);
+        if (v != v) saw_nan = 1;
+        if (best < v) best = v;
+    }
+    return saw_nan ? NAN : best;
+}
+
+/* ---- GEMM: row-major storage, C[M x N] = op(A) op(B).
+ * trans_a == 0: A stored M x K (lda >= K), else A stored K x M (lda >= M).
+ * trans_b == 0: B stored K x N (ldb >= N), else B stored N x K (ldb >= K). */
+static inline float a_at(const float *A, int64_t lda, int ta, int64_t m, int64_t k) {
+    return ta ? A[k * lda + m] : A[m * lda + k];
+}
+static inline float b_at(const float *B, int64_t ldb, int tb, int64_t k, int64_t n) {
+    return tb ? B[n * ldb + k] : B[k * ldb + n];
+}
+
+/* fp64-accumulated yard-stick (products formed in fp64 too). */
+void cn_oracle_gemm_f64acc(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A,
+                           int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        double *row = (double *)calloc((size_t)N, sizeof(double));
+        for (int64_t k = 0; k < K; ++k) {
+            double av = (double)a_at(A, lda, ta, m, k);
+            if (!tb) {
+                const float *brow = B + k * ldb;
+                for (int64_t n = 0; n < N; ++n) row[n] += av * (double)brow[n];
+            } else {
+                for (int64_t n = 0; n < N; ++n) row[n] += av * (double)B[n * ldb + k];
+            }
+        }
+        for (int64_t n = 0; n < N; ++n) C[m * ldc + n] = (float)row[n];
+        free(row);
+    }
+}
+
+/* Same as above but also returns sum_k |a||b| per output (the forward-error denominator). */
+void cn_oracle_gemm_f64acc_abs(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A,
+                               int64_t lda, const float *B, int64_t ldb, double *C, double *Cabs) {
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        for (int64_t n = 0; n < N; ++n) {
+            double s = 0.0, sa = 0.0;
+            for (int64_t k = 0; k < K; ++k) {
+                double p = (double)a_at(A, lda, ta, m, k) * (double)b_at(B, ldb, tb, k, n);
+                s += p;
+                sa += fabs(p);
+            }
+            C[m * N + n] = s;
+            Cabs[m * N + n] = sa;
+        }
+    }
+}
+
+/* Sequential-k single-precision fused multiply-add accumulation: the order that reproduces the
+ * literals of the reference's known-answer tests exactly. */
+void cn_oracle_gemm_f32_seqfma(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A,
+                               int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc) {
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            float s = 0.0f;
+            for (int64_t k = 0; k < K; ++k)
+                s = fmaf(a_at(A, lda, ta, m, k), b_at(B, ldb, tb, k, n), s);
+            C[m * ldc + n] = s;
+        }
+}
+
+/* Selected output columns only (full-size spot checks): C[m][j] = sum_k opA[m][k] opB[k][cols[j]],
+ * fp64 accumulation, C is M x ncols dense. */
+void cn_oracle_gemm_cols_f64acc(int ta, int tb, int64_t M, int64_t K, const float *A, int64_t lda,
+                                const float *B, int64_t ldb, const int64_t *cols, int64_t ncols,
+                                double *C, double *Cabs) {
+#pragma omp parallel for schedule(dynamic, 4)
+    for (int64_t j = 0; j < ncols; ++j) {
+        int64_t n = cols[j];
+        for (int64_t m = 0; m < M; ++m) {
+            double s = 0.0, sa = 0.0;
+            for (int64_t k = 0; k < K; ++k) {
+                double p = (double)a_at(A, lda, ta, m, k) * (double)b_at(B, ldb, tb, k, n);
+                s += p;
+                sa += fabs(p);
+            }
+            C[m * ncols + j] = s;
+            if (Cabs) Cabs[m * ncols + j] = sa;
+        }
+    }
+}
+
+/* C = A (M x K, row-major) times decode(W codes K x N, scale). */
+void cn_oracle_gemm_w8_f64acc(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                              const uint8_t *W, int64_t ldw, float scale, float *C, int64_t ldc) {
+    float lut[256];
+    cn_oracle_decode_lut(scale, lut);
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        double *row = (double *)calloc((size_t)N, sizeof(double));
+        for (int64_t k = 0; k < K; ++k) {
+            double av = (double)A[m * lda + k];
+            const uint8_t *wrow = W + k * ldw;
+            for (int64_t n = 0; n < N; ++n) row[n] += av * (double)lut[wrow[n]];
+        }
+        for (int64_t n = 0; n < N; ++n) C[m * ldc + n] = (float)row[n];
+        free(row);
+    }
+}
+
+/* ---- helpers of the training step (row-major, flat). */
+
+/* out[r][c] = A[r][c] + v[c]   (bias broadcast over rows) */
+void cn_oracle_add_row_vector(const float *A, const float *v, int64_t rows, int64_t cols,
+                              float *out) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) out[r * cols + c] = A[r * cols + c] + v[c];
+}
+
+/* Maxout over `pool` consecutive columns: out is rows x cols/pool; argmax holds the absolute
+ * column index of the winner as a float (first maximum wins). */
+void cn_oracle_maxout(const float *A, int64_t rows, int64_t cols, int pool, float *out,
+                      float *argmax) {
+    int64_t oc = cols / pool;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t o = 0; o < oc; ++o) {
+            int64_t best = o * pool;
+            float bv = A[r * cols + best];
+            for (int p = 1; p < pool; ++p) {
+                float v = A[r * cols + o * pool + p];
+                if (v > bv) { bv = v; best = o * pool + p; }
+            }
+            out[r * oc + o] = bv;
+            argmax[r * oc + o] = (float)best;
+        }
+}
+
+/* Scatter each pooled error to its winner's column; everything else is zero. */
+void cn_oracle_expand_to_maxout_grad(const float *err, const float *argmax, int64_t rows,
+                                     int64_t pooled_cols, int pool, float *out) {
+    int64_t cols = pooled_cols * pool;
+    for (int64_t i = 0; i < rows * cols; ++i) out[i] = 0.0f;
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t o = 0; o < pooled_cols; ++o)
+            out[r * cols + (int64_t)argmax[r * pooled_cols + o]] = err[r * pooled_cols + o];
+}
+
+/* Row-wise softmax with max subtraction, fp64 internally. */
+void cn_oracle_softmax(const float *A, int64_t rows, int64_t cols, float *out) {
+    for (int64_t r = 0; r < rows; ++r) {
+        double mx = -INFINITY, s = 0.0;
+        for (int64_t c = 0; c < cols; ++c) if (A[r * cols + c] > mx) mx = A[r * cols + c];
+        for (int64_t c = 0; c < cols; ++c) s += exp((double)A[r * cols + c] - mx);
+        for (int64_t c = 0; c < cols; ++c)
+            out[r * cols + c] = (float)(exp((double)A[r * cols + c] - mx) / s);
+    }
+}
+
+/* ---- bit helpers for the tests */
+uint32_t cn_oracle_float_bits(float f) { return float_to_bits(f); }
+float cn_oracle_bits_float(uint32_t u) { return bits_to_float(u); }

@@ -1,0 +1,98 @@
+"""Pins the CPU GEMM checker against the reference's own known-answer tests (no GPU needed).
+
+Literals come from tests/clusterNet_test.cu of the reference: :22-23 (operands), :72-75 (dot),
+:111-119 and :125-128 (Tdot), :161-164 (dotT), :257-276 (0.3 x 1.1748345 all-constant product),
+:338-394 (all-ones closed forms 8783, 317, 17).  The reference compares with exact float
+equality; sequential-k fp32 FMA accumulation reproduces every literal bit for bit.
+"""
+import numpy as np
+
+import oracle
+
+M1 = np.array([[0, 2, 3], [0, 0.83, 59.1387]], np.float32)
+M2 = np.array([[17, 0], [3, 4], [0, 0]], np.float32)
+f32 = lambda rows: np.array(rows, np.float32)
+
+
+def test_reference_kats_exact_with_seqfma():
+    assert np.array_equal(oracle.gemm(M1, M2, mode="seqfma"), f32([[6, 8], [2.49, 3.32]]))
+    assert np.array_equal(oracle.gemm(M1, M1, ta=True, mode="seqfma"),
+                          f32([[0, 0, 0], [0, 4.6889, 55.085117], [0, 55.085117, 3506.385742]]))
+    assert np.array_equal(oracle.gemm(M2, M2, ta=True, mode="seqfma"), f32([[298, 12], [12, 16]]))
+    assert np.array_equal(oracle.gemm(M1, M1, tb=True, mode="seqfma"),
+                          f32([[13, 179.0761], [179.0761, 3498.074463]]))
+
+
+def test_reference_kats_f64acc_within_one_ulp():
+    for got, want in (
+        (oracle.gemm(M1, M2), f32([[6, 8], [2.49, 3.32]])),
+        (oracle.gemm(M1, M1, ta=True), f32([[0, 0, 0], [0, 4.6889, 55.085117],
+                                           [0, 55.085117, 3506.385742]])),
+        (oracle.gemm(M1, M1, tb=True), f32([[13, 179.0761], [179.0761, 3498.074463]])),
+    ):
+        np.testing.assert_allclose(got, want, rtol=1.2e-7, atol=0)
+
+
+def test_all_ones_closed_forms():
+    assert np.all(oracle.gemm(np.ones((111, 8783), np.float32), np.ones((8783, 317), np.float32)) == 8783.0)
+    # dotT(m3 17x317, m1 8783x317) -> 17 x 8783 of 317
+    assert np.all(oracle.gemm(np.ones((17, 317), np.float32), np.ones((8783, 317), np.float32), tb=True) == 317.0)
+    assert np.all(oracle.gemm(np.ones((8783, 17), np.float32), np.ones((17, 317), np.float32)) == 17.0)
+
+
+def test_constant_product():
+    a = np.full((200, 400), 0.3, np.float32)
+    b = np.full((400, 800), np.float32(1.0) + np.float32(0.1748345), np.float32)
+    c = oracle.gemm(a, b)
+    want = np.float32(400 * float(np.float32(0.3)) * float(b[0, 0]))
+    assert c.shape == (200, 800) and np.all(c == want)
+
+
+def test_transpose_identities_and_numpy_cross_check():
+    rng = np.random.default_rng(0)
+    A = rng.uniform(0, 1, (37, 53)).astype(np.float32)
+    B = rng.normal(0, 1, (53, 29)).astype(np.float32)
+    want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(oracle.gemm(A, B), want)
+    assert np.array_equal(oracle.gemm(np.ascontiguousarray(A.T), B, ta=True), want)
+    assert np.array_equal(oracle.gemm(A, np.ascontiguousarray(B.T), tb=True), want)
+    np.testing.assert_allclose(oracle.gemm(A, B, mode="seqfma"), want, rtol=2e-5, atol=1e-5)
+    np.testing.assert_allclose(oracle.port_gemm_nn(A, B), want, rtol=2e-5, atol=1e-5)
+    C, Cabs = oracle.gemm_with_abs(A, B)
+    np.testing.assert_allclose(C, A.astype(np.float64) @ B.astype(np.float64), rtol=1e-12)
+    np.testing.assert_allclose(Cabs, np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64), rtol=1e-12)
+    cols = np.array([0, 5, 28])
+    Cc, _ = oracle.gemm_cols(A, B, cols)
+    np.testing.assert_allclose(Cc, C[:, cols], rtol=1e-12)
+
+
+def test_w8_gemm_is_gemm_of_decoded_weights():
+    rng = np.random.default_rng(2)
+    A = rng.normal(0, 1, (9, 40)).astype(np.float32)
+    W = rng.integers(0, 256, (40, 13), dtype=np.uint8)
+    assert np.array_equal(oracle.gemm_w8(A, W, 0.37), oracle.gemm(A, oracle.decompress(W, 0.37)))
+
+
+def test_training_step_helpers_brute_force():
+    rng = np.random.default_rng(4)
+    A = rng.normal(0, 1, (7, 12)).astype(np.float32)
+    v = rng.normal(0, 1, 12).astype(np.float32)
+    assert np.array_equal(oracle.add_row_vector(A, v), A + v[None, :])
+    for pool in (2, 3, 4):
+        out, arg = oracle.maxout(A, pool)
+        blocks = A.reshape(7, 12 // pool, pool)
+        assert np.array_equal(out, blocks.max(axis=2))
+        assert np.array_equal(arg, (blocks.argmax(axis=2) + np.arange(12 // pool)[None, :] * pool).astype(np.float32))
+        err = rng.normal(0, 1, out.shape).astype(np.float32)
+        g = oracle.expand_to_maxout_grad(err, arg, pool)
+        want = np.zeros_like(A)
+        for r in range(7):
+            for o in range(12 // pool):
+                want[r, int(arg[r, o])] = err[r, o]
+        assert np.array_equal(g, want)
+    s = oracle.softmax(np.zeros((5, 10), np.float32))
+    assert np.allclose(s, 0.1)
+    s = oracle.softmax(A)
+    np.testing.assert_allclose(s.sum(axis=1), 1.0, rtol=1e-6)
+    e = np.exp(A.astype(np.float64) - A.max(axis=1, keepdims=True))
+    np.testing.assert_allclose(s, e / e.sum(axis=1, keepdims=True), rtol=1e-6)
