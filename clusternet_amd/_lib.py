@@ -1,0 +1,187 @@
+"""ctypes binding of libcnhip.so.  No computation happens here and there is no CPU fallback: if
+the library is missing or no GPU is usable, calls raise."""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_PATH = os.path.join(_HERE, "libcnhip.so")
+_lib = None
+
+
+class CnError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__("libcnhip status %d: %s" % (status, message))
+        self.status = status
+
+
+def lib_path():
+    return _PATH
+
+
+def lib():
+    """Loads libcnhip.so (after torch, so that both share one HIP runtime)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_PATH):
+        raise ImportError("%s is not built; run `python -m clusternet_amd.build`" % _PATH)
+    try:
+        import torch  # noqa: F401  (loads the HIP runtime that owns the tensors we are handed)
+    except ImportError:
+        pass
+    L = C.CDLL(_PATH)
+    i64, vp, f32, sz = C.c_int64, C.c_void_p, C.c_float, C.c_size_t
+    L.cn_status_string.restype = C.c_char_p
+    L.cn_status_string.argtypes = [C.c_int]
+    L.cn_last_error.restype = C.c_char_p
+    L.cn_init.argtypes = [C.c_int]
+    L.cn_num_compute_units.restype = C.c_int
+    L.cn_malloc.argtypes = [C.POINTER(vp), sz]
+    L.cn_free.argtypes = [vp]
+    L.cn_memcpy_h2d.argtypes = [vp, vp, sz]
+    L.cn_memcpy_d2h.argtypes = [vp, vp, sz]
+    L.cn_memcpy_d2d.argtypes = [vp, vp, sz, vp]
+    L.cn_fill_f32.argtypes = [vp, f32, sz, vp]
+    L.cn_synchronize.argtypes = [vp]
+    L.cn_table_get.argtypes = [C.POINTER(f32)]
+    L.cn_gemm_f32.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp]
+    L.cn_gemm_f32_w8.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, vp, i64, vp]
+    L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
+    L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
+    L.cn_compress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
+    L.cn_decompress_8bit.argtypes = [vp, f32, sz, vp, vp]
+    L.cn_decompress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
+    L.cn_host_encode_lut_lookup.argtypes = [C.c_uint32, C.POINTER(C.c_int)]
+    L.cn_host_encode_magnitude.argtypes = [f32]
+    L.cn_host_plan_gemm.argtypes = [i64, i64, i64, C.c_int, sz, C.POINTER(i64)]
+    L.cn_host_plan_gemm.restype = None
+    _lib = L
+    return L
+
+
+def check(status):
+    if status != 0:
+        L = lib()
+        raise CnError(status, "%s: %s" % (L.cn_status_string(status).decode(), L.cn_last_error().decode()))
+
+
+def init(device=0):
+    check(lib().cn_init(int(device)))
+
+
+def num_compute_units():
+    return int(lib().cn_num_compute_units())
+
+
+def table():
+    import numpy as np
+    buf = (C.c_float * 126)()
+    check(lib().cn_table_get(buf))
+    return np.frombuffer(buf, dtype=np.float32).copy()
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(t, dtype, what):
+    import torch
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype):
+        raise TypeError("%s must be a CUDA/HIP tensor of dtype %s" % (what, dtype))
+    if t.dim() == 2 and t.stride(1) != 1 and t.shape[1] > 1:
+        raise ValueError("%s must be row-major (unit column stride)" % what)
+
+
+def _ld(t):
+    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
+
+
+def gemm(A, B, trans_a=False, trans_b=False, out=None):
+    """out = op(A) op(B) on row-major fp32 matrices; mirrors ClusterNet::dot(A,B,out,T1,T2)."""
+    import torch
+    _need(A, torch.float32, "A")
+    _need(B, torch.float32, "B")
+    M, K = (A.shape[1], A.shape[0]) if trans_a else A.shape
+    K2, N = (B.shape[1], B.shape[0]) if trans_b else B.shape
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=A.device)
+    _need(out, torch.float32, "out")
+    if K != K2 or tuple(out.shape) != (M, N):
+        raise CnError(2, "Matrix size error: op(A) %dx%d, op(B) %dx%d, out %dx%d"
+                      % (M, K, K2, N, out.shape[0], out.shape[1]))
+    check(lib().cn_gemm_f32(int(trans_a), int(trans_b), M, N, K, A.data_ptr(), _ld(A), B.data_ptr(),
+                            _ld(B), out.data_ptr(), _ld(out), _stream()))
+    return out
+
+
+def dot(A, B, out=None):
+    return gemm(A, B, False, False, out)
+
+
+def Tdot(A, B, out=None):
+    return gemm(A, B, True, False, out)
+
+
+def dotT(A, B, out=None):
+    return gemm(A, B, False, True, out)
+
+
+def gemm_w8(A, W, scale, out=None):
+    """out = A decode(W, scale): A fp32 M x K, W uint8 codes K x N."""
+    import torch
+    _need(A, torch.float32, "A")
+    _need(W, torch.uint8, "W")
+    M, K = A.shape
+    K2, N = W.shape
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=A.device)
+    _need(out, torch.float32, "out")
+    if K != K2 or tuple(out.shape) != (M, N):
+        raise CnError(2, "Matrix size error")
+    check(lib().cn_gemm_f32_w8(M, N, K, A.data_ptr(), _ld(A), W.data_ptr(), _ld(W), float(scale),
+                               out.data_ptr(), _ld(out), _stream()))
+    return out
+
+
+def absmax(x, out=None):
+    """Device scalar max|x| (one-element fp32 tensor)."""
+    import torch
+    _need(x, torch.float32, "x")
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    if out is None:
+        out = torch.empty(1, dtype=torch.float32, device=x.device)
+    check(lib().cn_absmax_f32(x.data_ptr(), x.numel(), out.data_ptr(), _stream()))
+    return out
+
+
+def compression_8bit(A, precision, out=None):
+    """uint8 codes of A / precision; precision is a float or a one-element device tensor."""
+    import torch
+    _need(A, torch.float32, "A")
+    if not A.is_contiguous():
+        raise ValueError("A must be contiguous")
+    if out is None:
+        out = torch.empty(A.shape, dtype=torch.uint8, device=A.device)
+    _need(out, torch.uint8, "out")
+    if isinstance(precision, torch.Tensor):
+        check(lib().cn_compress_8bit_dp(A.data_ptr(), precision.data_ptr(), A.numel(), out.data_ptr(), _stream()))
+    else:
+        check(lib().cn_compress_8bit(A.data_ptr(), float(precision), A.numel(), out.data_ptr(), _stream()))
+    return out
+
+
+def decompression_8bit(codes, precision, out=None):
+    import torch
+    _need(codes, torch.uint8, "codes")
+    if not codes.is_contiguous():
+        raise ValueError("codes must be contiguous")
+    if out is None:
+        out = torch.empty(codes.shape, dtype=torch.float32, device=codes.device)
+    _need(out, torch.float32, "out")
+    if isinstance(precision, torch.Tensor):
+        check(lib().cn_decompress_8bit_dp(codes.data_ptr(), precision.data_ptr(), codes.numel(), out.data_ptr(), _stream()))
+    else:
+        check(lib().cn_decompress_8bit(codes.data_ptr(), float(precision), codes.numel(), out.data_ptr(), _stream()))
+    return out

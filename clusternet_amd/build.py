@@ -1,0 +1,86 @@
+"""Compiles the HIP sources under clusternet_amd/csrc into clusternet_amd/libcnhip.so (gfx950).
+
+Usage: python -m clusternet_amd.build [--facade]
+The library is built in-tree so that it travels with the source tree; nothing is installed.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+FACADE = os.path.join(HERE, "facade")
+ROOT = os.path.dirname(HERE)
+LIB = os.path.join(HERE, "libcnhip.so")
+FACADE_LIB = os.path.join(HERE, "libclusternet.so")
+
+ARCH = "gfx950"
+# -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.
+# -ffp-contract=off: the codec must round every operation exactly like the reference's kernels.
+HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument"]
+SOURCES = ["cn_runtime.cpp", "cn_encode_lut.cpp", "cn_gemm_plan.cpp", "cn_codec.hip", "cn_gemm.hip",
+           "cn_layers.hip"]
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("build failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_library(verbose=False):
+    objs = []
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    for src in SOURCES:
+        path = os.path.join(CSRC, src)
+        if not os.path.exists(path):
+            continue
+        obj = os.path.join(objdir, src + ".o")
+        cmd = [hipcc()] + HIP_FLAGS + ["-c", path, "-o", obj]
+        out = _run(cmd)
+        if verbose and out.strip():
+            print(out)
+        objs.append(obj)
+    _run([hipcc(), "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LIB] + objs)
+    return LIB
+
+
+def build_facade(verbose=False):
+    """The C++ ClusterNet / Matrix layer over the C-ABI, plus its test binary."""
+    src = os.path.join(FACADE, "clusterNet.cpp")
+    if not os.path.exists(src):
+        return None
+    cxx = shutil.which("g++") or "g++"
+    inc = ["-I" + os.path.join(ROOT, "include"), "-I" + FACADE]
+    _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", FACADE_LIB, src,
+          os.path.join(FACADE, "basicOps.cpp")] + inc +
+         ["-L" + HERE, "-lcnhip", "-Wl,-rpath,$ORIGIN"])
+    test_src = os.path.join(ROOT, "tests", "cpp", "facade_test.cpp")
+    if os.path.exists(test_src):
+        _run([cxx, "-O2", "-std=c++17", "-Wall", "-o", os.path.join(ROOT, "tests", "cpp", "facade_test"),
+              test_src] + inc + ["-L" + HERE, "-lclusternet", "-lcnhip", "-Wl,-rpath," + HERE])
+    return FACADE_LIB
+
+
+def main(argv=None):
+    argv = sys.argv[1:] if argv is None else argv
+    print(build_library(verbose=True))
+    if "--facade" in argv:
+        print(build_facade(verbose=True))
+
+
+if __name__ == "__main__":
+    main()

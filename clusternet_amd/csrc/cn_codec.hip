@@ -1,0 +1,398 @@
+// 8-bit codec and abs-max kernels for gfx950.  All three are HBM-bound streaming kernels:
+//   compress    4 B read + 1 B written per element
+//   decompress  1 B read + 4 B written per element
+//   absmax      4 B read per element
+// Each lane moves 16-byte vectors laid out so that one wavefront instruction touches one
+// contiguous 1 KiB (fp32 side) / 256 B (code side) span.
+#include "cn_internal.h"
+
+namespace cn {
+
+constexpr int kThreads = 256;
+constexpr int kVecPerThread = 4;                         // float4 per lane per tile
+constexpr int kTileVec = kThreads * kVecPerThread;       // float4 per workgroup tile (4096 floats)
+constexpr uint32_t kLutCapacity = (127 - 107 + 1) * (1 << kMantBits) + 2;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// ---- exact encoder: the reference procedure, element by element --------------------------------
+// Follows kCompression_8bit (source/clusterKernels.cu:1163-1232): IEEE division, sign split,
+// two threshold exits, 6-step pivot search over the table, two-candidate pick.  `slot` is the
+// 128-entry LDS copy of the table whose entry 126 holds 1.0f.
+__device__ __forceinline__ uint32_t encode_exact(float x, float precision, const float *slot) {
+    float a = x / precision;
+    uint32_t neg = 0;
+    if (a < 0.0f) { neg = 0x80u; a = -a; }
+    if (a < 0.0000015f) return 254u;
+    if (a > 0.995703f) return 127u | neg;
+    int lo = 0, hi = 125, p = 63;
+#pragma unroll
+    for (int step = 32; step > 0; step >>= 1) {
+        if (a > slot[p]) { lo = p; p += step; }
+        else             { hi = p; p -= step; }
+    }
+    int c;
+    if (lo == p) c = (fabsf(slot[p] - a) < (slot[hi] - a)) ? p : hi;
+    else         c = ((slot[p] - a) < fabsf(slot[lo] - a)) ? p : lo;
+    return (uint32_t)c | neg;
+}
+
+struct EncodeShared {
+    EncodeBucket lut[kLutCapacity];
+    float slot[128];
+};
+
+__device__ __forceinline__ void stage_encoder(EncodeShared &sh, const EncodeBucket *lut,
+                                              uint32_t lut_count, const float *table) {
+    const uint2 *src = reinterpret_cast<const uint2 *>(lut);
+    uint2 *dst = reinterpret_cast<uint2 *>(sh.lut);
+    for (uint32_t i = threadIdx.x; i < lut_count; i += blockDim.x) dst[i] = src[i];
+    if (threadIdx.x < 126) sh.slot[threadIdx.x] = table[threadIdx.x];
+    if (threadIdx.x == 126) sh.slot[126] = 1.0f;
+    if (threadIdx.x == 127) sh.slot[127] = 0.0f;
+    __syncthreads();
+}
+
+// Fast path for one element: approximate quotient x * (1/precision), bucket lookup, one compare.
+// The approximate quotient is within kGuard bit patterns of the correctly rounded one; `near`
+// collects whether any element sits within kGuard of its bucket's boundary, in which case the
+// caller recomputes with encode_exact.
+__device__ __forceinline__ uint32_t encode_fast(float x, float recip, const EncodeBucket *lut,
+                                                uint32_t first, uint32_t last, uint32_t &near,
+                                                uint32_t &magmax) {
+    float a0 = x * recip;
+    uint32_t bits = __float_as_uint(a0);
+    uint32_t mag = bits & 0x7fffffffu;
+    magmax = max(magmax, mag);
+    uint32_t b = min(max(mag >> kBucketShift, first), last) - first;
+    EncodeBucket e = lut[b];
+    int32_t d = (int32_t)(mag - e.boundary_minus_guard);
+    near |= ((uint32_t)d <= 2u * kGuard) ? 1u : 0u;
+    uint32_t c = (d >= (int32_t)kGuard) ? (e.codes >> 8) : e.codes;
+    return (c & 0xffu) | ((bits >> 24) & 0x80u);
+}
+
+// The approximation x * (1/p) is trusted only when 1/p is a normal number with full precision.
+__device__ __forceinline__ bool precision_allows_fast_path(float p) {
+    float ap = fabsf(p);
+    return ap >= 8.67361738e-19f /* 2^-60 */ && ap <= 1.15292150e18f /* 2^60 */;
+}
+
+template <bool kVector>
+__global__ __launch_bounds__(kThreads) void compress_kernel(
+    const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr,
+    size_t n, uint8_t *__restrict__ codes, const EncodeBucket *__restrict__ lut,
+    uint32_t lut_first, uint32_t lut_count, const float *__restrict__ table) {
+    __shared__ EncodeShared sh;
+    stage_encoder(sh, lut, lut_count, table);
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
+    const bool fast_ok = precision_allows_fast_path(precision);
+    const float recip = 1.0f / precision;
+    const uint32_t first = lut_first, last = lut_first + lut_count - 1;
+
+    if (kVector) {
+        const size_t nvec = n / 4;
+        const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
+        uint32_t *c4 = reinterpret_cast<uint32_t *>(codes);
+        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
+        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+            const size_t base = tile * kTileVec + threadIdx.x;
+            f32x4 v[kVecPerThread];
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                size_t i = base + (size_t)j * kThreads;
+                v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+            uint32_t packed[kVecPerThread];
+            uint32_t near = 0, magmax = 0;
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                uint32_t c0 = encode_fast(v[j].x, recip, sh.lut, first, last, near, magmax);
+                uint32_t c1 = encode_fast(v[j].y, recip, sh.lut, first, last, near, magmax);
+                uint32_t c2 = encode_fast(v[j].z, recip, sh.lut, first, last, near, magmax);
+                uint32_t c3 = encode_fast(v[j].w, recip, sh.lut, first, last, near, magmax);
+                packed[j] = c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
+            }
+            if (!fast_ok || near != 0 || magmax > 0x7f800000u) {
+#pragma unroll
+                for (int j = 0; j < kVecPerThread; ++j) {
+                    uint32_t c0 = encode_exact(v[j].x, precision, sh.slot);
+                    uint32_t c1 = encode_exact(v[j].y, precision, sh.slot);
+                    uint32_t c2 = encode_exact(v[j].z, precision, sh.slot);
+                    uint32_t c3 = encode_exact(v[j].w, precision, sh.slot);
+                    packed[j] = c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                size_t i = base + (size_t)j * kThreads;
+                if (i < nvec) __builtin_nontemporal_store(packed[j], &c4[i]);
+            }
+        }
+        // ragged tail (n % 4 elements)
+        if (blockIdx.x == 0) {
+            size_t i = nvec * 4 + threadIdx.x;
+            if (i < n) codes[i] = (uint8_t)encode_exact(x[i], precision, sh.slot);
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
+            codes[i] = (uint8_t)encode_exact(x[i], precision, sh.slot);
+    }
+}
+
+// Follows kDecompression_8bit (source/clusterKernels.cu:1135-1160): a 256-entry table scaled by
+// the precision, rebuilt once per workgroup, then a pure gather.
+template <bool kVector>
+__global__ __launch_bounds__(kThreads) void decompress_kernel(
+    const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr,
+    size_t n, float *__restrict__ out, const float *__restrict__ table) {
+    __shared__ float lut[256];
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
+    if (threadIdx.x < 126) {
+        float v = table[threadIdx.x] * precision;
+        lut[threadIdx.x] = v;
+        lut[threadIdx.x + 128] = -v;
+    } else if (threadIdx.x == 126) {
+        lut[126] = precision;
+        lut[127] = precision;
+        lut[254] = precision;
+        lut[255] = -precision;
+    }
+    __syncthreads();
+
+    if (kVector) {
+        const size_t nvec = n / 4;
+        const uint32_t *c4 = reinterpret_cast<const uint32_t *>(codes);
+        f32x4 *o4 = reinterpret_cast<f32x4 *>(out);
+        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
+        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+            const size_t base = tile * kTileVec + threadIdx.x;
+            uint32_t w[kVecPerThread];
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                size_t i = base + (size_t)j * kThreads;
+                w[j] = (i < nvec) ? __builtin_nontemporal_load(&c4[i]) : 0u;
+            }
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                size_t i = base + (size_t)j * kThreads;
+                f32x4 o;
+                o.x = lut[w[j] & 0xffu];
+                o.y = lut[(w[j] >> 8) & 0xffu];
+                o.z = lut[(w[j] >> 16) & 0xffu];
+                o.w = lut[w[j] >> 24];
+                if (i < nvec) __builtin_nontemporal_store(o, &o4[i]);
+            }
+        }
+        if (blockIdx.x == 0) {
+            size_t i = nvec * 4 + threadIdx.x;
+            if (i < n) out[i] = lut[codes[i]];
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
+            out[i] = lut[codes[i]];
+    }
+}
+
+// ---- abs-max ------------------------------------------------------------------------------------
+// Non-negative fp32 values order like their bit patterns, so the reduction runs on
+// (pattern & 0x7fffffff) with integer max: exact, order-independent, and a NaN (pattern above
+// 0x7f800000) wins and is returned as NaN.
+__device__ __forceinline__ uint32_t wave_max(uint32_t v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = max(v, (uint32_t)__shfl_xor((int)v, off, 64));
+    return v;
+}
+
+__device__ __forceinline__ uint32_t block_max(uint32_t v, uint32_t *smem) {
+    v = wave_max(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    if (wave == 0) {
+        v = (lane < (int)(blockDim.x >> 6)) ? smem[lane] : 0u;
+        v = wave_max(v);
+    }
+    return v;  // valid in wave 0
+}
+
+template <bool kVector>
+__global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restrict__ x, size_t n,
+                                                          float *__restrict__ out,
+                                                          uint32_t *__restrict__ scratch) {
+    __shared__ uint32_t smem[kThreads / 64];
+    __shared__ uint32_t s_last;
+    uint32_t m = 0;
+    if (kVector) {
+        const size_t nvec = n / 4;
+        const u32x4 *x4 = reinterpret_cast<const u32x4 *>(x);
+        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
+        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+            const size_t base = tile * kTileVec + threadIdx.x;
+            u32x4 v[kVecPerThread];
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                size_t i = base + (size_t)j * kThreads;
+                v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : u32x4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int j = 0; j < kVecPerThread; ++j) {
+                m = max(m, v[j].x & 0x7fffffffu);
+                m = max(m, v[j].y & 0x7fffffffu);
+                m = max(m, v[j].z & 0x7fffffffu);
+                m = max(m, v[j].w & 0x7fffffffu);
+            }
+        }
+        if (blockIdx.x == 0) {
+            size_t i = nvec * 4 + threadIdx.x;
+            if (i < n) m = max(m, __float_as_uint(x[i]) & 0x7fffffffu);
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
+            m = max(m, __float_as_uint(x[i]) & 0x7fffffffu);
+    }
+    m = block_max(m, smem);
+    // Publish the workgroup's maximum, then let the last workgroup to arrive fold all of them.
+    // scratch[0..gridDim.x) = partial maxima, scratch[kReduceSlots] = arrival counter (left at 0).
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&scratch[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        uint32_t ticket = atomicAdd(&scratch[kReduceSlots], 1u);
+        s_last = (ticket == gridDim.x - 1) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (s_last) {
+        __threadfence();
+        uint32_t r = 0;
+        for (uint32_t i = threadIdx.x; i < gridDim.x; i += blockDim.x)
+            r = max(r, __hip_atomic_load(&scratch[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        __syncthreads();
+        r = block_max(r, smem);
+        if (threadIdx.x == 0) {
+            out[0] = __uint_as_float(r);
+            __hip_atomic_store(&scratch[kReduceSlots], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+__global__ void set_scalar_kernel(float *out, float v) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) out[0] = v;
+}
+
+__global__ __launch_bounds__(kThreads) void fill_kernel(float *__restrict__ dst, float v, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
+        dst[i] = v;
+}
+
+static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+
+static int stream_grid(const Context *ctx, size_t n, int per_cu) {
+    size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
+    size_t cap = (size_t)ctx->num_cu * per_cu;
+    if (cap > (size_t)kReduceSlots) cap = kReduceSlots;
+    size_t g = tiles < cap ? tiles : cap;
+    return (int)(g < 1 ? 1 : g);
+}
+
+static cn_status compress_impl(const float *x, float precision, const float *precision_dev, size_t n,
+                               uint8_t *codes, void *stream) {
+    if (n == 0) return CN_OK;
+    if (!x || !codes) { set_error("compress_8bit: NULL pointer"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    int grid = stream_grid(ctx, n, 6);
+    if (aligned(x, 16) && aligned(codes, 4))
+        hipLaunchKernelGGL(compress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, precision,
+                           precision_dev, n, codes, ctx->encode_lut, ctx->lut_first, ctx->lut_count, ctx->table);
+    else
+        hipLaunchKernelGGL(compress_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, precision,
+                           precision_dev, n, codes, ctx->encode_lut, ctx->lut_first, ctx->lut_count, ctx->table);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+static cn_status decompress_impl(const uint8_t *codes, float precision, const float *precision_dev,
+                                 size_t n, float *out, void *stream) {
+    if (n == 0) return CN_OK;
+    if (!codes || !out) { set_error("decompress_8bit: NULL pointer"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    int grid = stream_grid(ctx, n, 8);
+    if (aligned(codes, 4) && aligned(out, 16))
+        hipLaunchKernelGGL(decompress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
+                           precision_dev, n, out, ctx->table);
+    else
+        hipLaunchKernelGGL(decompress_kernel<false>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
+                           precision_dev, n, out, ctx->table);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+}  // namespace cn
+
+using namespace cn;
+
+extern "C" {
+
+cn_status cn_compress_8bit(const float *x, float precision, size_t n, uint8_t *codes, void *stream) {
+    return compress_impl(x, precision, nullptr, n, codes, stream);
+}
+
+cn_status cn_compress_8bit_dp(const float *x, const float *precision_device, size_t n, uint8_t *codes,
+                              void *stream) {
+    if (n != 0 && !precision_device) { set_error("compress_8bit_dp: NULL precision"); return CN_ERR_NULL; }
+    return compress_impl(x, 0.0f, precision_device, n, codes, stream);
+}
+
+cn_status cn_decompress_8bit(const uint8_t *codes, float precision, size_t n, float *out, void *stream) {
+    return decompress_impl(codes, precision, nullptr, n, out, stream);
+}
+
+cn_status cn_decompress_8bit_dp(const uint8_t *codes, const float *precision_device, size_t n, float *out,
+                                void *stream) {
+    if (n != 0 && !precision_device) { set_error("decompress_8bit_dp: NULL precision"); return CN_ERR_NULL; }
+    return decompress_impl(codes, 0.0f, precision_device, n, out, stream);
+}
+
+cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
+    if (!out) { set_error("absmax_f32: NULL output"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    if (n == 0) {
+        // the reference's reduction starts from -1 and returns it for an empty range
+        hipLaunchKernelGGL(set_scalar_kernel, dim3(1), dim3(64), 0, st, out, -1.0f);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
+    if (!x) { set_error("absmax_f32: NULL input"); return CN_ERR_NULL; }
+    int grid = stream_grid(ctx, n, 8);
+    if (aligned(x, 16))
+        hipLaunchKernelGGL(absmax_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+    else
+        hipLaunchKernelGGL(absmax_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_fill_f32(float *dst, float value, size_t n, void *stream) {
+    if (n == 0) return CN_OK;
+    if (!dst) { set_error("fill_f32: NULL pointer"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    size_t blocks = (n + kThreads - 1) / kThreads;
+    size_t cap = (size_t)ctx->num_cu * 16;
+    int grid = (int)(blocks < cap ? blocks : cap);
+    hipLaunchKernelGGL(fill_kernel, dim3(grid), dim3(kThreads), 0, (hipStream_t)stream, dst, value, n);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,200 @@
+// Library state: status strings, per-device contexts, memory helpers.
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+
+#include "cn_internal.h"
+
+namespace cn {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+cn_status hip_fail(hipError_t e, const char *what, const char *file, int line) {
+    set_error("%s failed: %s (%s:%d)", what, hipGetErrorString(e), file, line);
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) return CN_ERR_NO_DEVICE;
+    return CN_ERR_HIP;
+}
+
+void host_table(float out[126]);
+
+static Context g_ctx[kMaxDevices];
+static std::mutex g_mutex;
+
+static cn_status init_device(int device) {
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        set_error("no HIP device available (%s)", e == hipSuccess ? "device count is 0" : hipGetErrorString(e));
+        return CN_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= count || device >= kMaxDevices) {
+        set_error("device %d out of range (%d visible)", device, count);
+        return CN_ERR_NO_DEVICE;
+    }
+    Context &c = g_ctx[device];
+    if (c.ready) return CN_OK;
+
+    int previous = 0;
+    CN_HIP(hipGetDevice(&previous));
+    CN_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    CN_HIP(hipGetDeviceProperties(&prop, device));
+    c.device = device;
+    c.num_cu = prop.multiProcessorCount;
+
+    float table[126];
+    host_table(table);
+    CN_HIP(hipMalloc((void **)&c.table, sizeof(table)));
+    CN_HIP(hipMemcpy(c.table, table, sizeof(table), hipMemcpyHostToDevice));
+
+    static EncodeLut lut;
+    if (!build_encode_lut(&lut)) return CN_ERR_ARG;
+    c.lut_first = lut.first_bucket;
+    c.lut_count = lut.count;
+    CN_HIP(hipMalloc((void **)&c.encode_lut, lut.count * sizeof(EncodeBucket)));
+    CN_HIP(hipMemcpy(c.encode_lut, lut.entry, lut.count * sizeof(EncodeBucket), hipMemcpyHostToDevice));
+
+    size_t mib = 1024;
+    if (const char *env = getenv("CNHIP_WORKSPACE_MB")) {
+        long v = atol(env);
+        if (v >= 16) mib = (size_t)v;
+    }
+    c.workspace_bytes = mib << 20;
+    CN_HIP(hipMalloc(&c.workspace, c.workspace_bytes));
+
+    CN_HIP(hipMalloc((void **)&c.reduce_scratch, (kReduceSlots + 64) * sizeof(uint32_t)));
+    CN_HIP(hipMemset(c.reduce_scratch, 0, (kReduceSlots + 64) * sizeof(uint32_t)));
+    CN_HIP(hipDeviceSynchronize());
+    CN_HIP(hipSetDevice(previous));
+    c.ready = true;
+    return CN_OK;
+}
+
+cn_status current_context(Context **out) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) {
+        set_error("no HIP device available (%s)", hipGetErrorString(e));
+        return CN_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= kMaxDevices) {
+        set_error("device %d out of range", device);
+        return CN_ERR_NO_DEVICE;
+    }
+    if (!g_ctx[device].ready) {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        cn_status s = init_device(device);
+        if (s != CN_OK) return s;
+    }
+    *out = &g_ctx[device];
+    return CN_OK;
+}
+
+}  // namespace cn
+
+using namespace cn;
+
+extern "C" {
+
+const char *cn_status_string(cn_status s) {
+    switch (s) {
+        case CN_OK: return "CN_OK";
+        case CN_ERR_NULL: return "CN_ERR_NULL";
+        case CN_ERR_SHAPE: return "CN_ERR_SHAPE";
+        case CN_ERR_NO_DEVICE: return "CN_ERR_NO_DEVICE";
+        case CN_ERR_HIP: return "CN_ERR_HIP";
+        case CN_ERR_WORKSPACE: return "CN_ERR_WORKSPACE";
+        case CN_ERR_ARG: return "CN_ERR_ARG";
+        default: return "CN_ERR_UNKNOWN";
+    }
+}
+
+const char *cn_last_error(void) { return g_error; }
+
+cn_status cn_init(int device) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    return init_device(device);
+}
+
+cn_status cn_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    int previous = 0;
+    bool have_prev = hipGetDevice(&previous) == hipSuccess;
+    for (int d = 0; d < kMaxDevices; ++d) {
+        Context &c = g_ctx[d];
+        if (!c.ready) continue;
+        CN_HIP(hipSetDevice(d));
+        CN_HIP(hipDeviceSynchronize());
+        CN_HIP(hipFree(c.table));
+        CN_HIP(hipFree(c.encode_lut));
+        CN_HIP(hipFree(c.workspace));
+        CN_HIP(hipFree(c.reduce_scratch));
+        c = Context();
+    }
+    if (have_prev) CN_HIP(hipSetDevice(previous));
+    return CN_OK;
+}
+
+int cn_num_compute_units(void) {
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 0;
+    return g_ctx[device].ready ? g_ctx[device].num_cu : 0;
+}
+
+cn_status cn_malloc(void **device_ptr, size_t bytes) {
+    if (!device_ptr) { set_error("cn_malloc: NULL result pointer"); return CN_ERR_NULL; }
+    *device_ptr = nullptr;
+    if (bytes == 0) return CN_OK;
+    CN_HIP(hipMalloc(device_ptr, bytes));
+    return CN_OK;
+}
+
+cn_status cn_free(void *device_ptr) {
+    if (!device_ptr) return CN_OK;
+    CN_HIP(hipFree(device_ptr));
+    return CN_OK;
+}
+
+cn_status cn_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+    if (bytes == 0) return CN_OK;
+    if (!dst || !src) { set_error("cn_memcpy_h2d: NULL pointer"); return CN_ERR_NULL; }
+    CN_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return CN_OK;
+}
+
+cn_status cn_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+    if (bytes == 0) return CN_OK;
+    if (!dst || !src) { set_error("cn_memcpy_d2h: NULL pointer"); return CN_ERR_NULL; }
+    CN_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return CN_OK;
+}
+
+cn_status cn_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream) {
+    if (bytes == 0) return CN_OK;
+    if (!dst || !src) { set_error("cn_memcpy_d2d: NULL pointer"); return CN_ERR_NULL; }
+    CN_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return CN_OK;
+}
+
+cn_status cn_synchronize(void *stream) {
+    CN_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return CN_OK;
+}
+
+cn_status cn_table_get(float out_host[126]) {
+    if (!out_host) { set_error("cn_table_get: NULL pointer"); return CN_ERR_NULL; }
+    host_table(out_host);
+    return CN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,115 @@
+/* libcnhip: C-ABI of the MI355X (gfx950) implementation of clusterNet's matrix-multiply and
+ * 8-bit codec path.
+ *
+ * Plain pointers and sizes only; every pointer named "device" is a HIP device address, every
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream, which is where the
+ * reference runs everything).  All calls are asynchronous on `stream` unless stated otherwise.
+ * Every function returns a cn_status; 0 is success.  The library never falls back to the CPU:
+ * without a usable GPU, cn_init and every compute entry point return CN_ERR_NO_DEVICE.
+ *
+ * Storage convention: matrices are ROW-major with an explicit leading dimension (elements per
+ * row).  The reference keeps device matrices column-major (source/basicOps.cu:14-33) and calls
+ * cublasSgemm with lda = rows (source/clusterNet.cpp:459-461); a column-major M x K matrix is the
+ * same bytes as a row-major K x M one, so a column-major caller obtains C = op(A) op(B) by asking
+ * for C^T = op(B)^T op(A)^T, i.e. cn_gemm_f32(transB, transA, N, M, K, B, ldb, A, lda, C, ldc).
+ */
+#ifndef CNHIP_H
+#define CNHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int cn_status;
+enum {
+    CN_OK = 0,
+    CN_ERR_NULL = 1,       /* a required pointer is NULL */
+    CN_ERR_SHAPE = 2,      /* negative dimension, leading dimension too small, size mismatch */
+    CN_ERR_NO_DEVICE = 3,  /* no HIP device / device index out of range */
+    CN_ERR_HIP = 4,        /* a HIP runtime call failed; see cn_last_error() */
+    CN_ERR_WORKSPACE = 5,  /* internal workspace too small for the request */
+    CN_ERR_ARG = 6         /* any other invalid argument */
+};
+
+/* Human-readable name of a status code. */
+const char *cn_status_string(cn_status s);
+/* Text of the most recent failure on the calling thread ("" if none). */
+const char *cn_last_error(void);
+
+/* Prepares `device`: uploads the 126-entry codebook and the encoder's bucket table, allocates the
+ * split-K workspace (size in MiB from the environment variable CNHIP_WORKSPACE_MB, default 1024).
+ * Replaces the table upload of ClusterNet::init (source/clusterNet.cpp:73) and the lazy per-device
+ * cuBLAS handle creation (source/clusterNet.cpp:413-426).  Idempotent.  Compute entry points call
+ * it on first use for the current device, so calling it explicitly is optional.  Synchronous. */
+cn_status cn_init(int device);
+/* Frees everything cn_init allocated on every device.  Synchronous. */
+cn_status cn_shutdown(void);
+/* Number of compute units of the current device as seen by the library (0 before init). */
+int cn_num_compute_units(void);
+
+/* Device memory for hosts that have no allocator of their own (the C++ facade).  Replace the
+ * cudaMalloc / cudaFree / cudaMemcpy calls inside the Matrix allocators and to_gpu / to_host
+ * (source/basicOps.cu:14-88,214-262).  cn_memcpy_* are synchronous with respect to the host. */
+cn_status cn_malloc(void **device_ptr, size_t bytes);
+cn_status cn_free(void *device_ptr);
+cn_status cn_memcpy_h2d(void *device_dst, const void *host_src, size_t bytes);
+cn_status cn_memcpy_d2h(void *host_dst, const void *device_src, size_t bytes);
+cn_status cn_memcpy_d2d(void *device_dst, const void *device_src, size_t bytes, void *stream);
+cn_status cn_fill_f32(float *device_dst, float value, size_t n, void *stream);
+cn_status cn_synchronize(void *stream);
+
+/* Copies the 126 codebook magnitudes (ascending, in (0,1)) to host memory.
+ * Replaces reading source/8bit_floats.hdf5 through read_hdf5 (source/util.cu:100-131). */
+cn_status cn_table_get(float out_host[126]);
+
+/* C[M x N] = op(A) op(B), fp32, alpha = 1, beta = 0 (C is overwritten, never read).
+ *   trans_a == 0: A is stored M x K (lda >= K);  trans_a != 0: A is stored K x M (lda >= M).
+ *   trans_b == 0: B is stored K x N (ldb >= N);  trans_b != 0: B is stored N x K (ldb >= K).
+ *   C is stored M x N (ldc >= N).  M, N, K >= 0 (a zero dimension is a no-op; K == 0 zeroes C).
+ * Replaces the cublasSgemm call of ClusterNet::dot(A,B,out,T1,T2) (source/clusterNet.cpp:404-461):
+ * dot = (0,0), Tdot = (1,0), dotT = (0,1).  Uses the library's workspace when it splits K, so two
+ * GEMMs must not run concurrently on different streams of one device. */
+cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
+                      const float *A_device, int64_t lda, const float *B_device, int64_t ldb,
+                      float *C_device, int64_t ldc, void *stream);
+
+/* C[M x N] = A[M x K] decode(W[K x N], scale): W holds 8-bit codes (row-major, ldw >= N) that are
+ * expanded inside the kernel with exactly the table of cn_decompress_8bit(scale).  No counterpart
+ * in the reference; its relatives are dot8bit / dot8bit_shared (source/clusterNet.cpp:1409-1431,
+ * source/clusterKernels.cu:1717-1843), which take both operands coded. */
+cn_status cn_gemm_f32_w8(int64_t M, int64_t N, int64_t K, const float *A_device, int64_t lda,
+                         const uint8_t *W_device, int64_t ldw, float scale, float *C_device,
+                         int64_t ldc, void *stream);
+
+/* *out_device = max_i |x_i| (n == 0 gives 0; a NaN input gives NaN).  One pass, no temporary.
+ * Replaces the abs + max pair callers use to obtain `precision` (source/basicOps.cu:810-822 and
+ * :1076-1081; call sites source/test.cu:2108-2109, source/DeepNeuralNetwork.cpp:218-222). */
+cn_status cn_absmax_f32(const float *x_device, size_t n, float *out_device, void *stream);
+
+/* codes[i] = 8-bit code of x[i] / precision, bit-exact with kCompression_8bit
+ * (source/clusterKernels.cu:1163-1232; launcher source/basicOps.cu:1163-1168), flat over n
+ * elements.  Inputs whose scaled magnitude falls in (0.99140614, 0.995703], for which the
+ * reference reads a table slot it never wrote, encode as 125 / 253. */
+cn_status cn_compress_8bit(const float *x_device, float precision, size_t n,
+                           uint8_t *codes_device, void *stream);
+/* Same, with precision read from device memory (e.g. the output of cn_absmax_f32), so that the
+ * absmax -> compress sequence needs no host synchronisation. */
+cn_status cn_compress_8bit_dp(const float *x_device, const float *precision_device, size_t n,
+                              uint8_t *codes_device, void *stream);
+
+/* out[i] = lut[codes[i]] with lut[c] = table[c] * precision, lut[c + 128] = -lut[c] (c < 126),
+ * lut[126] = lut[127] = lut[254] = +precision, lut[255] = -precision: bit-exact with
+ * kDecompression_8bit (source/clusterKernels.cu:1135-1160; launcher source/basicOps.cu:1172-1176).
+ * Note that code 254 (emitted for near-zero inputs) decodes to +precision, as in the reference. */
+cn_status cn_decompress_8bit(const uint8_t *codes_device, float precision, size_t n,
+                             float *out_device, void *stream);
+cn_status cn_decompress_8bit_dp(const uint8_t *codes_device, const float *precision_device,
+                                size_t n, float *out_device, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CNHIP_H */

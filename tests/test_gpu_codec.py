@@ -1,0 +1,167 @@
+"""Bit-exact parity of the HIP codec kernels with the CPU checker, through the C-ABI."""
+import numpy as np
+import pytest
+
+import oracle
+from util import cfg2_tensor
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    import clusternet_amd as cn
+    cn.init(0)
+    return torch.device("cuda:0")
+
+
+def _t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _adversarial():
+    t = oracle.table()
+    pts = [t, np.nextafter(t, np.float32(0)), np.nextafter(t, np.float32(2))]
+    mids = ((t[:-1].astype(np.float64) + t[1:].astype(np.float64)) / 2).astype(np.float32)
+    for k in range(-3, 4):
+        pts.append((mids.view(np.uint32).astype(np.int64) + k).astype(np.uint32).view(np.float32))
+    for thr in (np.float32(0.0000015), np.float32(0.995703), np.float32(1.0), t[125]):
+        b = int(np.array([thr]).view(np.uint32)[0])
+        pts.append(np.arange(b - 8, b + 9, dtype=np.uint32).view(np.float32))
+    pts.append(np.array([0.0, -0.0, 1e-45, 1e-38, 1.1754944e-38, 0.5, 0.25, 0.1, 0.01, 0.001, 0.993,
+                         0.9957, 0.9958, 1.0, 1.5, 3e38, np.inf, np.nan], np.float32))
+    x = np.concatenate([np.asarray(p, np.float32).reshape(-1) for p in pts])
+    return np.concatenate([x, -x])
+
+
+def test_absmax_matches_numpy(dev):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(0)
+    for n in (1, 2, 3, 5, 63, 64, 4095, 4096, 4097, 128 * 40000, 10_000_019):
+        x = rng.normal(0, 1, n).astype(np.float32)
+        got = float(cn.absmax(_t(x, dev)).cpu()[0])
+        assert got == float(np.abs(x).max()) == oracle.absmax(x), n
+    # unaligned start, empty input, NaN propagation, repeated calls reuse the scratch correctly
+    x = rng.normal(0, 1, 100_001).astype(np.float32)
+    xt = _t(x, dev)
+    for off in (1, 2, 3):
+        assert float(cn.absmax(xt[off:]).cpu()[0]) == float(np.abs(x[off:]).max())
+    assert float(cn.absmax(xt[:0]).cpu()[0]) == -1.0
+    x[777] = np.nan
+    assert np.isnan(float(cn.absmax(_t(x, dev)).cpu()[0]))
+    for _ in range(3):
+        assert float(cn.absmax(xt).cpu()[0]) == oracle.absmax(xt.cpu().numpy())
+
+
+def test_compress_config2_bit_exact(dev):
+    import clusternet_amd as cn
+    x = cfg2_tensor(np.random.default_rng(42))
+    xt = _t(x, dev)
+    prec_dev = cn.absmax(xt)
+    prec = float(prec_dev.cpu()[0])
+    assert prec == float(np.abs(x).max())
+    want = oracle.compress(x, prec, 0)
+    got = cn.compression_8bit(xt, prec).cpu().numpy()
+    assert got.dtype == np.uint8 and got.shape == x.shape
+    assert np.array_equal(got, want)
+    # precision taken from device memory gives the same codes
+    assert np.array_equal(cn.compression_8bit(xt, prec_dev).cpu().numpy(), want)
+    # decompression, both ways of passing the precision
+    back = cn.decompression_8bit(_t(want, dev), prec).cpu().numpy()
+    assert np.array_equal(back.view(np.uint32), oracle.decompress(want, prec).view(np.uint32))
+    back2 = cn.decompression_8bit(_t(want, dev), prec_dev).cpu().numpy()
+    assert np.array_equal(back2.view(np.uint32), back.view(np.uint32))
+
+
+@pytest.mark.parametrize("prec", [1.0, 0.1, 0.5, 2.0, 3.7, 1e-3, 1e3, -1.0, 1e-30, 1e30, 1e-42,
+                                  0.0, float("inf"), float("nan")])
+def test_compress_adversarial_inputs(dev, prec):
+    import clusternet_amd as cn
+    x = _adversarial()
+    with np.errstate(all="ignore"):
+        scale = np.float32(prec) if np.isfinite(prec) and prec != 0 else np.float32(1.0)
+        xs = (x * scale).astype(np.float32)
+        want = oracle.compress(xs, prec, 0)
+    got = cn.compression_8bit(_t(xs, dev), prec).cpu().numpy()
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, (prec, xs[bad[:5]], got[bad[:5]], want[bad[:5]])
+
+
+def test_compress_sizes_and_alignment(dev):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(5)
+    base = rng.normal(0, 0.3, 70_000).astype(np.float32)
+    bt = _t(base, dev)
+    for n in (0, 1, 2, 3, 4, 5, 7, 255, 256, 1023, 1024, 4095, 4096, 4097, 16385, 65_537):
+        for off in (0, 1, 2, 3):
+            x = base[off:off + n]
+            got = cn.compression_8bit(bt[off:off + n], 0.9).cpu().numpy()
+            assert np.array_equal(got, oracle.compress(x, 0.9, 0)), (n, off)
+    codes = rng.integers(0, 256, 70_000, dtype=np.uint8)
+    ct = _t(codes, dev)
+    for n in (0, 1, 3, 4, 5, 1023, 4096, 4099, 65_537):
+        for off in (0, 1, 2, 3):
+            got = cn.decompression_8bit(ct[off:off + n], 0.37).cpu().numpy()
+            want = oracle.decompress(codes[off:off + n], 0.37)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (n, off)
+
+
+def test_decompress_every_code(dev):
+    import clusternet_amd as cn
+    codes = np.arange(256, dtype=np.uint8)
+    for prec in (1.0, 0.1, 0.0234, 17.0, 1e-20, -2.0):
+        got = cn.decompression_8bit(_t(codes, dev), prec).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), oracle.decode_lut(prec).view(np.uint32))
+        assert got[254] == np.float32(prec)  # the "zero" code decodes to +precision
+
+
+def test_compress_exhaustive_over_the_table_range(dev):
+    """Every fp32 pattern from 2^-25 to just above 1, both signs, at precision 1."""
+    import torch
+    import clusternet_amd as cn
+    lo, hi = 0x33000000, 0x3f900000
+    step = 1 << 26
+    for start in range(lo, hi, step):
+        mags = np.arange(start, min(start + step, hi), dtype=np.uint32)
+        want = oracle.port_compress(mags.view(np.float32), 1.0)
+        xt = _t(mags.view(np.float32), dev)
+        got = cn.compression_8bit(xt, 1.0)
+        assert np.array_equal(got.cpu().numpy(), want), hex(start)
+        neg = cn.compression_8bit(-xt, 1.0)
+        expect_neg = torch.where(got == 254, got, got | 0x80)
+        assert torch.equal(neg, expect_neg), hex(start)
+
+
+def test_compress_random_precisions(dev):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(77)
+    for prec in list(rng.uniform(1e-4, 50, 6)) + [2.0 ** -40, 2.0 ** 40]:
+        x = (np.exp(rng.uniform(np.log(1e-7), np.log(1.3), 2_000_000)) * prec).astype(np.float32)
+        x *= rng.choice([-1.0, 1.0], x.size).astype(np.float32)
+        got = cn.compression_8bit(_t(x, dev), float(prec)).cpu().numpy()
+        assert np.array_equal(got, oracle.port_compress(x, float(prec))), prec
+
+
+def test_large_tensor_by_tiling(dev):
+    """A 1.07e9-element tensor (4.3 GB) built by repeating a block whose codes are verified on the
+    CPU: every repetition must carry the same codes, and decoding must repeat likewise."""
+    import torch
+    import clusternet_amd as cn
+    rng = np.random.default_rng(9)
+    block = cfg2_tensor(rng, 1, 1 << 20).reshape(-1)
+    block[123] = 0.75  # make sure max is not unique-position dependent
+    prec = float(np.abs(block).max())
+    want = oracle.port_compress(block, prec)
+    reps = 1024
+    big = _t(block, dev).repeat(reps)
+    assert big.numel() == reps << 20
+    assert float(cn.absmax(big).cpu()[0]) == prec
+    codes = cn.compression_8bit(big, prec)
+    wt = _t(want, dev)
+    assert torch.equal(codes.view(reps, -1), wt.unsqueeze(0).expand(reps, -1))
+    del big
+    back = cn.decompression_8bit(codes, prec)
+    bt = _t(oracle.decompress(want, prec), dev)
+    assert torch.equal(back.view(reps, -1).view(torch.int32), bt.view(torch.int32).unsqueeze(0).expand(reps, -1))

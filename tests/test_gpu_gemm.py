@@ -1,0 +1,245 @@
+"""Parity of the HIP fp32 GEMM kernels (dot / Tdot / dotT and the fused 8-bit-weight variant) with
+the CPU checker, through the C-ABI.  Tolerance: max relative error 1e-4 for K <= 4096 and
+1e-4 * sqrt(K / 4096) above, measured both against max|C_ref| and element-wise against
+sum_k |a||b|; integer-valued and one-hot cases must be exact."""
+import numpy as np
+import pytest
+
+import oracle
+from util import gemm_errors, gemm_tolerance
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    import clusternet_amd as cn
+    cn.init(0)
+    return torch.device("cuda:0")
+
+
+def _t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _check(cn, dev, A, B, ta=False, tb=False):
+    got = cn.gemm(_t(A, dev), _t(B, dev), ta, tb).cpu().numpy()
+    Cref, Cabs = oracle.gemm_with_abs(A, B, ta, tb)
+    K = A.shape[0] if ta else A.shape[1]
+    e1, e2 = gemm_errors(got, Cref, Cabs)
+    tol = gemm_tolerance(K)
+    assert e1 <= tol and e2 <= tol, (A.shape, B.shape, ta, tb, e1, e2, tol)
+    return got
+
+
+def test_reference_known_answers(dev):
+    # literals of the reference's tests/clusterNet_test.cu:22-23,72-75,111-119,125-128,161-164;
+    # the reference compares with ==, which sequential fp32 FMA meets; a matrix-core kernel may
+    # differ in the last bit
+    import clusternet_amd as cn
+    m1 = np.array([[0, 2, 3], [0, 0.83, 59.1387]], np.float32)
+    m2 = np.array([[17, 0], [3, 4], [0, 0]], np.float32)
+    f = lambda r: np.array(r, np.float32)
+    np.testing.assert_allclose(cn.dot(_t(m1, dev), _t(m2, dev)).cpu().numpy(), f([[6, 8], [2.49, 3.32]]), rtol=1e-6)
+    np.testing.assert_allclose(cn.Tdot(_t(m1, dev), _t(m1, dev)).cpu().numpy(),
+                               f([[0, 0, 0], [0, 4.6889, 55.085117], [0, 55.085117, 3506.385742]]), rtol=1e-6)
+    np.testing.assert_allclose(cn.Tdot(_t(m2, dev), _t(m2, dev)).cpu().numpy(), f([[298, 12], [12, 16]]), rtol=1e-6)
+    np.testing.assert_allclose(cn.dotT(_t(m1, dev), _t(m1, dev)).cpu().numpy(),
+                               f([[13, 179.0761], [179.0761, 3498.074463]]), rtol=1e-6)
+
+
+def test_all_ones_closed_forms_exact(dev):
+    # tests/clusterNet_test.cu:338-394: 8783, 317 and 17 with exact equality
+    import torch
+    import clusternet_amd as cn
+    ones = lambda r, c: torch.ones((r, c), dtype=torch.float32, device=dev)
+    assert bool((cn.dot(ones(111, 8783), ones(8783, 317)) == 8783.0).all())
+    out = cn.dotT(ones(17, 317), ones(8783, 317))
+    assert tuple(out.shape) == (17, 8783) and bool((out == 317.0).all())
+    out = ones(8783, 317)
+    cn.dot(ones(8783, 17), ones(17, 317), out=out)
+    assert bool((out == 17.0).all())
+    # tests/clusterNet_test.cu:257-276: a constant product, every entry identical
+    a = torch.full((200, 400), 0.3, dtype=torch.float32, device=dev)
+    b = torch.full((400, 800), 1.0, dtype=torch.float32, device=dev) + 0.1748345
+    c = cn.dot(a, b)
+    assert tuple(c.shape) == (200, 800) and bool((c == c[0, 0]).all())
+    assert abs(float(c[0, 0]) - 400 * 0.3 * 1.1748345) < 1e-3
+
+
+def test_config1_mlp_layer(dev):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(1)
+    lim = np.sqrt(6.0 / (784 + 1024))
+    A = rng.uniform(0, 1, (128, 784)).astype(np.float32)
+    W = rng.uniform(-lim, lim, (784, 1024)).astype(np.float32)
+    dC = rng.normal(0, 0.01, (128, 1024)).astype(np.float32)
+    C = _check(cn, dev, A, W)                  # dot  -> 128 x 1024
+    assert C.shape == (128, 1024)
+    G = _check(cn, dev, A, dC, ta=True)        # Tdot -> 784 x 1024
+    assert G.shape == (784, 1024)
+    E = _check(cn, dev, dC, W, tb=True)        # dotT -> 128 x 784
+    assert E.shape == (128, 784)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (2, 2, 3), (128, 128, 32), (129, 130, 33),
+                                   (64, 200, 31), (257, 100, 64), (100, 10, 4096), (200, 300, 1000),
+                                   (128, 512, 8192), (37, 1029, 515), (1000, 4, 128)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (False, True), (True, True)])
+def test_ragged_shapes_all_transposes(dev, shape, ta, tb):
+    import clusternet_amd as cn
+    M, N, K = shape
+    rng = np.random.default_rng(M * 131 + N * 17 + K)
+    A = rng.normal(0, 1, (K, M) if ta else (M, K)).astype(np.float32)
+    B = rng.normal(0, 1, (N, K) if tb else (K, N)).astype(np.float32)
+    _check(cn, dev, A, B, ta, tb)
+
+
+def test_identity_operand_is_exact(dev):
+    import torch
+    import clusternet_amd as cn
+    rng = np.random.default_rng(3)
+    B = rng.normal(0, 1, (300, 517)).astype(np.float32)
+    I = np.eye(300, dtype=np.float32)
+    assert np.array_equal(cn.dot(_t(I, dev), _t(B, dev)).cpu().numpy(), B)
+    assert np.array_equal(cn.Tdot(_t(I, dev), _t(B, dev)).cpu().numpy(), B)
+    A = rng.normal(0, 1, (211, 300)).astype(np.float32)
+    assert np.array_equal(cn.dot(_t(A, dev), _t(I, dev)).cpu().numpy(), A)
+    assert np.array_equal(cn.dotT(_t(A, dev), _t(I, dev)).cpu().numpy(), A)
+    # a permutation picks rows: the k index of every product lands where it should
+    perm = rng.permutation(300)
+    P = np.zeros((300, 300), np.float32)
+    P[np.arange(300), perm] = 1
+    assert np.array_equal(cn.dot(_t(P, dev), _t(B, dev)).cpu().numpy(), B[perm])
+
+
+def test_strided_operands_and_output_overwrite(dev):
+    import torch
+    import clusternet_amd as cn
+    rng = np.random.default_rng(4)
+    big_a = rng.normal(0, 1, (70, 203)).astype(np.float32)
+    big_b = rng.normal(0, 1, (150, 99)).astype(np.float32)
+    A, B = big_a[:, 3:153], big_b[:, 2:90]            # lda 203 > K 150, ldb 99 > N 88, odd offsets
+    at, bt = _t(big_a, dev)[:, 3:153], _t(big_b, dev)[:, 2:90]
+    out_big = torch.full((70, 120), float("nan"), dtype=torch.float32, device=dev)
+    out = out_big[:, 5:93]
+    cn.dot(at, bt, out=out)                           # beta = 0: NaNs in out must not leak
+    Cref, Cabs = oracle.gemm_with_abs(np.ascontiguousarray(A), np.ascontiguousarray(B))
+    e1, e2 = gemm_errors(out.cpu().numpy(), Cref, Cabs)
+    assert e1 < 1e-4 and e2 < 1e-4
+    assert bool(torch.isnan(out_big[:, :5]).all()) and bool(torch.isnan(out_big[:, 93:]).all())
+
+
+def test_shape_errors_are_reported(dev):
+    import torch
+    import clusternet_amd as cn
+    a = torch.zeros((4, 5), device=dev)
+    b = torch.zeros((6, 7), device=dev)
+    with pytest.raises(cn.CnError):
+        cn.dot(a, b)
+    with pytest.raises(cn.CnError):
+        cn.dot(a, torch.zeros((5, 7), device=dev), out=torch.zeros((4, 8), device=dev))
+    L = cn.lib()
+    assert L.cn_gemm_f32(0, 0, 4, 7, 5, a.data_ptr(), 4, b.data_ptr(), 7, a.data_ptr(), 7, None) == 2
+    assert L.cn_gemm_f32(0, 0, 4, 7, 5, None, 5, b.data_ptr(), 7, a.data_ptr(), 7, None) == 1
+    # K = 0 zeroes the output
+    out = torch.full((4, 7), 3.0, device=dev)
+    assert L.cn_gemm_f32(0, 0, 4, 7, 0, None, 1, None, 7, out.data_ptr(), 7, None) == 0
+    assert bool((out == 0).all())
+
+
+def test_linearity_and_transpose_identities_large(dev):
+    """Size-independent properties on a K = 20000 product: dot(A, B1 + B2) = dot(A,B1) + dot(A,B2)
+    up to rounding, Tdot(A^T stored, B) = dot(A, B), dotT(A, B^T stored) = dot(A, B)."""
+    import torch
+    import clusternet_amd as cn
+    g = torch.Generator(device=dev).manual_seed(7)
+    A = torch.rand((128, 20000), device=dev, generator=g)
+    B1 = (torch.rand((20000, 1536), device=dev, generator=g) - 0.5) * 0.02
+    B2 = (torch.rand((20000, 1536), device=dev, generator=g) - 0.5) * 0.02
+    c1, c2, c12 = cn.dot(A, B1), cn.dot(A, B2), cn.dot(A, B1 + B2)
+    scale = float(c12.abs().max())
+    assert float((c12 - (c1 + c2)).abs().max()) / scale < gemm_tolerance(20000)
+    ct = cn.Tdot(A.t().contiguous(), B1)
+    cT = cn.dotT(A, B1.t().contiguous())
+    assert float((ct - c1).abs().max()) / scale < gemm_tolerance(20000)
+    assert float((cT - c1).abs().max()) / scale < gemm_tolerance(20000)
+
+
+def test_config3_full_size_sampled_columns(dev):
+    """README workload on one GPU: 128x100000 . 100000x40000, then . 40000x20000.  All rows and 48
+    sampled columns of each product are recomputed on the CPU in fp64."""
+    import torch
+    import clusternet_amd as cn
+    g = torch.Generator(device=dev).manual_seed(11)
+    batch = torch.rand((128, 100000), device=dev, generator=g)
+    lim1, lim2 = float(np.sqrt(6.0 / 140000)), float(np.sqrt(6.0 / 60000))
+    W1 = torch.empty((100000, 40000), device=dev)
+    for r in range(0, 100000, 10000):
+        W1[r:r + 10000] = (torch.rand((10000, 40000), device=dev, generator=g) * 2 - 1) * lim1
+    W2 = (torch.rand((40000, 20000), device=dev, generator=g) * 2 - 1) * lim2
+    out1 = cn.dot(batch, W1)
+    out2 = cn.dot(out1, W2)
+    assert tuple(out1.shape) == (128, 40000) and tuple(out2.shape) == (128, 20000)
+    rng = np.random.default_rng(5)
+    for A, W, out, K in ((batch, W1, out1, 100000), (out1, W2, out2, 40000)):
+        N = W.shape[1]
+        cols = np.unique(np.concatenate([[0, 1, 127, 128, N - 129, N - 128, N - 1], rng.integers(0, N, 41)]))
+        Wc = W[:, torch.from_numpy(cols).to(dev)].contiguous().cpu().numpy()
+        Cref, Cabs = oracle.gemm_with_abs(A.cpu().numpy(), Wc)
+        got = out[:, torch.from_numpy(cols).to(dev)].cpu().numpy()
+        e1, e2 = gemm_errors(got, Cref, Cabs)
+        tol = gemm_tolerance(K)
+        assert e1 <= tol and e2 <= tol, (K, e1, e2, tol)
+    # every column got written: compare column sums against a torch matmul of the column-summed W
+    colsum_ref = batch.double() @ W1[:, ::397].double()
+    assert float((out1[:, ::397].double() - colsum_ref).abs().max()) / float(colsum_ref.abs().max()) < gemm_tolerance(100000)
+
+
+def test_fused_w8_decode_is_bit_identical(dev):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(6)
+    K, N = 300, 1000
+    W = rng.integers(0, 256, (K, N), dtype=np.uint8)
+    I = np.eye(K, dtype=np.float32)
+    for scale in (1.0, 0.0371, 11.5):
+        got = cn.gemm_w8(_t(I, dev), _t(W, dev), scale).cpu().numpy()
+        want = oracle.decompress(W, scale)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), scale
+
+
+@pytest.mark.parametrize("batch", [32, 128, 512])
+def test_config4_fused_w8_gemm(dev, batch):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(8 + batch)
+    A = rng.normal(0, 1, (batch, 4096)).astype(np.float32)
+    Wf = rng.normal(0, 1 / 64.0, (4096, 4096)).astype(np.float32)
+    wt = _t(Wf, dev)
+    scale_dev = cn.absmax(wt)
+    scale = float(scale_dev.cpu()[0])
+    codes_t = cn.compression_8bit(wt, scale)
+    codes = codes_t.cpu().numpy()
+    assert np.array_equal(codes, oracle.port_compress(Wf, scale))
+    fused = cn.gemm_w8(_t(A, dev), codes_t, scale).cpu().numpy()
+    Wd = oracle.decompress(codes, scale)
+    Cref, Cabs = oracle.gemm_with_abs(A, Wd)
+    e1, e2 = gemm_errors(fused, Cref, Cabs)
+    assert e1 <= 1e-4 and e2 <= 1e-4, (e1, e2)
+    # and it agrees with decompress-then-dot on the device to the same tolerance
+    unfused = cn.dot(_t(A, dev), cn.decompression_8bit(codes_t, scale)).cpu().numpy()
+    assert np.abs(unfused - fused).max() / np.abs(Cref).max() <= 1e-4
+
+
+@pytest.mark.parametrize("shape", [(5, 7, 9), (130, 131, 65), (128, 1000, 30), (64, 4099, 257)])
+def test_fused_w8_ragged(dev, shape):
+    import clusternet_amd as cn
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    A = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = rng.integers(0, 256, (K, N), dtype=np.uint8)
+    got = cn.gemm_w8(_t(A, dev), _t(W, dev), 0.25).cpu().numpy()
+    Cref, Cabs = oracle.gemm_with_abs(A, oracle.decompress(W, 0.25))
+    e1, e2 = gemm_errors(got, Cref, Cabs)
+    assert e1 <= 1e-4 and e2 <= 1e-4, (e1, e2)
