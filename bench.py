@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the matrix-multiply + 8-bit codec path on one MI355X.
+
+A step is the README workload of the reference on ONE GPU, un-sharded and resident in HBM:
+    out1 = batch(128 x 100000) . W1(100000 x 40000);  out2 = out1 . W2(40000 x 20000)
+(fp32, ~19 GB, uniform inputs, synthetic).  `value` is (2*128*100000*40000 + 2*128*40000*20000)
+FLOP divided by the wall time of a step.  The dominant kernel is the 128 x 40000 x 100000 dot; its
+own duration is measured with events on the launch stream inside the timed steps and priced
+against the fp32 matrix-core peak.  After the timed region the codec kernels (compression_8bit,
+decompression_8bit, absmax) and the fused 8-bit-weight GEMM are measured on their own workloads and
+reported under "extra"; the CPU port of the same arithmetic is timed on a bounded sample.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|codec|fused] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_HBM_GBPS = 8000.0          # MI355X HBM3E peak
+
+M, K1, N1, N2 = 128, 100000, 40000, 20000
+FLOP1 = 2.0 * M * N1 * K1
+FLOP2 = 2.0 * M * N2 * N1
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
+# scaled by the reading of the same counters on a copy kernel of known size (see profiles/).
+# None until measured.
+TRAFFIC_BYTES_GEMM1 = None
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_uniform(torch, shape, limit, dev, gen, chunk_rows=10000):
+    out = torch.empty(shape, dtype=torch.float32, device=dev)
+    for r in range(0, shape[0], chunk_rows):
+        blk = out[r:r + chunk_rows]
+        blk.uniform_(-limit, limit, generator=gen)
+    return out
+
+
+def event_pair(torch):
+    return torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+
+def time_region(torch, fn, iters, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    s, e = event_pair(torch)
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters  # ms
+
+
+def bench_gemm(torch, cn, dev, steps, warmup):
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    batch = torch.rand((M, K1), device=dev, generator=gen)
+    W1 = make_uniform(torch, (K1, N1), (6.0 / (K1 + N1)) ** 0.5, dev, gen)
+    W2 = make_uniform(torch, (N1, N2), (6.0 / (N1 + N2)) ** 0.5, dev, gen)
+    out1 = torch.empty((M, N1), device=dev)
+    out2 = torch.empty((M, N2), device=dev)
+
+    def step(ev=None):
+        if ev is not None:
+            ev[0].record()
+        cn.dot(batch, W1, out1)
+        if ev is not None:
+            ev[1].record()
+        cn.dot(out1, W2, out2)
+        if ev is not None:
+            ev[2].record()
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    g1 = sum(e[0].elapsed_time(e[1]) for e in events) / steps
+    g2 = sum(e[1].elapsed_time(e[2]) for e in events) / steps
+    return {"wall_ms": wall_ms, "gemm1_ms": g1, "gemm2_ms": g2,
+            "tensors": (batch, W1, W2, out1, out2)}
+
+
+def bench_codec(torch, cn, dev):
+    """compression_8bit / decompression_8bit / absmax on the 100000 x 8192 gradient of the training
+    configuration (819.2 M elements, 3.28 GB fp32) and on the 128 x 40000 round-trip tensor."""
+    res = {}
+    gen = torch.Generator(device=dev).manual_seed(99)
+    for name, n, iters in (("grad_100000x8192", 100000 * 8192, 20), ("cfg2_128x40000", 128 * 40000, 200),
+                           ("ref_microbench_5120x5120", 5120 * 5120, 100)):
+        x = torch.empty(n, device=dev).normal_(0.0, 0.02, generator=gen)
+        idx = torch.randint(0, n, (n // 100,), device=dev, generator=gen)
+        x[idx] = torch.empty(idx.numel(), device=dev).normal_(0.0, 0.5, generator=gen)
+        del idx
+        prec_t = cn.absmax(x)
+        prec = float(prec_t.cpu()[0])
+        codes = torch.empty(n, dtype=torch.uint8, device=dev)
+        back = torch.empty(n, device=dev)
+        t_abs = time_region(torch, lambda: cn.absmax(x, prec_t), iters, 3)
+        t_c = time_region(torch, lambda: cn.compression_8bit(x, prec, codes), iters, 3)
+        t_d = time_region(torch, lambda: cn.decompression_8bit(codes, prec, back), iters, 3)
+        t_copy = time_region(torch, lambda: back.copy_(x), iters, 3)
+        res[name] = {
+            "elements": n,
+            "absmax_GBps": 4.0 * n / t_abs / 1e6, "absmax_us": t_abs * 1e3,
+            "compress_GBps": 5.0 * n / t_c / 1e6, "compress_us": t_c * 1e3,
+            "decompress_GBps": 5.0 * n / t_d / 1e6, "decompress_us": t_d * 1e3,
+            "copy_GBps": 8.0 * n / t_copy / 1e6,
+            "compress_frac_hbm_peak": 5.0 * n / t_c / 1e6 / PEAK_HBM_GBPS,
+            "decompress_frac_hbm_peak": 5.0 * n / t_d / 1e6 / PEAK_HBM_GBPS,
+        }
+        del x, codes, back
+    return res
+
+
+def bench_fused(torch, cn, dev):
+    """C = A . decode(W8) for A {32,128,512} x 4096, W 4096 x 4096: fused kernel against
+    decompression_8bit followed by dot."""
+    res = {}
+    gen = torch.Generator(device=dev).manual_seed(7)
+    W = torch.empty((4096, 4096), device=dev).normal_(0.0, 1.0 / 64.0, generator=gen)
+    scale = float(cn.absmax(W).cpu()[0])
+    codes = cn.compression_8bit(W, scale)
+    Wd = torch.empty_like(W)
+    for b in (32, 128, 512):
+        A = torch.empty((b, 4096), device=dev).normal_(0.0, 1.0, generator=gen)
+        C = torch.empty((b, 4096), device=dev)
+        t_f = time_region(torch, lambda: cn.gemm_w8(A, codes, scale, C), 200, 5)
+
+        def unfused():
+            cn.decompression_8bit(codes, scale, Wd)
+            cn.dot(A, Wd, C)
+        t_u = time_region(torch, unfused, 200, 5)
+        t_g = time_region(torch, lambda: cn.dot(A, Wd, C), 200, 5)
+        res["batch%d" % b] = {"fused_us": t_f * 1e3, "decompress_plus_dot_us": t_u * 1e3,
+                              "dot_fp32_only_us": t_g * 1e3, "speedup": t_u / t_f,
+                              "fused_TFLOPs": 2.0 * b * 4096 * 4096 / t_f / 1e9}
+    return res
+
+
+def cpu_baseline(torch, tensors):
+    """The CPU port (oracle/cpu_port.c, all OpenMP threads) on a column sample of the first dot."""
+    import numpy as np
+    import oracle
+    batch, W1 = tensors[0], tensors[1]
+    A = batch.cpu().numpy()
+    cols = 256
+    Ws = np.ascontiguousarray(W1[:, :cols].cpu().numpy())
+    t0 = time.perf_counter()
+    oracle.port_gemm_nn(A, Ws)
+    dt = time.perf_counter() - t0
+    rate = 2.0 * M * cols * K1 / dt
+    want = int(min(4096, max(256, (12.0 * rate) / (2.0 * M * K1))) // 256 * 256)
+    if want > cols:
+        cols = want
+        Ws = np.ascontiguousarray(W1[:, :cols].cpu().numpy())
+        t0 = time.perf_counter()
+        oracle.port_gemm_nn(A, Ws)
+        dt = time.perf_counter() - t0
+    return {"value": 2.0 * M * cols * K1 / dt / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(),
+            "kind": "port",
+            "sample": "first dot of the step on the first %d of %d output columns "
+                      "(128 x %d x %d fp32, %.2f s)" % (cols, N1, K1, cols, dt)}
+
+
+def cpu_codec_baseline():
+    """The literal per-element codec loops on all OpenMP threads, 64 M elements."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(0)
+    x = rng.normal(0.0, 0.02, 1 << 26).astype(np.float32)
+    prec = oracle.port_absmax(x)
+    t0 = time.perf_counter(); codes = oracle.port_compress(x, prec); tc = time.perf_counter() - t0
+    t0 = time.perf_counter(); oracle.port_decompress(codes, prec); td = time.perf_counter() - t0
+    return {"elements": x.size, "cores": oracle.num_threads(), "kind": "port",
+            "compress_GBps": 5.0 * x.size / tc / 1e9, "decompress_GBps": 5.0 * x.size / td / 1e9}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--only", choices=["gemm", "codec", "fused"], default=None,
+                    help="run one part only (for profiling); prints a reduced JSON line")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build runs the un-sharded workload on a single "
+                 "MI355X and has no multi-GPU path (--gpus %d refused)" % args.gpus)
+
+    import torch
+    import clusternet_amd as cn
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    cn.init(0)
+
+    line = {"metric": "fp32 GEMM TFLOP/s at 128x100000x40000 (%MFMA peak); 8-bit codec GB/s",
+            "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic",
+            "config": {"workload": "README dotMPI pair on one GPU, un-sharded: 128x100000 . 100000x40000 "
+                                   "then 128x40000 . 40000x20000, fp32, resident in HBM"}}
+    extra = {}
+    if args.only in (None, "gemm"):
+        g = bench_gemm(torch, cn, dev, args.steps, args.warmup)
+        line["value"] = (FLOP1 + FLOP2) / (g["wall_ms"] * 1e-3) / 1e12
+        line["ms_per_step"] = g["wall_ms"]
+        achieved = FLOP1 / (g["gemm1_ms"] * 1e-3) / 1e12
+        line["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
+                            "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                            "traffic": TRAFFIC_BYTES_GEMM1,
+                            "kernel": "gemm_kernel<A k-contiguous, B n-contiguous> + splitk_reduce_kernel, "
+                                      "128x40000x100000", "avg_ms": g["gemm1_ms"]}
+        extra["gemm2_128x20000x40000"] = {"ms": g["gemm2_ms"], "TFLOPs": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12,
+                                          "frac_mfma_peak": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS}
+        extra["readme_pair_ms_reference_unknown_hw"] = 117.704285
+        if not args.no_cpu and args.only is None:
+            line["cpu_baseline"] = cpu_baseline(torch, g["tensors"])
+        del g
+        torch.cuda.empty_cache()
+    if args.only in (None, "codec"):
+        extra["codec"] = bench_codec(torch, cn, dev)
+        torch.cuda.empty_cache()
+        if not args.no_cpu and args.only is None:
+            extra["codec"]["cpu_port"] = cpu_codec_baseline()
+    if args.only in (None, "fused"):
+        extra["fused_w8_gemm_4096x4096"] = bench_fused(torch, cn, dev)
+    line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -185,3 +185,119 @@ def decompression_8bit(codes, precision, out=None):
     else:
         check(lib().cn_decompress_8bit(codes.data_ptr(), float(precision), codes.numel(), out.data_ptr(), _stream()))
     return out
+
+
+# ---- small kernels around the path (bias, maxout, softmax, ...) ---------------------------------
+def _declare_layers(L):
+    i64, vp, f32, sz = C.c_int64, C.c_void_p, C.c_float, C.c_size_t
+    L.cn_transpose_f32.argtypes = [vp, i64, i64, vp, vp]
+    L.cn_affine_f32.argtypes = [vp, f32, f32, sz, vp, vp]
+    L.cn_abs_f32.argtypes = [vp, sz, vp, vp]
+    L.cn_sub_f32.argtypes = [vp, vp, sz, vp, vp]
+    L.cn_sum_f32.argtypes = [vp, sz, vp, vp]
+    L.cn_max_f32.argtypes = [vp, sz, vp, vp]
+    L.cn_sgd_update_f32.argtypes = [vp, vp, f32, sz, vp]
+    L.cn_add_row_vector_f32.argtypes = [vp, vp, i64, i64, vp, vp]
+    L.cn_maxout_f32.argtypes = [vp, i64, i64, C.c_int, vp, vp, vp]
+    L.cn_expand_to_maxout_grad_f32.argtypes = [vp, vp, i64, i64, C.c_int, vp, vp]
+    L.cn_softmax_f32.argtypes = [vp, i64, i64, vp, vp]
+    L.cn_timer_start.argtypes = [C.POINTER(vp), vp]
+    L.cn_timer_stop.argtypes = [vp, vp, C.POINTER(f32)]
+    return L
+
+
+def _contig(t, what):
+    import torch
+    _need(t, torch.float32, what)
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % what)
+    return t
+
+
+def transpose(A, out=None):
+    import torch
+    L = _declare_layers(lib())
+    _contig(A, "A")
+    if out is None:
+        out = torch.empty((A.shape[1], A.shape[0]), dtype=torch.float32, device=A.device)
+    check(L.cn_transpose_f32(A.data_ptr(), A.shape[0], A.shape[1], out.data_ptr(), _stream()))
+    return out
+
+
+def add_row_vector(A, v, out=None):
+    import torch
+    L = _declare_layers(lib())
+    _contig(A, "A")
+    _contig(v, "v")
+    if v.numel() != A.shape[1]:
+        raise CnError(2, "vector length %d does not match %d columns" % (v.numel(), A.shape[1]))
+    out = torch.empty_like(A) if out is None else out
+    check(L.cn_add_row_vector_f32(A.data_ptr(), v.data_ptr(), A.shape[0], A.shape[1], out.data_ptr(), _stream()))
+    return out
+
+
+def maxout(A, pool):
+    import torch
+    L = _declare_layers(lib())
+    _contig(A, "A")
+    out = torch.empty((A.shape[0], A.shape[1] // pool), dtype=torch.float32, device=A.device)
+    arg = torch.empty_like(out)
+    check(L.cn_maxout_f32(A.data_ptr(), A.shape[0], A.shape[1], int(pool), out.data_ptr(), arg.data_ptr(), _stream()))
+    return out, arg
+
+
+def expand_to_maxout_grad(err, argmax, pool, out=None):
+    import torch
+    L = _declare_layers(lib())
+    _contig(err, "err")
+    _contig(argmax, "argmax")
+    if out is None:
+        out = torch.empty((err.shape[0], err.shape[1] * pool), dtype=torch.float32, device=err.device)
+    check(L.cn_expand_to_maxout_grad_f32(err.data_ptr(), argmax.data_ptr(), err.shape[0], err.shape[1], int(pool),
+                                         out.data_ptr(), _stream()))
+    return out
+
+
+def softmax(A, out=None):
+    import torch
+    L = _declare_layers(lib())
+    _contig(A, "A")
+    out = torch.empty_like(A) if out is None else out
+    check(L.cn_softmax_f32(A.data_ptr(), A.shape[0], A.shape[1], out.data_ptr(), _stream()))
+    return out
+
+
+def sub(a, b, out=None):
+    import torch
+    L = _declare_layers(lib())
+    _contig(a, "a")
+    _contig(b, "b")
+    out = torch.empty_like(a) if out is None else out
+    check(L.cn_sub_f32(a.data_ptr(), b.data_ptr(), a.numel(), out.data_ptr(), _stream()))
+    return out
+
+
+def sgd_update(w, grad, rate):
+    L = _declare_layers(lib())
+    _contig(w, "w")
+    _contig(grad, "grad")
+    check(L.cn_sgd_update_f32(w.data_ptr(), grad.data_ptr(), float(rate), w.numel(), _stream()))
+    return w
+
+
+def reduce_sum(x):
+    import torch
+    L = _declare_layers(lib())
+    _contig(x, "x")
+    out = torch.empty(1, dtype=torch.float32, device=x.device)
+    check(L.cn_sum_f32(x.data_ptr(), x.numel(), out.data_ptr(), _stream()))
+    return out
+
+
+def reduce_max(x):
+    import torch
+    L = _declare_layers(lib())
+    _contig(x, "x")
+    out = torch.empty(1, dtype=torch.float32, device=x.device)
+    check(L.cn_max_f32(x.data_ptr(), x.numel(), out.data_ptr(), _stream()))
+    return out

@@ -69,9 +69,12 @@ def build_facade(verbose=False):
           os.path.join(FACADE, "basicOps.cpp")] + inc +
          ["-L" + HERE, "-lcnhip", "-Wl,-rpath,$ORIGIN"])
     test_src = os.path.join(ROOT, "tests", "cpp", "facade_test.cpp")
-    if os.path.exists(test_src):
+    oracle_dir = os.path.join(ROOT, "oracle")
+    if os.path.exists(test_src) and os.path.exists(os.path.join(oracle_dir, "liboracle.so")):
+        # the test program (not the library) links the CPU checker to compare codes bit for bit
         _run([cxx, "-O2", "-std=c++17", "-Wall", "-o", os.path.join(ROOT, "tests", "cpp", "facade_test"),
-              test_src] + inc + ["-L" + HERE, "-lclusternet", "-lcnhip", "-Wl,-rpath," + HERE])
+              test_src] + inc + ["-L" + HERE, "-lclusternet", "-lcnhip", "-L" + oracle_dir, "-loracle",
+                                 "-Wl,-rpath,$ORIGIN/../../clusternet_amd", "-Wl,-rpath,$ORIGIN/../../oracle"])
     return FACADE_LIB
 
 

@@ -217,13 +217,27 @@ __device__ __forceinline__ uint32_t block_max(uint32_t v, uint32_t *smem) {
     return v;  // valid in wave 0
 }
 
-template <bool kVector>
+// kAbs: key = |x| pattern.  Otherwise (plain max, start value -1 as in the reference's reduction)
+// the key is the usual order-preserving map of a signed fp32 pattern onto unsigned integers.
+template <bool kAbs>
+__device__ __forceinline__ uint32_t max_key(uint32_t bits) {
+    if (kAbs) return bits & 0x7fffffffu;
+    return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+}
+template <bool kAbs>
+__device__ __forceinline__ float max_unkey(uint32_t key) {
+    if (kAbs) return __uint_as_float(key);
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+template <bool kVector, bool kAbs>
 __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restrict__ x, size_t n,
                                                           float *__restrict__ out,
                                                           uint32_t *__restrict__ scratch) {
     __shared__ uint32_t smem[kThreads / 64];
     __shared__ uint32_t s_last;
-    uint32_t m = 0;
+    const uint32_t start = kAbs ? 0u : max_key<false>(0xbf800000u);
+    uint32_t m = start;
     if (kVector) {
         const size_t nvec = n / 4;
         const u32x4 *x4 = reinterpret_cast<const u32x4 *>(x);
@@ -234,23 +248,25 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
 #pragma unroll
             for (int j = 0; j < kVecPerThread; ++j) {
                 size_t i = base + (size_t)j * kThreads;
-                v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : u32x4{0u, 0u, 0u, 0u};
+                // positions past the end take the pattern whose key is the smallest possible
+                const uint32_t pad = kAbs ? 0u : 0xffffffffu;
+                v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : u32x4{pad, pad, pad, pad};
             }
 #pragma unroll
             for (int j = 0; j < kVecPerThread; ++j) {
-                m = max(m, v[j].x & 0x7fffffffu);
-                m = max(m, v[j].y & 0x7fffffffu);
-                m = max(m, v[j].z & 0x7fffffffu);
-                m = max(m, v[j].w & 0x7fffffffu);
+                m = max(m, max_key<kAbs>(v[j].x));
+                m = max(m, max_key<kAbs>(v[j].y));
+                m = max(m, max_key<kAbs>(v[j].z));
+                m = max(m, max_key<kAbs>(v[j].w));
             }
         }
         if (blockIdx.x == 0) {
             size_t i = nvec * 4 + threadIdx.x;
-            if (i < n) m = max(m, __float_as_uint(x[i]) & 0x7fffffffu);
+            if (i < n) m = max(m, max_key<kAbs>(__float_as_uint(x[i])));
         }
     } else {
         for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
-            m = max(m, __float_as_uint(x[i]) & 0x7fffffffu);
+            m = max(m, max_key<kAbs>(__float_as_uint(x[i])));
     }
     m = block_max(m, smem);
     // Publish the workgroup's maximum, then let the last workgroup to arrive fold all of them.
@@ -264,13 +280,13 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
     __syncthreads();
     if (s_last) {
         __threadfence();
-        uint32_t r = 0;
+        uint32_t r = start;
         for (uint32_t i = threadIdx.x; i < gridDim.x; i += blockDim.x)
             r = max(r, __hip_atomic_load(&scratch[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
         __syncthreads();
         r = block_max(r, smem);
         if (threadIdx.x == 0) {
-            out[0] = __uint_as_float(r);
+            out[0] = max_unkey<kAbs>(r);
             __hip_atomic_store(&scratch[kReduceSlots], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
@@ -374,9 +390,30 @@ cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
     if (!x) { set_error("absmax_f32: NULL input"); return CN_ERR_NULL; }
     int grid = stream_grid(ctx, n, 8);
     if (aligned(x, 16))
-        hipLaunchKernelGGL(absmax_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+        hipLaunchKernelGGL((absmax_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
     else
-        hipLaunchKernelGGL(absmax_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+        hipLaunchKernelGGL((absmax_kernel<false, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_max_f32(const float *x, size_t n, float *out, void *stream) {
+    if (!out) { set_error("max_f32: NULL output"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    if (n == 0) {
+        hipLaunchKernelGGL(set_scalar_kernel, dim3(1), dim3(64), 0, st, out, -1.0f);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
+    if (!x) { set_error("max_f32: NULL input"); return CN_ERR_NULL; }
+    int grid = stream_grid(ctx, n, 8);
+    if (aligned(x, 16))
+        hipLaunchKernelGGL((absmax_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+    else
+        hipLaunchKernelGGL((absmax_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

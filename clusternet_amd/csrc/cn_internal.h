@@ -54,7 +54,8 @@ struct Context {
     uint32_t lut_first = 0, lut_count = 0;
     void *workspace = nullptr;       // split-K partial sums
     size_t workspace_bytes = 0;
-    uint32_t *reduce_scratch = nullptr;  // per-workgroup partial maxima + ticket counter
+    uint32_t *reduce_scratch = nullptr;  // per-workgroup partial maxima + ticket counters
+    double *sum_scratch = nullptr;       // per-workgroup partial sums (1024 doubles)
 };
 constexpr int kMaxDevices = 16;
 constexpr int kReduceSlots = 4096;

@@ -1,0 +1,306 @@
+// Small element-wise / layout kernels the callers of the GEMM + codec path use around it: layout
+// transpose, scalar affine map, sum, bias broadcast, maxout with arg-max, its gradient scatter,
+// row softmax, difference, and a plain gradient step.  All row-major, all HBM-bound streaming
+// kernels; none of them is on the measured hot path.
+#include <float.h>
+
+#include "cn_internal.h"
+
+namespace cn {
+
+constexpr int kT = 256;
+
+static inline int grid_for(const Context *ctx, int64_t work_items, int per_cu = 8) {
+    int64_t blocks = (work_items + kT - 1) / kT;
+    int64_t cap = (int64_t)ctx->num_cu * per_cu;
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// out[c][r] = in[r][c]; 32 x 32 tiles through LDS (33-float pitch), both sides coalesced.
+__global__ __launch_bounds__(kT) void transpose_kernel(const float *__restrict__ in, int64_t rows, int64_t cols,
+                                                       float *__restrict__ out) {
+    __shared__ float tile[32][33];
+    const int64_t tiles_c = (cols + 31) / 32, tiles_r = (rows + 31) / 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int64_t t = blockIdx.x; t < tiles_c * tiles_r; t += gridDim.x) {
+        const int64_t r0 = (t / tiles_c) * 32, c0 = (t % tiles_c) * 32;
+#pragma unroll
+        for (int j = 0; j < 32; j += 8) {
+            int64_t r = r0 + ty + j, c = c0 + tx;
+            if (r < rows && c < cols) tile[ty + j][tx] = in[r * cols + c];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 32; j += 8) {
+            int64_t c = c0 + ty + j, r = r0 + tx;
+            if (r < rows && c < cols) out[c * rows + r] = tile[tx][ty + j];
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(kT) void affine_kernel(const float *__restrict__ x, float mul, float add, int64_t n,
+                                                    float *__restrict__ out) {
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
+        out[i] = x[i] * mul + add;
+}
+
+__global__ __launch_bounds__(kT) void abs_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ out) {
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
+        out[i] = fabsf(x[i]);
+}
+
+__global__ __launch_bounds__(kT) void sub_kernel(const float *__restrict__ a, const float *__restrict__ b, int64_t n,
+                                                 float *__restrict__ out) {
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
+        out[i] = a[i] - b[i];
+}
+
+// w[i] -= rate * g[i]
+__global__ __launch_bounds__(kT) void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, float rate,
+                                                 int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
+        w[i] = w[i] - rate * g[i];
+}
+
+// out[r][c] = A[r][c] + v[c]
+__global__ __launch_bounds__(kT) void add_row_vector_kernel(const float *__restrict__ A, const float *__restrict__ v,
+                                                            int64_t rows, int64_t cols, float *__restrict__ out) {
+    const int64_t n = rows * cols;
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
+        out[i] = A[i] + v[i % cols];
+}
+
+// Maxout over `pool` consecutive columns; arg-max is the absolute column index as a float, the
+// first maximum wins (strict comparison, as the reference's reduction).
+__global__ __launch_bounds__(kT) void maxout_kernel(const float *__restrict__ A, int64_t rows, int64_t cols, int pool,
+                                                    float *__restrict__ out, float *__restrict__ argmax) {
+    const int64_t oc = cols / pool, n = rows * oc;
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) {
+        const int64_t r = i / oc, o = i % oc;
+        const float *src = A + r * cols + o * pool;
+        float best = src[0];
+        int arg = 0;
+        for (int p = 1; p < pool; ++p) {
+            float v = src[p];
+            if (best < v) { best = v; arg = p; }
+        }
+        out[i] = best;
+        argmax[i] = (float)(o * pool + arg);
+    }
+}
+
+// out (rows x pooled*pool): the pooled error lands on the winner's column, zero elsewhere.
+__global__ __launch_bounds__(kT) void expand_maxout_grad_kernel(const float *__restrict__ err,
+                                                                const float *__restrict__ argmax, int64_t rows,
+                                                                int64_t pooled, int pool, float *__restrict__ out) {
+    const int64_t cols = pooled * pool, n = rows * cols;
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) {
+        const int64_t r = i / cols, c = i % cols;
+        const int64_t o = c / pool;
+        out[i] = ((int64_t)argmax[r * pooled + o] == c) ? err[r * pooled + o] : 0.0f;
+    }
+}
+
+// One wavefront per row: max, sum of exp, normalise.
+__global__ __launch_bounds__(kT) void softmax_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
+                                                     float *__restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = ((int64_t)blockIdx.x * kT + threadIdx.x) >> 6;
+    const int64_t nwaves = ((int64_t)gridDim.x * kT) >> 6;
+    for (int64_t r = wave; r < rows; r += nwaves) {
+        const float *src = A + r * cols;
+        float m = -FLT_MAX;
+        for (int64_t c = lane; c < cols; c += 64) m = fmaxf(m, src[c]);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+        float s = 0.0f;
+        for (int64_t c = lane; c < cols; c += 64) s += expf(src[c] - m);
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+        for (int64_t c = lane; c < cols; c += 64) out[r * cols + c] = expf(src[c] - m) / s;
+    }
+}
+
+// Deterministic two-stage sum in fp64: fixed grid, per-workgroup partials, last workgroup folds.
+__global__ __launch_bounds__(kT) void sum_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ out,
+                                                 double *__restrict__ partial, uint32_t *__restrict__ counter) {
+    __shared__ double sm[kT];
+    __shared__ uint32_t s_last;
+    double s = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) s += (double)x[i];
+    sm[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = kT / 2; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) sm[threadIdx.x] += sm[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&partial[blockIdx.x], sm[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();
+        s_last = (atomicAdd(counter, 1u) == gridDim.x - 1) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (s_last && threadIdx.x == 0) {
+        __threadfence();
+        double t = 0.0;
+        for (uint32_t b = 0; b < gridDim.x; ++b)
+            t += __hip_atomic_load(&partial[b], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        out[0] = (float)t;
+        __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+}  // namespace cn
+
+using namespace cn;
+
+#define CN_ENTER(name)                                   \
+    Context *ctx;                                        \
+    {                                                    \
+        cn_status s_ = current_context(&ctx);            \
+        if (s_ != CN_OK) return s_;                      \
+    }                                                    \
+    hipStream_t st = (hipStream_t)stream;                \
+    (void)st;
+
+#define CN_REQUIRE(cond, code, msg)                      \
+    do {                                                 \
+        if (!(cond)) { set_error("%s", msg); return code; } \
+    } while (0)
+
+extern "C" {
+
+cn_status cn_transpose_f32(const float *in, int64_t rows, int64_t cols, float *out, void *stream) {
+    CN_REQUIRE(rows >= 0 && cols >= 0, CN_ERR_SHAPE, "transpose_f32: negative dimension");
+    if (rows == 0 || cols == 0) return CN_OK;
+    CN_REQUIRE(in && out, CN_ERR_NULL, "transpose_f32: NULL pointer");
+    CN_REQUIRE(in != out, CN_ERR_ARG, "transpose_f32: in-place transpose is not supported");
+    CN_ENTER();
+    int64_t tiles = ((rows + 31) / 32) * ((cols + 31) / 32);
+    int64_t cap = (int64_t)ctx->num_cu * 8;
+    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(kT), 0, st, in, rows, cols, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_affine_f32(const float *x, float mul, float add, size_t n, float *out, void *stream) {
+    if (n == 0) return CN_OK;
+    CN_REQUIRE(x && out, CN_ERR_NULL, "affine_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(affine_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, x, mul, add, (int64_t)n, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_abs_f32(const float *x, size_t n, float *out, void *stream) {
+    if (n == 0) return CN_OK;
+    CN_REQUIRE(x && out, CN_ERR_NULL, "abs_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(abs_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, x, (int64_t)n, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_sub_f32(const float *a, const float *b, size_t n, float *out, void *stream) {
+    if (n == 0) return CN_OK;
+    CN_REQUIRE(a && b && out, CN_ERR_NULL, "sub_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(sub_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, a, b, (int64_t)n, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_sgd_update_f32(float *w, const float *grad, float rate, size_t n, void *stream) {
+    if (n == 0) return CN_OK;
+    CN_REQUIRE(w && grad, CN_ERR_NULL, "sgd_update_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, w, grad, rate, (int64_t)n);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_add_row_vector_f32(const float *A, const float *v, int64_t rows, int64_t cols, float *out, void *stream) {
+    CN_REQUIRE(rows >= 0 && cols >= 0, CN_ERR_SHAPE, "add_row_vector_f32: negative dimension");
+    if (rows == 0 || cols == 0) return CN_OK;
+    CN_REQUIRE(A && v && out, CN_ERR_NULL, "add_row_vector_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(add_row_vector_kernel, dim3(grid_for(ctx, rows * cols)), dim3(kT), 0, st, A, v, rows, cols, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_maxout_f32(const float *A, int64_t rows, int64_t cols, int pool, float *out, float *argmax, void *stream) {
+    CN_REQUIRE(rows >= 0 && cols >= 0 && pool >= 1, CN_ERR_SHAPE, "maxout_f32: bad dimension");
+    CN_REQUIRE(cols % pool == 0, CN_ERR_SHAPE, "maxout_f32: columns are not a multiple of the pool size");
+    if (rows == 0 || cols == 0) return CN_OK;
+    CN_REQUIRE(A && out && argmax, CN_ERR_NULL, "maxout_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(maxout_kernel, dim3(grid_for(ctx, rows * (cols / pool))), dim3(kT), 0, st, A, rows, cols, pool, out, argmax);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_expand_to_maxout_grad_f32(const float *err, const float *argmax, int64_t rows, int64_t pooled_cols,
+                                       int pool, float *out, void *stream) {
+    CN_REQUIRE(rows >= 0 && pooled_cols >= 0 && pool >= 1, CN_ERR_SHAPE, "expand_to_maxout_grad_f32: bad dimension");
+    if (rows == 0 || pooled_cols == 0) return CN_OK;
+    CN_REQUIRE(err && argmax && out, CN_ERR_NULL, "expand_to_maxout_grad_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(expand_maxout_grad_kernel, dim3(grid_for(ctx, rows * pooled_cols * pool)), dim3(kT), 0, st,
+                       err, argmax, rows, pooled_cols, pool, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_softmax_f32(const float *A, int64_t rows, int64_t cols, float *out, void *stream) {
+    CN_REQUIRE(rows >= 0 && cols >= 0, CN_ERR_SHAPE, "softmax_f32: negative dimension");
+    if (rows == 0 || cols == 0) return CN_OK;
+    CN_REQUIRE(A && out, CN_ERR_NULL, "softmax_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(softmax_kernel, dim3(grid_for(ctx, rows * 64)), dim3(kT), 0, st, A, rows, cols, out);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_sum_f32(const float *x, size_t n, float *out_device, void *stream) {
+    CN_REQUIRE(out_device, CN_ERR_NULL, "sum_f32: NULL output");
+    CN_REQUIRE(n == 0 || x, CN_ERR_NULL, "sum_f32: NULL input");
+    CN_ENTER();
+    int grid = grid_for(ctx, (int64_t)(n ? n : 1), 4);
+    if (grid > 1024) grid = 1024;
+    // arrival counter: the slot after the abs-max kernel's counter
+    hipLaunchKernelGGL(sum_kernel, dim3(grid), dim3(kT), 0, st, x, (int64_t)n, out_device, ctx->sum_scratch,
+                       ctx->reduce_scratch + kReduceSlots + 1);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+// Stopwatch on a stream (hipEvent pair), the counterpart of the reference's tick/tock helpers
+// (source/util.cu:218-252).
+struct cn_timer { hipEvent_t start, stop; };
+
+cn_status cn_timer_start(void **handle, void *stream) {
+    CN_REQUIRE(handle, CN_ERR_NULL, "timer_start: NULL handle");
+    cn_timer *t = new cn_timer;
+    CN_HIP(hipEventCreate(&t->start));
+    CN_HIP(hipEventCreate(&t->stop));
+    CN_HIP(hipEventRecord(t->start, (hipStream_t)stream));
+    *handle = t;
+    return CN_OK;
+}
+
+cn_status cn_timer_stop(void *handle, void *stream, float *milliseconds) {
+    CN_REQUIRE(handle && milliseconds, CN_ERR_NULL, "timer_stop: NULL pointer");
+    cn_timer *t = static_cast<cn_timer *>(handle);
+    CN_HIP(hipEventRecord(t->stop, (hipStream_t)stream));
+    CN_HIP(hipEventSynchronize(t->stop));
+    CN_HIP(hipEventElapsedTime(milliseconds, t->start, t->stop));
+    CN_HIP(hipEventDestroy(t->start));
+    CN_HIP(hipEventDestroy(t->stop));
+    delete t;
+    return CN_OK;
+}
+
+}  // extern "C"

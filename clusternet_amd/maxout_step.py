@@ -1,0 +1,52 @@
+"""One training step of a maxout MLP written against the path's operators, the way the reference's
+callers compose them (forward: source/test.cu:266-291 and source/Layer.cpp:250-261; backward:
+source/Layer.cpp:314-339; 8-bit gradient round trip: source/Layer.cpp:365,433 and
+source/DeepNeuralNetwork.cpp:334-339).  Host-side glue only: every array operation is one call
+into libcnhip.
+
+    z1 = X W1 + b1;  h1, a1 = maxout(z1);  z2 = h1 W2 + b2;  h2, a2 = maxout(z2)
+    p  = softmax(h2 W3 + b3);  e3 = p - onehot(y)
+    gW3 = h2^T e3;  e2 = expand(e3 W3^T, a2);  gW2 = h1^T e2;  e1 = expand(e2 W2^T, a1);  gW1 = X^T e1
+    each gW -> absmax -> compression_8bit -> decompression_8bit -> W -= rate * gW'
+Biases are inputs and are not updated.
+"""
+from . import _lib as L
+
+
+def forward(X, params, pool=2):
+    W1, b1, W2, b2, W3, b3 = params
+    z1 = L.add_row_vector(L.dot(X, W1), b1)
+    h1, a1 = L.maxout(z1, pool)
+    z2 = L.add_row_vector(L.dot(h1, W2), b2)
+    h2, a2 = L.maxout(z2, pool)
+    p = L.softmax(L.add_row_vector(L.dot(h2, W3), b3))
+    return p, (h1, a1, h2, a2)
+
+
+def backward(X, onehot, params, p, cache, pool=2):
+    W1, b1, W2, b2, W3, b3 = params
+    h1, a1, h2, a2 = cache
+    e3 = L.sub(p, onehot)
+    gW3 = L.Tdot(h2, e3)
+    e2 = L.expand_to_maxout_grad(L.dotT(e3, W3), a2, pool)
+    gW2 = L.Tdot(h1, e2)
+    e1 = L.expand_to_maxout_grad(L.dotT(e2, W2), a1, pool)
+    gW1 = L.Tdot(X, e1)
+    return gW1, gW2, gW3
+
+
+def codec_round_trip(grad):
+    """absmax -> compression_8bit -> decompression_8bit without a host synchronisation."""
+    prec = L.absmax(grad)
+    codes = L.compression_8bit(grad, prec)
+    return L.decompression_8bit(codes, prec, out=grad), codes, prec
+
+
+def step(X, onehot, params, rate, pool=2):
+    p, cache = forward(X, params, pool)
+    grads = backward(X, onehot, params, p, cache, pool)
+    W = (params[0], params[2], params[4])
+    for w, g in zip(W, grads):
+        g8, _, _ = codec_round_trip(g)
+        L.sgd_update(w, g8, rate)
+    return p

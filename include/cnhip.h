@@ -84,10 +84,14 @@ cn_status cn_gemm_f32_w8(int64_t M, int64_t N, int64_t K, const float *A_device,
                          const uint8_t *W_device, int64_t ldw, float scale, float *C_device,
                          int64_t ldc, void *stream);
 
-/* *out_device = max_i |x_i| (n == 0 gives 0; a NaN input gives NaN).  One pass, no temporary.
+/* *out_device = max_i |x_i| (n == 0 gives -1, the start value of the reference's reduction; a NaN
+ * input gives NaN).  One pass, no temporary.
  * Replaces the abs + max pair callers use to obtain `precision` (source/basicOps.cu:810-822 and
  * :1076-1081; call sites source/test.cu:2108-2109, source/DeepNeuralNetwork.cpp:218-222). */
 cn_status cn_absmax_f32(const float *x_device, size_t n, float *out_device, void *stream);
+/* *out_device = max(-1, max_i x_i): the reference's max (source/basicOps.cu:1076-1081), whose
+ * reduction starts from -1.  NaN inputs are ordered by their bit pattern. */
+cn_status cn_max_f32(const float *x_device, size_t n, float *out_device, void *stream);
 
 /* codes[i] = 8-bit code of x[i] / precision, bit-exact with kCompression_8bit
  * (source/clusterKernels.cu:1163-1232; launcher source/basicOps.cu:1163-1168), flat over n
@@ -108,6 +112,50 @@ cn_status cn_decompress_8bit(const uint8_t *codes_device, float precision, size_
                              float *out_device, void *stream);
 cn_status cn_decompress_8bit_dp(const uint8_t *codes_device, const float *precision_device,
                                 size_t n, float *out_device, void *stream);
+
+/* ---- small kernels used around the path by its callers (row-major, flat where no shape is given).
+ * They are not on the measured hot path; each names the reference routine it stands in for. */
+
+/* out[c][r] = in[r][c] (out is cols x rows).  kTranspose, source/clusterKernels.cu:457-482, the
+ * engine of to_col_major / to_row_major / T (source/basicOps.cu:91-137). */
+cn_status cn_transpose_f32(const float *in_device, int64_t rows, int64_t cols, float *out_device,
+                           void *stream);
+/* out[i] = x[i] * mul + add.  scalarMul / scalarAdd, source/basicOps.cu:603-631. */
+cn_status cn_affine_f32(const float *x_device, float mul, float add, size_t n, float *out_device,
+                        void *stream);
+/* out[i] = |x[i]|.  abs, source/basicOps.cu:810-822. */
+cn_status cn_abs_f32(const float *x_device, size_t n, float *out_device, void *stream);
+/* out[i] = a[i] - b[i].  sub, source/basicOps.cu:456-468. */
+cn_status cn_sub_f32(const float *a_device, const float *b_device, size_t n, float *out_device,
+                     void *stream);
+/* *out_device = sum_i x[i], accumulated in fp64 in a fixed order.  sum, source/basicOps.cu:1070-1074. */
+cn_status cn_sum_f32(const float *x_device, size_t n, float *out_device, void *stream);
+/* w[i] -= rate * grad[i]: the plain gradient step of the training configuration (the reference's
+ * fused optimisers, source/clusterKernels.cu:1306-1346, are outside this path). */
+cn_status cn_sgd_update_f32(float *w_device, const float *grad_device, float rate, size_t n,
+                            void *stream);
+/* out[r][c] = A[r][c] + v[c].  addMatrixVector, source/basicOps.cu:966-974. */
+cn_status cn_add_row_vector_f32(const float *A_device, const float *v_device, int64_t rows,
+                                int64_t cols, float *out_device, void *stream);
+/* Maxout over `pool` consecutive columns: out and argmax are rows x cols/pool; argmax holds the
+ * winner's absolute column index as a float, first maximum wins.  maxout,
+ * source/basicOps.cu:1272-1299 (defined by the expectations of tests/basicOps_test.cu:580-610). */
+cn_status cn_maxout_f32(const float *A_device, int64_t rows, int64_t cols, int pool,
+                        float *out_device, float *argmax_device, void *stream);
+/* out (rows x pooled_cols*pool) receives err at each winner's column and zero elsewhere.
+ * expand_to_maxout_grad, source/basicOps.cu:1315-1321 (tests/basicOps_test.cu:612-638). */
+cn_status cn_expand_to_maxout_grad_f32(const float *err_device, const float *argmax_device,
+                                       int64_t rows, int64_t pooled_cols, int pool,
+                                       float *out_device, void *stream);
+/* Row-wise softmax with max subtraction.  softmax, source/basicOps.cu:1012-1018. */
+cn_status cn_softmax_f32(const float *A_device, int64_t rows, int64_t cols, float *out_device,
+                         void *stream);
+
+/* Stopwatch on a stream: cn_timer_start records a start event and returns a handle;
+ * cn_timer_stop records the stop event, waits for it, returns the elapsed milliseconds and
+ * releases the handle.  tick / tock, source/util.cu:218-252. */
+cn_status cn_timer_start(void **handle, void *stream);
+cn_status cn_timer_stop(void *handle, void *stream, float *milliseconds);
 
 #ifdef __cplusplus
 }

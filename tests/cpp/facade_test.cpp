@@ -1,0 +1,319 @@
+// Test program for the C++ ClusterNet / Matrix layer, written the way the reference tests itself
+// (tests/clusterNet_test.cu, tests/basicOps_test.cu): one ClusterNet object passed by value, host
+// matrices built by hand, to_gpu / to_host around every call, asserts on literals.  Where the
+// reference compares floats with ==, a matrix-core kernel may differ in the last bit, so the
+// product literals are compared to 1e-6 relative; integer-valued results stay exact.
+// The codec is checked bit for bit against the CPU checker (oracle/liboracle.so).
+// Run by tests/test_gpu_facade.py on the GPU box; prints "ALL FACADE TESTS PASSED" on success.
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <vector>
+
+#include "clusterNet.h"
+
+extern "C" {
+void cn_oracle_compress_literal(const float *x, float precision, size_t n, uint8_t *codes, int sliver_rule);
+void cn_oracle_decompress(const uint8_t *codes, float precision, size_t n, float *out);
+}
+
+static int failures = 0;
+#define CHECK(cond, msg)                                                        \
+    do {                                                                        \
+        if (!(cond)) { printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, msg); ++failures; } \
+    } while (0)
+
+static bool close_to(float got, float want, const char *msg) {
+    float tol = 1e-6f * fabsf(want);
+    if (fabsf(got - want) <= tol) return true;
+    printf("%s: %.9g != %.9g\n", msg, got, want);
+    return false;
+}
+
+static bool test_matrix(Matrix *A, int rows, int cols) {
+    return A->rows == rows && A->cols == cols && A->size == (long long)rows * cols &&
+           A->bytes == sizeof(float) * (size_t)rows * cols;
+}
+
+static Matrix *host_matrix(int rows, int cols, const float *values) {
+    Matrix *m = empty_cpu(rows, cols);
+    memcpy(m->data, values, m->bytes);
+    return m;
+}
+
+static void run_clusterNet_test(ClusterNet gpus) {
+    ClusterNet gpu = ClusterNet(12345);
+    gpu.tick("ClusterNet test ran in");
+
+    //      0 2    3             17 0
+    // m1 = 0 0.83 59.1387  m2 =  3 4
+    //                            0 0
+    const float m1_data[6] = {0, 2, 3, 0, 0.83f, 59.1387f};
+    const float m2_data[6] = {17, 0, 3, 4, 0, 0};
+    Matrix *m1 = to_gpu(host_matrix(2, 3, m1_data));
+    Matrix *m2 = to_gpu(host_matrix(3, 2, m2_data));
+
+    Matrix *m_host = to_host(m1);
+    for (int i = 0; i < 6; ++i) CHECK(m_host->data[i] == m1_data[i], "to_gpu/to_host round trip");
+
+    // dot
+    Matrix *m3 = gpu.dot(m1, m2);
+    m_host = to_host(m3);
+    CHECK(test_matrix(m_host, 2, 2), "dot shape");
+    CHECK(close_to(m_host->data[0], 6.0f, "Dot data."), "dot");
+    CHECK(close_to(m_host->data[1], 8.0f, "Dot data."), "dot");
+    CHECK(close_to(m_host->data[2], 2.49f, "Dot data."), "dot");
+    CHECK(close_to(m_host->data[3], 3.32f, "Dot data."), "dot");
+    Matrix *out = zeros(2, 2);
+    gpu.dot(m1, m2, out);
+    m_host = to_host(out);
+    CHECK(close_to(m_host->data[0], 6.0f, "Dot data."), "dot out");
+    CHECK(close_to(m_host->data[3], 3.32f, "Dot data."), "dot out");
+
+    // Tdot
+    out = zeros(3, 3);
+    gpu.Tdot(m1, m1, out);
+    m_host = to_host(out);
+    const float tdot_want[9] = {0, 0, 0, 0, 4.6889f, 55.085117f, 0, 55.085117f, 3506.385742f};
+    for (int i = 0; i < 9; ++i) CHECK(close_to(m_host->data[i], tdot_want[i], "Tdot data."), "Tdot");
+    out = zeros(2, 2);
+    gpu.Tdot(m2, m2, out);
+    m_host = to_host(out);
+    const float tdot2_want[4] = {298, 12, 12, 16};
+    for (int i = 0; i < 4; ++i) CHECK(m_host->data[i] == tdot2_want[i], "Tdot integer data");
+    Matrix *t = gpu.Tdot(m1, m1);
+    CHECK(test_matrix(t, 3, 3), "Tdot value overload shape");
+
+    // dotT
+    gpu.dotT(m1, m1, out);
+    m_host = to_host(out);
+    const float dott_want[4] = {13.0f, 179.0761f, 179.0761f, 3498.074463f};
+    for (int i = 0; i < 4; ++i) CHECK(close_to(m_host->data[i], dott_want[i], "dotT data."), "dotT");
+
+    // shape errors throw the reference's literal
+    bool threw = false;
+    try { gpu.dot(m1, m1); } catch (const char *e) { threw = strcmp(e, "Matrix *size error:\n") == 0; }
+    CHECK(threw, "dot with mismatching inner dimensions must throw");
+    threw = false;
+    try { gpu.dot(m1, m2, zeros(3, 2)); } catch (const char *e) { threw = strcmp(e, "Matrix *size error:\n") == 0; }
+    CHECK(threw, "dot with a wrong output shape must throw");
+
+    // dotMPI == dot, element by element (reference: 0.3 x (1 + 0.1748345) constants)
+    m1 = scalarMul(ones(200, 400), 0.3f);
+    m2 = scalarAdd(ones(400, 800), 0.1748345f);
+    m3 = to_host(gpus.dot(m1, m2));
+    Matrix *m4 = to_host(gpus.dotMPI(m1, m2));
+    CHECK(test_matrix(m3, 200, 800) && test_matrix(m4, 200, 800), "dotMPI shape");
+    for (long long i = 0; i < m3->size; ++i)
+        if (m3->data[i] != m4->data[i]) { CHECK(false, "dotMPI Test"); break; }
+
+    // all-ones closed forms through dot / dotTMPI / dot into an existing matrix
+    m1 = gpus.distributed_ones(8783, 317);
+    m2 = ones(111, 8783);
+    m3 = ones(17, 317);
+    m4 = ones(8783, 17);
+    for (int epoch = 0; epoch < 2; ++epoch) {
+        m_host = to_host(gpus.dot(m2, m1));
+        CHECK(test_matrix(m_host, 111, 317), "ones dot shape");
+        for (long long i = 0; i < m_host->size; ++i)
+            if (m_host->data[i] != 8783.0f) { CHECK(false, "dotMPI test 8783"); break; }
+        m_host = to_host(gpus.dotTMPI(m3, m1));
+        CHECK(test_matrix(m_host, 17, 8783), "ones dotT shape");
+        for (long long i = 0; i < m_host->size; ++i)
+            if (m_host->data[i] != 317.0f) { CHECK(false, "dotMPI test 317"); break; }
+        gpus.dotMPI(m4, m3, m1);
+        m_host = to_host(m1);
+        for (long long i = 0; i < m_host->size; ++i)
+            if (m_host->data[i] != 17.0f) { CHECK(false, "dotMPI test 17"); break; }
+        m1 = gpus.distributed_ones(8783, 317);
+    }
+
+    // uniformSqrtWeight bounds (reference: +-4 sqrt(6 / (in + out)), almost never exactly zero)
+    m_host = to_host(gpus.distributed_uniformSqrtWeight(1000, 100));
+    int zeros_seen = 0;
+    const float lim = 4.0f * sqrtf(6.0f / (1000.0f + 100.0f));
+    for (long long i = 0; i < m_host->size; ++i) {
+        if (!(m_host->data[i] > -lim && m_host->data[i] < lim)) { CHECK(false, "RdmSqrtWeight bound"); break; }
+        if (m_host->data[i] == 0) ++zeros_seen;
+    }
+    CHECK(zeros_seen < 10, "RdmSqrtWeight zeros");
+
+    // rand / randn statistics
+    m_host = to_host(gpu.rand(100, 100));
+    int upper = 0, lower = 0;
+    for (long long i = 0; i < m_host->size; ++i) {
+        CHECK(m_host->data[i] >= 0.0f && m_host->data[i] < 1.0f, "rand range");
+        if (m_host->data[i] > 0.5f) ++upper; else ++lower;
+    }
+    CHECK(upper > 4600 && upper < 5400 && lower > 4600 && lower < 5400, "rand halves");
+    m_host = to_host(gpu.randn(100, 100));
+    double mean = 0;
+    for (long long i = 0; i < m_host->size; ++i) mean += m_host->data[i];
+    CHECK(fabs(mean / m_host->size) < 0.05, "randn mean");
+
+    float ms = gpu.tock("ClusterNet test ran in");
+    CHECK(ms > 0.0f, "tick/tock measures time");
+    // cumulative mode: tick twice accumulates, tock returns the total once
+    gpu.tick("acc"); gpu.tick("acc"); gpu.tick("acc"); gpu.tick("acc");
+    CHECK(gpu.tock("acc") >= 0.0f, "cumulative tock");
+}
+
+static void run_codec_test(ClusterNet gpu) {
+    // gradient-like data with outliers, precision = max |x| obtained both ways
+    Matrix *A = gpu.randn(128, 4000, 0.0f, 0.02f);
+    Matrix *a_host = to_host(A);
+    for (long long i = 0; i < a_host->size; i += 97) a_host->data[i] *= 25.0f;
+    A = to_gpu(a_host);
+    float precision = max(abs(A));
+    CHECK(precision == absmax(A), "max(abs(A)) equals absmax(A)");
+    float host_max = 0;
+    for (long long i = 0; i < a_host->size; ++i) host_max = fmaxf(host_max, fabsf(a_host->data[i]));
+    CHECK(precision == host_max, "precision equals the host maximum");
+
+    Matrix *codes = gpu.compression_8bit(A, precision);
+    CHECK(codes->rows == 128 && codes->cols == 4000 && codes->bytes == 128 * 4000, "empty_char shape");
+    Matrix *codes_host = to_host(codes);
+    std::vector<uint8_t> want(a_host->size);
+    cn_oracle_compress_literal(a_host->data, precision, (size_t)a_host->size, want.data(), 0);
+    CHECK(memcmp(want.data(), codes_host->char_data, want.size()) == 0, "compression_8bit codes are bit-exact");
+
+    Matrix *back = gpu.decompression_8bit(codes, precision);
+    Matrix *back_host = to_host(back);
+    std::vector<float> want_f(a_host->size);
+    cn_oracle_decompress(want.data(), precision, want.size(), want_f.data());
+    CHECK(memcmp(want_f.data(), back_host->data, back_host->bytes) == 0, "decompression_8bit is bit-exact");
+
+    // out-overloads write into caller storage
+    Matrix *codes2 = empty_char(128, 4000);
+    gpu.compression_8bit(A, precision, codes2);
+    CHECK(memcmp(to_host(codes2)->char_data, want.data(), want.size()) == 0, "compression_8bit(out)");
+    Matrix *back2 = empty(128, 4000);
+    gpu.decompression_8bit(codes2, precision, back2);
+    CHECK(memcmp(to_host(back2)->data, want_f.data(), back_host->bytes) == 0, "decompression_8bit(out)");
+
+    // fused product on coded weights against dot on the decoded weights
+    Matrix *W = gpu.randn(4000, 96, 0.0f, 0.05f);
+    float pw = absmax(W);
+    Matrix *Wc = gpu.compression_8bit(W, pw);
+    Matrix *X = gpu.rand(128, 4000);
+    Matrix *fused = to_host(gpu.dot8bit_weights(X, Wc, pw));
+    Matrix *plain = to_host(gpu.dot(X, gpu.decompression_8bit(Wc, pw)));
+    float worst = 0, scale = 0;
+    for (long long i = 0; i < fused->size; ++i) {
+        worst = fmaxf(worst, fabsf(fused->data[i] - plain->data[i]));
+        scale = fmaxf(scale, fabsf(plain->data[i]));
+    }
+    CHECK(worst <= 1e-4f * scale, "fused 8-bit-weight product matches decompress + dot");
+}
+
+static void run_basicOps_test(ClusterNet gpu) {
+    // layout round trips (reference tests/basicOps_test.cu:20-57,200-247)
+    Matrix *m1 = gpu.rand(37, 53);
+    Matrix *h = to_host(m1);
+    Matrix *t = to_host(T(m1));
+    CHECK(test_matrix(t, 53, 37), "T shape");
+    for (int r = 0; r < 37; ++r)
+        for (int c = 0; c < 53; ++c)
+            if (t->data[c * 37 + r] != h->data[r * 53 + c]) { CHECK(false, "T data"); r = 37; break; }
+    Matrix *rt = to_host(to_row_major(to_col_major(m1)));
+    CHECK(memcmp(rt->data, h->data, h->bytes) == 0, "to_col_major / to_row_major round trip");
+
+    // element-wise helpers with closed-form expectations
+    Matrix *o = to_host(scalarAdd(scalarMul(ones(10, 7), 3.0f), 0.5f));
+    for (long long i = 0; i < o->size; ++i) CHECK(o->data[i] == 3.5f, "scalarMul/scalarAdd");
+    CHECK(sum(ones(123, 45)) == 123.0f * 45.0f, "sum of ones");
+    CHECK(max(scalarMul(ones(5, 5), -7.0f)) == -1.0f, "max starts from -1 like the reference");
+    CHECK(max(scalarMul(ones(5, 5), 4.0f)) == 4.0f, "max");
+
+    // softmax: uniform input gives 1/cols; rows sum to 1
+    Matrix *s = to_host(softmax(ones(20, 10)));
+    for (long long i = 0; i < s->size; ++i) CHECK(fabsf(s->data[i] - 0.1f) < 1e-6f, "softmax uniform");
+    s = to_host(softmax(gpu.randn(64, 10)));
+    for (int r = 0; r < 64; ++r) {
+        float acc = 0;
+        for (int c = 0; c < 10; ++c) acc += s->data[r * 10 + c];
+        CHECK(fabsf(acc - 1.0f) < 1e-5f, "softmax rows sum to one");
+    }
+
+    // bias broadcast
+    Matrix *A = gpu.rand(9, 6);
+    Matrix *v = gpu.rand(1, 6);
+    Matrix *av = to_host(addMatrixVector(A, v));
+    Matrix *ah = to_host(A), *vh = to_host(v);
+    for (int r = 0; r < 9; ++r)
+        for (int c = 0; c < 6; ++c) CHECK(av->data[r * 6 + c] == ah->data[r * 6 + c] + vh->data[c], "addMatrixVector");
+
+    // maxout against the reference's brute-force expectation (tests/basicOps_test.cu:580-610)
+    m1 = gpu.rand(128, 1736);
+    int maxout_level = 8;
+    Matrix **mo = maxout(m1, maxout_level);
+    Matrix *m2 = to_host(mo[0]), *m3 = to_host(mo[1]);
+    CHECK(test_matrix(m2, 128, 1736 / 8) && test_matrix(m3, 128, 1736 / 8), "maxout shapes");
+    h = to_host(m1);
+    for (int row = 0; row < h->rows; ++row) {
+        float max_value = -2.0f, max_col_value = 0.0f;
+        for (int col = 0; col < h->cols; ++col) {
+            if (h->data[row * h->cols + col] > max_value) {
+                max_value = h->data[row * h->cols + col];
+                max_col_value = (float)col;
+            }
+            if ((col + 1) % maxout_level == 0) {
+                int o_idx = row * (h->cols / maxout_level) + col / maxout_level;
+                if (m2->data[o_idx] != max_value || m3->data[o_idx] != max_col_value) {
+                    CHECK(false, "maxout value / index");
+                    row = h->rows;
+                    break;
+                }
+                max_value = -2.0f;
+            }
+        }
+    }
+
+    // expand_to_maxout_grad (tests/basicOps_test.cu:612-638)
+    Matrix *grad = gpu.rand(2, 8), *error = gpu.rand(2, 4);
+    m1 = gpu.rand(2, 8);
+    mo = maxout(m1, 2);
+    expand_to_maxout_grad(error, mo[1], grad);
+    Matrix *gh = to_host(grad), *ih = to_host(mo[1]), *eh = to_host(error);
+    for (int row = 0; row < 2; ++row) {
+        int block = 0;
+        for (int col = 0; col < 8; ++col) {
+            float value = gh->data[row * 8 + col];
+            if (value != 0.0f) {
+                CHECK((int)ih->data[row * 4 + block] == col, "expand maxout: index");
+                CHECK(eh->data[row * 4 + block] == value, "expand maxout: value");
+                ++block;
+            }
+        }
+        CHECK(block == 4, "expand maxout: one non-zero per pool");
+    }
+
+    // shape-check helpers
+    CHECK(blnFaultySizes(ones(2, 3), ones(2, 3), ones(2, 3)) == 0, "blnFaultySizes ok");
+    CHECK(blnFaultySizes(ones(2, 3), ones(3, 2), ones(2, 3)) == 1, "blnFaultySizes bad");
+    CHECK(blnFaultyMatrixProductSizes(ones(2, 3), ones(3, 5), ones(2, 5), OP_N, OP_N) == 0, "product sizes ok");
+    CHECK(blnFaultyMatrixProductSizes(ones(3, 2), ones(3, 5), ones(2, 5), OP_T, OP_N) == 0, "product sizes T ok");
+    CHECK(blnFaultyMatrixProductSizes(ones(2, 3), ones(5, 3), ones(2, 5), OP_N, OP_T) == 0, "product sizes NT ok");
+    CHECK(blnFaultyMatrixProductSizes(ones(2, 3), ones(4, 5), ones(2, 5), OP_N, OP_N) == 1, "product sizes bad");
+}
+
+int main() {
+    try {
+        ClusterNet gpus = ClusterNet(132456);
+        run_basicOps_test(gpus);
+        run_clusterNet_test(gpus);
+        run_codec_test(gpus);
+    } catch (const char *e) {
+        printf("uncaught error: %s\n", e);
+        return 2;
+    }
+    if (failures) {
+        printf("%d FACADE TEST(S) FAILED\n", failures);
+        return 1;
+    }
+    printf("ALL FACADE TESTS PASSED\n");
+    return 0;
+}

@@ -1,0 +1,152 @@
+"""The small kernels around the path and one maxout training step composed from the path's
+operators, compared with the CPU checker."""
+import numpy as np
+import pytest
+
+import oracle
+from util import gemm_tolerance
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    import clusternet_amd as cn
+    cn.init(0)
+    return torch.device("cuda:0")
+
+
+def _t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def test_helpers_match_checker(dev):
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(0)
+    A = rng.normal(0, 1, (133, 1736)).astype(np.float32)
+    v = rng.normal(0, 1, 1736).astype(np.float32)
+    assert np.array_equal(L.add_row_vector(_t(A, dev), _t(v, dev)).cpu().numpy(), oracle.add_row_vector(A, v))
+    assert np.array_equal(L.transpose(_t(A, dev)).cpu().numpy(), A.T)
+    for pool in (2, 4, 8):
+        out, arg = L.maxout(_t(A, dev), pool)
+        wo, wa = oracle.maxout(A, pool)
+        assert np.array_equal(out.cpu().numpy(), wo) and np.array_equal(arg.cpu().numpy(), wa)
+        err = rng.normal(0, 1, wo.shape).astype(np.float32)
+        g = L.expand_to_maxout_grad(_t(err, dev), arg, pool).cpu().numpy()
+        assert np.array_equal(g, oracle.expand_to_maxout_grad(err, wa, pool))
+    s = L.softmax(_t(A[:, :10].copy(), dev)).cpu().numpy()
+    np.testing.assert_allclose(s, oracle.softmax(A[:, :10].copy()), rtol=2e-6, atol=1e-9)
+    assert np.allclose(L.softmax(_t(np.zeros((7, 10), np.float32), dev)).cpu().numpy(), 0.1)
+    B = rng.normal(0, 1, A.shape).astype(np.float32)
+    assert np.array_equal(L.sub(_t(A, dev), _t(B, dev)).cpu().numpy(), A - B)
+    w = _t(A, dev)
+    L.sgd_update(w, _t(B, dev), 0.125)
+    assert np.array_equal(w.cpu().numpy(), A - np.float32(0.125) * B)
+    assert abs(float(L.reduce_sum(_t(A, dev)).cpu()[0]) - A.astype(np.float64).sum()) < 1e-2
+    assert float(L.reduce_max(_t(A, dev)).cpu()[0]) == A.max()
+    assert float(L.reduce_max(_t(-np.abs(A) - 2, dev)).cpu()[0]) == -1.0
+    # ties in maxout: the first maximum wins
+    T = np.array([[1, 1, 0, 2, 2, 2]], np.float32)
+    out, arg = L.maxout(_t(T, dev), 3)
+    assert arg.cpu().numpy().tolist() == [[0.0, 3.0]]
+
+
+def _cpu_step(X, onehot, params, rate, pool):
+    W1, b1, W2, b2, W3, b3 = params
+    z1 = oracle.add_row_vector(oracle.gemm(X, W1), b1)
+    h1, a1 = oracle.maxout(z1, pool)
+    z2 = oracle.add_row_vector(oracle.gemm(h1, W2), b2)
+    h2, a2 = oracle.maxout(z2, pool)
+    p = oracle.softmax(oracle.add_row_vector(oracle.gemm(h2, W3), b3))
+    e3 = p - onehot
+    g3 = oracle.gemm(h2, e3, ta=True)
+    e2 = oracle.expand_to_maxout_grad(oracle.gemm(e3, W3, tb=True), a2, pool)
+    g2 = oracle.gemm(h1, e2, ta=True)
+    e1 = oracle.expand_to_maxout_grad(oracle.gemm(e2, W2, tb=True), a1, pool)
+    g1 = oracle.gemm(X, e1, ta=True)
+    return p, (g1, g2, g3), (a1, a2)
+
+
+def test_maxout_training_step_reduced_size(dev):
+    """Same layer structure as the 100000 -> 4096 -> 4096 -> 10 configuration at 1/16 scale."""
+    import torch
+    from clusternet_amd import maxout_step as ms
+    rng = np.random.default_rng(1)
+    B, D, H, O, pool = 128, 6250, 256, 10, 2
+    X = np.where(rng.random((B, D)) < 0.02, rng.random((B, D)), 0).astype(np.float32)
+    lim = lambda i, o: np.sqrt(6.0 / (i + o))
+    W1 = rng.uniform(-lim(D, 2 * H), lim(D, 2 * H), (D, 2 * H)).astype(np.float32)
+    W2 = rng.uniform(-lim(H, 2 * H), lim(H, 2 * H), (H, 2 * H)).astype(np.float32)
+    W3 = rng.uniform(-lim(H, O), lim(H, O), (H, O)).astype(np.float32)
+    b1, b2, b3 = (rng.normal(0, 0.01, n).astype(np.float32) for n in (2 * H, 2 * H, O))
+    y = rng.integers(0, O, B)
+    onehot = np.eye(O, dtype=np.float32)[y]
+    params = (W1, b1, W2, b2, W3, b3)
+    p_ref, g_ref, args_ref = _cpu_step(X, onehot, params, 0.01, pool)
+
+    dparams = tuple(_t(a, dev) for a in params)
+    p, cache = ms.forward(_t(X, dev), dparams, pool)
+    np.testing.assert_allclose(p.cpu().numpy(), p_ref, rtol=2e-4, atol=1e-7)
+    # winners can only differ where two pool members are equal within rounding
+    for a, a_ref in ((cache[1], args_ref[0]), (cache[3], args_ref[1])):
+        assert (a.cpu().numpy() != a_ref).mean() < 1e-3
+    grads = ms.backward(_t(X, dev), _t(onehot, dev), dparams, p, cache, pool)
+    for g, gr, K in zip(grads, g_ref, (B, B, B)):
+        err = np.abs(g.cpu().numpy() - gr).max() / np.abs(gr).max()
+        assert err < 2e-3, err  # a flipped winner moves one error entry to the neighbouring column
+    # gradient codec round trip on the device equals the checker's on the same gradient
+    g1 = grads[0].clone()
+    g8, codes, prec = ms.codec_round_trip(g1)
+    g_host = grads[0].cpu().numpy()
+    prec_h = oracle.absmax(g_host)
+    assert float(prec.cpu()[0]) == prec_h
+    want_codes = oracle.port_compress(g_host, prec_h)
+    assert np.array_equal(codes.cpu().numpy(), want_codes)
+    assert np.array_equal(g8.cpu().numpy().view(np.uint32), oracle.port_decompress(want_codes, prec_h).view(np.uint32))
+    # the full step runs and moves the weights by rate * decoded gradient
+    before = dparams[4].clone()
+    ms.step(_t(X, dev), _t(onehot, dev), dparams, 0.01, pool)
+    assert float((dparams[4] - before).abs().max()) > 0
+
+
+def test_maxout_training_step_full_size_properties(dev):
+    """100000 -> 4096 -> 4096 -> 10 with pool 2 at batch 128: shapes, probabilities, the sparsity
+    pattern of the expanded gradients, and sampled entries of the 100000 x 8192 weight gradient
+    recomputed on the CPU."""
+    import torch
+    from clusternet_amd import maxout_step as ms
+    g = torch.Generator(device=dev).manual_seed(3)
+    B, D, H, O, pool = 128, 100000, 4096, 10, 2
+    X = torch.rand((B, D), device=dev, generator=g)
+    X = torch.where(torch.rand((B, D), device=dev, generator=g) < 0.02, X, torch.zeros_like(X))
+    u = lambda r, c: (torch.rand((r, c), device=dev, generator=g) * 2 - 1) * float(np.sqrt(6.0 / (r + c)))
+    params = (u(D, 2 * H), torch.zeros(2 * H, device=dev), u(H, 2 * H), torch.zeros(2 * H, device=dev),
+              u(H, O), torch.zeros(O, device=dev))
+    y = torch.randint(0, O, (B,), device=dev, generator=g)
+    onehot = torch.nn.functional.one_hot(y, O).float()
+    p, cache = ms.forward(X, params, pool)
+    assert tuple(p.shape) == (B, O)
+    assert float((p.sum(dim=1) - 1).abs().max()) < 1e-5 and float(p.min()) >= 0
+    grads = ms.backward(X, onehot, params, p, cache, pool)
+    assert [tuple(t.shape) for t in grads] == [(D, 2 * H), (H, 2 * H), (H, O)]
+    # sampled columns of gW1 = X^T e1: recompute e1 on the device path, the product on the CPU
+    e3 = p - onehot
+    e2 = ms.L.expand_to_maxout_grad(ms.L.dotT(e3, params[4]), cache[3], pool)
+    e1 = ms.L.expand_to_maxout_grad(ms.L.dotT(e2, params[2]), cache[1], pool)
+    assert float((e1 != 0).float().mean()) <= 0.5 + 1e-6  # one winner per pool of two
+    cols = np.array([0, 1, 4095, 8191, 777, 5000])
+    Cref, Cabs = oracle.gemm_cols(X.cpu().numpy(), e1.cpu().numpy(), cols, ta=True)
+    got = grads[0][:, torch.from_numpy(cols).to(dev)].cpu().numpy().astype(np.float64)
+    assert (np.abs(got - Cref) / np.maximum(Cabs, 1e-300)).max() <= gemm_tolerance(B)
+    # 8-bit round trip of the 3.28 GB gradient: decoded values stay within the codebook's step
+    g1 = grads[0]
+    prec = ms.L.absmax(g1)
+    codes = ms.L.compression_8bit(g1, prec)
+    dec = ms.L.decompression_8bit(codes, prec)
+    pv = float(prec.cpu()[0])
+    keep = codes != 254
+    rel = ((dec - g1).abs() / pv)[keep]
+    assert float(rel.max()) <= 0.0172 + 1e-6
+    assert torch.equal(torch.sign(dec[keep]), torch.sign(g1[keep]))
