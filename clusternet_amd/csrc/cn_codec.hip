@@ -96,14 +96,16 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
         const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
         uint32_t *c4 = reinterpret_cast<uint32_t *>(codes);
         const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
-        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        auto load_tile = [&](size_t tile, f32x4 (&v)[kVecPerThread]) {
             const size_t base = tile * kTileVec + threadIdx.x;
-            f32x4 v[kVecPerThread];
 #pragma unroll
             for (int j = 0; j < kVecPerThread; ++j) {
                 size_t i = base + (size_t)j * kThreads;
                 v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
+        };
+        auto encode_tile = [&](size_t tile, const f32x4 (&v)[kVecPerThread]) {
+            const size_t base = tile * kTileVec + threadIdx.x;
             uint32_t packed[kVecPerThread];
             uint32_t near = 0, magmax = 0;
 #pragma unroll
@@ -128,6 +130,23 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
             for (int j = 0; j < kVecPerThread; ++j) {
                 size_t i = base + (size_t)j * kThreads;
                 if (i < nvec) __builtin_nontemporal_store(packed[j], &c4[i]);
+            }
+        };
+        // Two register sets: the loads of the next tile are in flight while this one is encoded,
+        // so the memory pipe stays busy even with only two wavefronts per SIMD.
+        f32x4 va[kVecPerThread], vb[kVecPerThread];
+        size_t t0 = blockIdx.x;
+        if (t0 < tiles) {
+            load_tile(t0, va);
+            for (;;) {
+                const size_t t1 = t0 + gridDim.x;
+                if (t1 < tiles) load_tile(t1, vb);
+                encode_tile(t0, va);
+                if (t1 >= tiles) break;
+                t0 = t1 + gridDim.x;
+                if (t0 < tiles) load_tile(t0, va);
+                encode_tile(t1, vb);
+                if (t0 >= tiles) break;
             }
         }
         // ragged tail (n % 4 elements)
@@ -319,7 +338,9 @@ static cn_status compress_impl(const float *x, float precision, const float *pre
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
-    int grid = stream_grid(ctx, n, 6);
+    // two workgroups per CU: mixed read/write streams run fastest on this part with few wavefronts
+    // in flight, and the kernel keeps its own next tile in flight to stay busy at that occupancy
+    int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16) && aligned(codes, 4))
         hipLaunchKernelGGL(compress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, precision,
                            precision_dev, n, codes, ctx->encode_lut, ctx->lut_first, ctx->lut_count, ctx->table);
@@ -388,7 +409,7 @@ cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
         return CN_OK;
     }
     if (!x) { set_error("absmax_f32: NULL input"); return CN_ERR_NULL; }
-    int grid = stream_grid(ctx, n, 8);
+    int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16))
         hipLaunchKernelGGL((absmax_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
     else
@@ -409,7 +430,7 @@ cn_status cn_max_f32(const float *x, size_t n, float *out, void *stream) {
         return CN_OK;
     }
     if (!x) { set_error("max_f32: NULL input"); return CN_ERR_NULL; }
-    int grid = stream_grid(ctx, n, 8);
+    int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16))
         hipLaunchKernelGGL((absmax_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
     else

@@ -1,30 +1,32 @@
-// fp32 GEMM for gfx950 on the matrix cores: C = op(A) op(B), row-major, alpha 1, beta 0.
+// fp32 GEMM for gfx950 on the matrix cores: C = op(A) op(B), row-major, alpha 1, beta 0, and the
+// fused variant whose B operand is 8-bit codes.
 //
-// Common structure of the kernels in this file:
+// One kernel template, gemm_kernel<A_KC, B_KIND>:
 //   * workgroup = 256 lanes = 4 wavefronts in a 2 x 2 arrangement, output tile 128 x 128, every
 //     wavefront owns 64 x 64 = 2 x 2 blocks of v_mfma_f32_32x32x2_f32 (64 accumulators per lane)
 //   * K advances 32 at a time through two LDS stages with one barrier per stage; the global loads
 //     of stage i + 1 are issued before the MFMAs of stage i
+//   * fp32 tiles go from global memory straight into LDS with buffer_load_dwordx4 ... lds, 1 KiB
+//     per wavefront instruction: no staging registers, no LDS store instructions.  An operand
+//     whose memory is contiguous along k (A of dot/dotT, B of dotT) sits in LDS as [index][k], its
+//     16-byte columns XOR-swizzled by the row (applied on the global-address side), and feeds four
+//     MFMAs per 16-byte LDS read; an operand contiguous along its row/column index (A of Tdot, B
+//     of dot/Tdot) sits as [k][index] and is read one value per MFMA with conflict-free 4-byte
+//     LDS reads
+//   * rows or columns of a ragged tile that lie outside the matrix are loaded like any other: they
+//     only ever feed outputs outside the matrix, which are not stored, and the buffer descriptor's
+//     range check turns addresses past the end of the matrix into zeros instead of memory accesses
+//   * 8-bit codes of the fused variant are read in coalesced 4-byte words along n, expanded through
+//     a 256-entry LDS table (the decode table of the stand-alone decompression kernel, bit for bit)
+//     and stored as fp32 into the same [k][n] LDS image, so the MFMA side does not change
+//   * the last, partial K stage and operands that do not allow 16-byte loads take a predicated
+//     register path (zero-filled) into the same LDS images
 //   * K may be split into chunks (one workgroup per chunk and tile); chunk results go to a
 //     workspace and a second kernel adds them in a fixed order
 //   * block ids are remapped so that the workgroups an XCD receives (ids congruent mod 8) cover a
 //     contiguous range of work units and share their A/B panels in that XCD's L2
 //   * global addresses are a uniform buffer descriptor (scalar registers) plus a 32-bit per-lane
 //     byte offset, which is why leading dimensions are limited to 2^22 elements.
-//
-// gemm_dl_kernel (dot, Tdot, dotT): tiles go from global memory straight into LDS with
-// buffer_load_dwordx4 ... lds, 1 KiB per wavefront instruction, no staging registers and no LDS
-// store instructions.  An operand whose memory is contiguous along k sits in LDS as [index][k]
-// (16-byte columns XOR-swizzled by the row, applied on the global-address side) and feeds four
-// MFMAs per 16-byte LDS read; an operand contiguous along its row/column index sits as
-// [k][index] and is read one value per MFMA with conflict-free 4-byte LDS reads.  Ragged edge
-// tiles and unaligned operands take a predicated register path into the same LDS layout.
-//
-// gemm_kernel (fused 8-bit weights, and the register-staged fallback): global -> registers ->
-// LDS; the index-contiguous operand is transposed 4 x 4 in registers on its way in, and 8-bit
-// codes are expanded through a 256-entry LDS table at that point.
-#include <stdlib.h>
-
 #include "cn_internal.h"
 
 namespace cn {
@@ -34,13 +36,10 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
-// Buffer descriptor with its origin at `p`, no stride, no range check (every access is either
-// known to be in range or individually predicated).  0x00020000 = 32-bit untyped data format.
+// Buffer descriptor with its origin at `p`, no stride, no range check (for accesses that are
+// individually predicated).  0x00020000 = 32-bit untyped data format.
 __device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0xffffffff, 0x00020000);
-}
-__device__ __forceinline__ f32x4 as_f32x4(u32x4 v) {
-    return f32x4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
 }
 
 constexpr int BM = kTileM, BN = kTileN, BK = kTileK;
@@ -48,8 +47,8 @@ constexpr int kGemmThreads = 256;
 constexpr int kStageFloats = 128 * BK;  // one operand, one stage
 constexpr int kNumXcd = 8;
 
-// How the B operand reaches the MFMAs.
-enum BMode { B_IC_LDS = 0, B_KC_LDS = 1, B_CODES_LDS = 2 };
+// What the B operand is.
+enum BKind { B_IC = 0 /* fp32 [k][n] */, B_KC = 1 /* fp32 [n][k] */, B_CODES = 2 /* uint8 [k][n] */ };
 
 struct GemmArgs {
     const float *A;
@@ -65,77 +64,133 @@ struct GemmArgs {
     const float *table;  // fused: 126-entry codebook
 };
 
+// LDS image of one operand tile (128 index values x 32 k, 16 KiB):
+//   KC (memory [index][k]): float offset lds_offset(index, k / 4) + k % 4   (swizzled 16-byte columns)
+//   IC (memory [k][index]): float offset k * 128 + index
 __device__ __forceinline__ int swizzle_of(int row) { return (row & 7) ^ ((row >> 3) & 3); }
 __device__ __forceinline__ int lds_offset(int row, int quad) {
     return row * BK + ((quad ^ swizzle_of(row)) << 2);
 }
 
-// ---- operand staged through LDS -------------------------------------------------------------------
-// Per-lane constants of one operand tile (128 index values x 32 k), computed once per workgroup.
-//   KC (memory [index][k]): load j covers k quad (t & 7) of index (t >> 3) + 32 j.
-//   IC (memory [k][index]): load r covers indices 4 (t & 31) .. +3 of k row 4 (t >> 5) + r.
-// `elem` is sizeof element in the global array (4, or 1 for codes).
+// ---- direct global -> LDS loads ------------------------------------------------------------------
+// A wavefront fills a tile 1 KiB at a time: block b = 4 j + wave (j = 0..3) is rows 8 b .. 8 b + 7 of
+// a KC tile or k rows 2 b, 2 b + 1 of an IC tile, lane l supplying bytes 16 l .. 16 l + 15 of the block.
 template <bool KC>
-struct TileLoader {
-    uint32_t off[4];     // byte offset of each of the four loads from the tile's (index0, k0) corner
-    uint32_t ok;         // KC: bit j = index of load j is in range;  IC: bit e = index 4 cq + e in range
-    int kfirst;          // KC: first k of the lane's quad;  IC: first k row of the lane
-    __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices, int elem) {
-        const int t = threadIdx.x;
-        ok = 0;
-        if (KC) {
-            const int kq = t & 7, rb = t >> 3;
-            kfirst = 4 * kq;
+struct DirectLoader {
+    uint32_t off[4];  // byte offset of this lane's 16 bytes of block 4 j + wave from the tile corner
+    __device__ __forceinline__ void init(int64_t ld, int wave) {
+        const int lane = threadIdx.x & 63;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                off[j] = (uint32_t)(((rb + 32 * j) * ld + 4 * kq) * elem);
-                if (index0 + rb + 32 * j < indices) ok |= 1u << j;
-            }
-        } else {
-            const int cq = t & 31, kq = t >> 5;
-            kfirst = 4 * kq;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) off[r] = (uint32_t)(((4 * kq + r) * ld + 4 * cq) * elem);
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (index0 + 4 * cq + e < indices) ok |= 1u << e;
-        }
-    }
-    // base = buffer descriptor whose origin is the tile corner (index0, k0); kleft = K - k0.
-    __device__ __forceinline__ void load(rsrc_t base, int64_t kleft, bool fast, f32x4 (&reg)[4]) const {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            if (fast) {
-                reg[i] = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(base, off[i], 0, 0));
+        for (int j = 0; j < 4; ++j) {
+            const int blk = 4 * j + wave;
+            if (KC) {
+                const int row = 8 * blk + (lane >> 3);
+                const int quad = (lane & 7) ^ swizzle_of(row);
+                off[j] = (uint32_t)((row * ld + 4 * quad) * 4);
             } else {
-                f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (KC) {
-                    if (ok & (1u << i)) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (kfirst + e < kleft)
-                                v[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(base, off[i] + 4 * e, 0, 0));
-                    }
-                } else {
-                    if (kfirst + i < kleft) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (ok & (1u << e))
-                                v[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(base, off[i] + 4 * e, 0, 0));
-                    }
-                }
-                reg[i] = v;
+                const int k = 2 * blk + (lane >> 5);
+                off[j] = (uint32_t)((k * ld + 4 * (lane & 31)) * 4);
             }
         }
     }
-    __device__ __forceinline__ void load_codes(rsrc_t base, int64_t kleft, bool fast, uint32_t (&reg)[4]) const {
+    // The loads are written as inline assembly on purpose: the compiler's wait-count insertion
+    // treats every LDS read that follows a compiler-visible LDS-writing load as dependent on it and
+    // would wait for the whole next stage before the first MFMA of the current one.  Completion is
+    // awaited explicitly (vmcnt(0)) before the barrier that publishes the stage.
+    // `limit` = bytes from the corner to the end of the matrix: the descriptor's range check makes
+    // every access at or beyond it return zero instead of touching memory.
+    __device__ __forceinline__ void issue(const void *corner, uint32_t limit, float *lds_stage, int wave) const {
+        const uint64_t addr = reinterpret_cast<uint64_t>(corner);
+        const u32x4 rsrc = {(uint32_t)addr, (uint32_t)(addr >> 32) & 0xffffu, limit, 0x00020000u};
+        const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(
+            (__attribute__((address_space(3))) float *)lds_stage) + (uint32_t)wave * 1024u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                         :
+                         : "s"(lds0 + (uint32_t)j * 4096u), "v"(off[j]), "s"(rsrc)
+                         : "memory", "m0");
+    }
+};
+
+// ---- predicated register paths (partial K stage, unaligned operands) ---------------------------------
+// KC operand: lane t covers k quad (t & 7) of rows (t >> 3) + 32 j, j = 0..3.
+struct GuardedKC {
+    uint32_t off[4];
+    uint32_t ok;  // bit j: row of load j is inside the matrix
+    int kfirst;
+    __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices) {
+        const int kq = threadIdx.x & 7, rb = threadIdx.x >> 3;
+        kfirst = 4 * kq;
+        ok = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            off[j] = (uint32_t)(((rb + 32 * j) * ld + 4 * kq) * 4);
+            if (index0 + rb + 32 * j < indices) ok |= 1u << j;
+        }
+    }
+    __device__ __forceinline__ void load(rsrc_t base, int64_t kleft, f32x4 (&reg)[4]) const {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (ok & (1u << j)) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (kfirst + e < kleft)
+                        v[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(base, off[j] + 4 * e, 0, 0));
+            }
+            reg[j] = v;
+        }
+    }
+    __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
+        const int kq = threadIdx.x & 7, rb = threadIdx.x >> 3;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<f32x4 *>(lds + lds_offset(rb + 32 * j, kq)) = reg[j];
+    }
+};
+
+// IC operand, fp32 or codes: lane t covers indices 4 (t & 31) .. +3 of k rows (t >> 5) + 8 r, r = 0..3.
+struct GuardedIC {
+    uint32_t off[4];  // byte offsets for an element size of `elem`
+    uint32_t ok;      // bit e: index 4 cq + e is inside the matrix
+    __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices, int elem) {
+        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
+        ok = 0;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) off[r] = (uint32_t)(((kr + 8 * r) * ld + 4 * cq) * elem);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (index0 + 4 * cq + e < indices) ok |= 1u << e;
+    }
+    __device__ __forceinline__ void load(rsrc_t base, int64_t kleft, f32x4 (&reg)[4]) const {
+        const int kr = threadIdx.x >> 5;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            if (fast) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (kr + 8 * r < kleft) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (ok & (1u << e))
+                        v[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(base, off[r] + 4 * e, 0, 0));
+            }
+            reg[r] = v;
+        }
+    }
+    __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
+        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) *reinterpret_cast<f32x4 *>(lds + (kr + 8 * r) * 128 + 4 * cq) = reg[r];
+    }
+    // Codes: four per 32-bit word.  `whole` = aligned words inside the matrix and inside K.
+    __device__ __forceinline__ void load_codes(rsrc_t base, int64_t kleft, bool whole, uint32_t (&reg)[4]) const {
+        const int kr = threadIdx.x >> 5;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            if (whole) {
                 reg[r] = __builtin_amdgcn_raw_buffer_load_b32(base, off[r], 0, 0);
             } else {
                 uint32_t w = 0;
-                if (kfirst + r < kleft) {
+                if (kr + 8 * r < kleft) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (ok & (1u << e))
@@ -145,51 +200,30 @@ struct TileLoader {
             }
         }
     }
-    __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
-        const int t = threadIdx.x;
-        if (KC) {
-            const int kq = t & 7, rb = t >> 3;
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                *reinterpret_cast<f32x4 *>(lds + lds_offset(rb + 32 * j, kq)) = reg[j];
-        } else {
-            const int cq = t & 31, kq = t >> 5;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                f32x4 v = {reg[0][e], reg[1][e], reg[2][e], reg[3][e]};
-                *reinterpret_cast<f32x4 *>(lds + lds_offset(4 * cq + e, kq)) = v;
-            }
-        }
-    }
-    // Decode four code words through the 256-entry table and store transposed.  Positions outside
-    // the matrix must contribute exactly zero, whatever code 0 decodes to.
+    // Expand through the decode table.  Rows at or beyond K must contribute exactly zero whatever
+    // code 0 decodes to; columns beyond N only reach outputs that are not stored.
     __device__ __forceinline__ void store_codes(float *__restrict__ lds, const float *__restrict__ lut,
-                                                const uint32_t (&reg)[4], int64_t kleft, bool fast) const {
-        const int t = threadIdx.x;
-        const int cq = t & 31, kq = t >> 5;
+                                                const uint32_t (&reg)[4], int64_t kleft) const {
+        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
+        for (int r = 0; r < 4; ++r) {
             f32x4 v;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float d = lut[(reg[r] >> (8 * e)) & 0xffu];
-                if (!fast && !((ok & (1u << e)) && kfirst + r < kleft)) d = 0.0f;
-                v[r] = d;
-            }
-            *reinterpret_cast<f32x4 *>(lds + lds_offset(4 * cq + e, kq)) = v;
+            for (int e = 0; e < 4; ++e) v[e] = lut[(reg[r] >> (8 * e)) & 0xffu];
+            if (kr + 8 * r >= kleft) v = f32x4{0.f, 0.f, 0.f, 0.f};
+            *reinterpret_cast<f32x4 *>(lds + (kr + 8 * r) * 128 + 4 * cq) = v;
         }
     }
 };
 
-template <bool A_KC, int B_MODE>
+template <bool A_KC, int B_KIND>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
-    constexpr bool kCodes = (B_MODE == B_CODES_LDS);
-    constexpr int WM = 2, WN = 2;
-
+    constexpr bool B_IS_KC = (B_KIND == B_KC);
+    constexpr bool kCodes = (B_KIND == B_CODES);
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *sA = smem;                                           // [2][kStageFloats]
-    float *sB = smem + 2 * kStageFloats;                        // [2][kStageFloats]
-    float *sLut = smem + 4 * kStageFloats;                      // [256], fused only
+    float *sA = smem;                       // [2][kStageFloats]
+    float *sB = smem + 2 * kStageFloats;    // [2][kStageFloats]
+    float *sLut = smem + 4 * kStageFloats;  // [256], fused only
 
     // Work unit of this workgroup.  Hardware hands consecutive block ids to the XCDs round-robin;
     // give XCD x the x-th contiguous slice of the unit range.
@@ -197,9 +231,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
     const uint32_t xcd = bid % kNumXcd, idx = bid / kNumXcd;
     const uint32_t per = U / kNumXcd, rem = U % kNumXcd;
     const uint32_t unit = xcd * per + (xcd < rem ? xcd : rem) + idx;
-
     // 32-bit unit arithmetic, then pinned to scalar registers: everything derived from these
-    // (tile corners, buffer descriptors) must stay wave-uniform for the buffer loads below.
+    // (tile corners, buffer descriptors) must stay wave-uniform.
     const uint32_t tiles32 = (uint32_t)g.tiles, tiles_n32 = (uint32_t)g.tiles_n;
     const uint32_t split_v = unit / tiles32, tile_v = unit - split_v * tiles32;
     const uint32_t tm_v = tile_v / tiles_n32, tn_v = tile_v - tm_v * tiles_n32;
@@ -227,212 +260,6 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
         __syncthreads();
     }
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wave_m = wave >> 1, wave_n = wave & 1;
-    const int half = lane >> 5, l32 = lane & 31;
-    int row_a[WM], row_b[WN];
-#pragma unroll
-    for (int i = 0; i < WM; ++i) row_a[i] = wave_m * (32 * WM) + i * 32 + l32;
-#pragma unroll
-    for (int i = 0; i < WN; ++i) row_b[i] = wave_n * (32 * WN) + i * 32 + l32;
-
-    f32x16 acc[WM][WN];
-#pragma unroll
-    for (int mi = 0; mi < WM; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < WN; ++ni)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
-
-    const bool inner_m = (m0 + BM <= g.M), inner_n = (n0 + BN <= g.N);
-    const uint8_t *Wc = reinterpret_cast<const uint8_t *>(g.B);
-    const float *Bf = reinterpret_cast<const float *>(g.B);
-
-    TileLoader<A_KC> la;
-    la.init(g.lda, m0, g.M, 4);
-    TileLoader<B_MODE == B_KC_LDS> lb;
-    lb.init(g.ldb, n0, g.N, kCodes ? 1 : 4);
-
-    // Corner addresses of stage `it` (uniform across the workgroup).
-    auto corner_a = [&](int it) { return A_KC ? g.A + m0 * g.lda + (int64_t)it * BK : g.A + (int64_t)it * BK * g.lda + m0; };
-    auto corner_b = [&](int it) {
-        return (B_MODE == B_KC_LDS) ? Bf + n0 * g.ldb + (int64_t)it * BK : Bf + (int64_t)it * BK * g.ldb + n0;
-    };
-
-    f32x4 ra[4], rb[4];
-    uint32_t rc[4];
-
-    auto fetch = [&](int it) {
-        const int64_t kleft = g.K - (int64_t)it * BK;
-        const bool inner_k = kleft >= BK;
-        la.load(make_rsrc(corner_a(it)), kleft, g.vec_a && inner_m && inner_k, ra);
-        if (kCodes) lb.load_codes(make_rsrc(Wc + (int64_t)it * BK * g.ldb + n0), kleft, g.vec_b && inner_n && inner_k, rc);
-        else             lb.load(make_rsrc(corner_b(it)), kleft, g.vec_b && inner_n && inner_k, rb);
-    };
-    // Registers -> LDS stage `buf`.
-    auto stash = [&](int it, int buf) {
-        const int64_t kleft = g.K - (int64_t)it * BK;
-        la.store(sA + buf * kStageFloats, ra);
-        if (kCodes) lb.store_codes(sB + buf * kStageFloats, sLut, rc, kleft, g.vec_b && inner_n && kleft >= BK);
-        else        lb.store(sB + buf * kStageFloats, rb);
-    };
-    // One K stage of MFMAs.  Within each group of 8 k values, MFMA s (0..3) consumes
-    // k = 8 g + 4 h + s from lane half h on both operands, i.e. the k order inside a stage is
-    // permuted identically for A and B.
-    auto compute = [&](int buf) {
-        const float *pa = sA + buf * kStageFloats, *pb = sB + buf * kStageFloats;
-#pragma unroll
-        for (int gq = 0; gq < BK / 8; ++gq) {
-            f32x4 a[WM], b[WN];
-#pragma unroll
-            for (int i = 0; i < WM; ++i)
-                a[i] = *reinterpret_cast<const f32x4 *>(pa + lds_offset(row_a[i], 2 * gq + half));
-#pragma unroll
-            for (int i = 0; i < WN; ++i)
-                b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset(row_b[i], 2 * gq + half));
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int mi = 0; mi < WM; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < WN; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi][s], b[ni][s], acc[mi][ni], 0, 0, 0);
-        }
-    };
-
-    if (it0 < it1) {
-        fetch(it0);
-        stash(it0, 0);
-        __syncthreads();
-        int buf = 0;
-        for (int it = it0; it < it1; ++it) {
-            const bool more = (it + 1 < it1);
-            if (more) fetch(it + 1);   // global loads fly while this stage's MFMAs run
-            compute(buf);
-            if (more) stash(it + 1, buf ^ 1);
-            __syncthreads();
-            buf ^= 1;
-        }
-    }
-
-    // Write-out.  Accumulator r of a lane holds row 8 (r / 4) + 4 half + (r % 4), column l32 of its
-    // 32 x 32 block: for a fixed r the 32 lanes of a half write 128 contiguous bytes.
-    float *dst;
-    int64_t ldd;
-    if (g.splits > 1) { dst = g.partial + (int64_t)split * g.M * g.N; ldd = g.N; }
-    else              { dst = g.C; ldd = g.ldc; }
-#pragma unroll
-    for (int mi = 0; mi < WM; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < WN; ++ni) {
-            const int64_t col = n0 + wave_n * (32 * WN) + ni * 32 + l32;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t row = m0 + wave_m * (32 * WM) + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (row < g.M && col < g.N) dst[row * ldd + col] = acc[mi][ni][r];
-            }
-        }
-}
-
-// ---- direct-to-LDS kernel ---------------------------------------------------------------------------
-// LDS image of one operand tile (128 index values x 32 k, 16 KiB), identical whichever way it is
-// filled:
-//   KC (memory [index][k]): float offset lds_offset(index, k / 4) + k % 4   (swizzled 16-byte columns)
-//   IC (memory [k][index]): float offset k * 128 + index
-// A wavefront fills it 1 KiB at a time: block b = 4 j + wave (j = 0..3) is rows 8 b .. 8 b + 7 of a
-// KC tile or k rows 2 b, 2 b + 1 of an IC tile, lane l supplying bytes 16 l .. 16 l + 15 of the block.
-template <bool KC>
-struct DirectLoader {
-    uint32_t off[4];  // byte offset of this lane's 16 bytes of block 4 j + wave from the tile corner
-    __device__ __forceinline__ void init(int64_t ld, int wave) {
-        const int lane = threadIdx.x & 63;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int blk = 4 * j + wave;
-            if (KC) {
-                const int row = 8 * blk + (lane >> 3);
-                const int quad = (lane & 7) ^ swizzle_of(row);
-                off[j] = (uint32_t)((row * ld + 4 * quad) * 4);
-            } else {
-                const int k = 2 * blk + (lane >> 5);
-                off[j] = (uint32_t)((k * ld + 4 * (lane & 31)) * 4);
-            }
-        }
-    }
-    // The loads are written as inline assembly on purpose: the compiler's wait-count insertion
-    // treats every LDS read that follows a compiler-visible LDS-writing load as dependent on it and
-    // would wait for the whole next stage before the first MFMA of the current one.  Completion is
-    // awaited explicitly (vmcnt(0)) before the barrier that publishes the stage.
-    __device__ __forceinline__ void issue(const void *corner, float *lds_stage, int wave) const {
-        const uint64_t addr = reinterpret_cast<uint64_t>(corner);
-        const u32x4 rsrc = {(uint32_t)addr, (uint32_t)(addr >> 32) & 0xffffu, 0xffffffffu, 0x00020000u};
-        const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(
-            (__attribute__((address_space(3))) float *)lds_stage) + (uint32_t)wave * 1024u;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                         :
-                         : "s"(lds0 + (uint32_t)j * 4096u), "v"(off[j]), "s"(rsrc)
-                         : "memory", "m0");
-    }
-};
-
-// Predicated register path for ragged tiles / unaligned operands of an IC operand (the KC operand
-// reuses TileLoader<true>, whose LDS image is the same as DirectLoader<true>'s).  Lane t covers
-// indices 4 (t & 31) .. +3 of k rows (t >> 5) + 8 r, r = 0..3.
-struct RowLoader {
-    uint32_t off[4];
-    uint32_t ok;  // bit e: index 4 cq + e is in range
-    __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices) {
-        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
-        ok = 0;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) off[r] = (uint32_t)(((kr + 8 * r) * ld + 4 * cq) * 4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            if (index0 + 4 * cq + e < indices) ok |= 1u << e;
-    }
-    __device__ __forceinline__ void load(rsrc_t base, int64_t kleft, f32x4 (&reg)[4]) const {
-        const int kr = threadIdx.x >> 5;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (kr + 8 * r < kleft) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (ok & (1u << e)) v[e] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(base, off[r] + 4 * e, 0, 0));
-            }
-            reg[r] = v;
-        }
-    }
-    __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
-        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) *reinterpret_cast<f32x4 *>(lds + (kr + 8 * r) * 128 + 4 * cq) = reg[r];
-    }
-};
-
-template <bool A_KC, bool B_KC>
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_dl_kernel(GemmArgs g) {
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *sA = smem;                     // [2][kStageFloats]
-    float *sB = smem + 2 * kStageFloats;  // [2][kStageFloats]
-
-    const uint32_t bid = blockIdx.x, U = g.units;
-    const uint32_t xcd = bid % kNumXcd, idx = bid / kNumXcd;
-    const uint32_t per = U / kNumXcd, rem = U % kNumXcd;
-    const uint32_t unit = xcd * per + (xcd < rem ? xcd : rem) + idx;
-    const uint32_t tiles32 = (uint32_t)g.tiles, tiles_n32 = (uint32_t)g.tiles_n;
-    const uint32_t split_v = unit / tiles32, tile_v = unit - split_v * tiles32;
-    const uint32_t tm_v = tile_v / tiles_n32, tn_v = tile_v - tm_v * tiles_n32;
-    const int64_t split = __builtin_amdgcn_readfirstlane((int)split_v);
-    const int64_t tm = __builtin_amdgcn_readfirstlane((int)tm_v);
-    const int64_t tn = __builtin_amdgcn_readfirstlane((int)tn_v);
-    const int64_t m0 = tm * BM, n0 = tn * BN;
-    const int it0 = (int)(split * g.iters_per_split);
-    int it1 = it0 + (int)g.iters_per_split;
-    if (it1 > (int)g.k_iters) it1 = (int)g.k_iters;
-
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int wave_m = wave >> 1, wave_n = wave & 1;
@@ -452,26 +279,34 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dl_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
-    // Whole-workgroup decisions: a tile that lies inside the matrix and whose operand allows
-    // 16-byte loads is filled by direct loads, stage by stage, as long as the stage is inside K.
-    const bool direct_a = g.vec_a && (m0 + BM <= g.M);
-    const bool direct_b = g.vec_b && (n0 + BN <= g.N);
+    const float *Bf = reinterpret_cast<const float *>(g.B);
+    const uint8_t *Bc = reinterpret_cast<const uint8_t *>(g.B);
+    // One past the last element that may be read, as an element offset from the matrix base.  An
+    // index-contiguous operand is read in aligned groups of four, hence the round-up.
+    const int64_t end_a = A_KC ? (g.M - 1) * g.lda + g.K : (g.K - 1) * g.lda + ((g.M + 3) & ~(int64_t)3);
+    const int64_t end_b = B_IS_KC ? (g.N - 1) * g.ldb + g.K : (g.K - 1) * g.ldb + ((g.N + 3) & ~(int64_t)3);
 
     DirectLoader<A_KC> da;
-    DirectLoader<B_KC> db;
+    DirectLoader<B_IS_KC> db;
     da.init(g.lda, wave);
-    db.init(g.ldb, wave);
-    TileLoader<true> ga_kc, gb_kc;  // predicated paths
-    RowLoader ga_ic, gb_ic;
-    if (A_KC) ga_kc.init(g.lda, m0, g.M, 4); else ga_ic.init(g.lda, m0, g.M);
-    if (B_KC) gb_kc.init(g.ldb, n0, g.N, 4); else gb_ic.init(g.ldb, n0, g.N);
+    if (!kCodes) db.init(g.ldb, wave);
+    GuardedKC ga_kc, gb_kc;
+    GuardedIC ga_ic, gb_ic;
+    if (A_KC) ga_kc.init(g.lda, m0, g.M); else ga_ic.init(g.lda, m0, g.M, 4);
+    if (B_IS_KC) gb_kc.init(g.ldb, n0, g.N); else gb_ic.init(g.ldb, n0, g.N, kCodes ? 1 : 4);
 
+    // Corner addresses of stage `it` (uniform across the workgroup).
     auto corner_a = [&](int it) { return A_KC ? g.A + m0 * g.lda + (int64_t)it * BK : g.A + (int64_t)it * BK * g.lda + m0; };
-    const float *Bf = reinterpret_cast<const float *>(g.B);
-    auto corner_b = [&](int it) { return B_KC ? Bf + n0 * g.ldb + (int64_t)it * BK : Bf + (int64_t)it * BK * g.ldb + n0; };
+    auto corner_b = [&](int it) { return B_IS_KC ? Bf + n0 * g.ldb + (int64_t)it * BK : Bf + (int64_t)it * BK * g.ldb + n0; };
+    auto corner_c = [&](int it) { return Bc + (int64_t)it * BK * g.ldb + n0; };
+    auto limit_of = [](const float *base, int64_t end, const float *corner) {
+        const int64_t bytes = (end - (corner - base)) * 4;
+        return bytes <= 0 ? 0u : (bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes);
+    };
 
     // One K stage of MFMAs.  Within each group of 8 k values, MFMA s (0..3) consumes
-    // k = 8 g + 4 h + s from lane half h on both operands.
+    // k = 8 g + 4 h + s from lane half h on both operands, i.e. the k order inside a stage is
+    // permuted identically for A and B.
     auto compute = [&](int buf) {
         const float *pa = sA + buf * kStageFloats, *pb = sB + buf * kStageFloats;
 #pragma unroll
@@ -485,7 +320,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dl_kernel(GemmArgs g) {
 #pragma unroll
                     for (int s = 0; s < 4; ++s) a[i][s] = pa[(8 * gq + 4 * half + s) * 128 + row_a[i]];
                 }
-                if (B_KC) {
+                if (B_IS_KC) {
                     b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset(row_b[i], 2 * gq + half));
                 } else {
 #pragma unroll
@@ -502,27 +337,37 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dl_kernel(GemmArgs g) {
         }
     };
 
-    // Stages [it0, it_direct) are filled by direct loads only (tile inside the matrix, operands
-    // 16-byte aligned, stage inside K); the rest, if any, goes through predicated registers.
+    // Stages [it0, it_direct) use the direct loads (operands allow 16-byte / 4-byte accesses and the
+    // stage lies inside K); the rest, if any, goes through predicated registers.
     int it_direct = it0;
-    if (direct_a && direct_b) {
+    if (g.vec_a && g.vec_b) {
         const int full = (int)(g.K / BK);
         it_direct = it1 < full ? it1 : full;
         if (it_direct < it0) it_direct = it0;
     }
 
     if (it0 < it_direct) {
-        da.issue(corner_a(it0), sA, wave);
-        db.issue(corner_b(it0), sB, wave);
+        uint32_t rc[4];
+        const bool whole_n = (n0 + BN <= g.N);
+        da.issue(corner_a(it0), limit_of(g.A, end_a, corner_a(it0)), sA, wave);
+        if (kCodes) {
+            gb_ic.load_codes(make_rsrc(corner_c(it0)), BK, whole_n, rc);
+            gb_ic.store_codes(sB, sLut, rc, BK);
+        } else {
+            db.issue(corner_b(it0), limit_of(Bf, end_b, corner_b(it0)), sB, wave);
+        }
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
         __syncthreads();
         int buf = 0;
         for (int it = it0; it < it_direct; ++it) {
-            if (it + 1 < it_direct) {  // lands in the other stage while this one is consumed
-                da.issue(corner_a(it + 1), sA + (buf ^ 1) * kStageFloats, wave);
-                db.issue(corner_b(it + 1), sB + (buf ^ 1) * kStageFloats, wave);
+            const bool more = (it + 1 < it_direct);
+            if (more) {  // lands in the other stage while this one is consumed
+                da.issue(corner_a(it + 1), limit_of(g.A, end_a, corner_a(it + 1)), sA + (buf ^ 1) * kStageFloats, wave);
+                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(it + 1)), BK, whole_n, rc);
+                else        db.issue(corner_b(it + 1), limit_of(Bf, end_b, corner_b(it + 1)), sB + (buf ^ 1) * kStageFloats, wave);
             }
             compute(buf);
+            if (kCodes && more) gb_ic.store_codes(sB + (buf ^ 1) * kStageFloats, sLut, rc, BK);
             __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
             buf ^= 1;
@@ -533,29 +378,37 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_dl_kernel(GemmArgs g) {
         // Predicated path: global -> registers (zero-filled outside the matrix) -> LDS, stage in
         // flight while the previous one is consumed.  Same LDS images as above.
         f32x4 ra[4], rb[4];
+        uint32_t rc[4];
         auto fetch = [&](int it) {
             const int64_t kleft = g.K - (int64_t)it * BK;
-            if (A_KC) ga_kc.load(make_rsrc(corner_a(it)), kleft, false, ra); else ga_ic.load(make_rsrc(corner_a(it)), kleft, ra);
-            if (B_KC) gb_kc.load(make_rsrc(corner_b(it)), kleft, false, rb); else gb_ic.load(make_rsrc(corner_b(it)), kleft, rb);
+            if (A_KC) ga_kc.load(make_rsrc(corner_a(it)), kleft, ra); else ga_ic.load(make_rsrc(corner_a(it)), kleft, ra);
+            if (kCodes)       gb_ic.load_codes(make_rsrc(corner_c(it)), kleft, false, rc);
+            else if (B_IS_KC) gb_kc.load(make_rsrc(corner_b(it)), kleft, rb);
+            else              gb_ic.load(make_rsrc(corner_b(it)), kleft, rb);
         };
-        auto stash = [&](int buf) {
+        auto stash = [&](int it, int buf) {
+            const int64_t kleft = g.K - (int64_t)it * BK;
             if (A_KC) ga_kc.store(sA + buf * kStageFloats, ra); else ga_ic.store(sA + buf * kStageFloats, ra);
-            if (B_KC) gb_kc.store(sB + buf * kStageFloats, rb); else gb_ic.store(sB + buf * kStageFloats, rb);
+            if (kCodes)       gb_ic.store_codes(sB + buf * kStageFloats, sLut, rc, kleft);
+            else if (B_IS_KC) gb_kc.store(sB + buf * kStageFloats, rb);
+            else              gb_ic.store(sB + buf * kStageFloats, rb);
         };
         fetch(it_direct);
-        stash(0);
+        stash(it_direct, 0);
         __syncthreads();
         int buf = 0;
         for (int it = it_direct; it < it1; ++it) {
             const bool more = (it + 1 < it1);
             if (more) fetch(it + 1);
             compute(buf);
-            if (more) stash(buf ^ 1);
+            if (more) stash(it + 1, buf ^ 1);
             __syncthreads();
             buf ^= 1;
         }
     }
 
+    // Write-out.  Accumulator r of a lane holds row 8 (r / 4) + 4 half + (r % 4), column l32 of its
+    // 32 x 32 block: for a fixed r the 32 lanes of a half write 128 contiguous bytes.
     float *dst;
     int64_t ldd;
     if (g.splits > 1) { dst = g.partial + (int64_t)split * g.M * g.N; ldd = g.N; }
@@ -608,24 +461,16 @@ __global__ __launch_bounds__(256) void zero_matrix_kernel(float *__restrict__ C,
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-template <bool A_KC, int B_MODE>
+template <bool A_KC, int B_KIND>
 static cn_status launch(const GemmArgs &args, hipStream_t st) {
-    const size_t lds = (size_t)(4 * kStageFloats + (B_MODE == B_CODES_LDS ? 256 : 0)) * sizeof(float);
+    const size_t lds = (size_t)(4 * kStageFloats + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_MODE>),
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         configured = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<A_KC, B_MODE>), dim3(args.units), dim3(kGemmThreads), lds, st, args);
-    CN_HIP(hipGetLastError());
-    return CN_OK;
-}
-
-template <bool A_KC, bool B_KC>
-static cn_status launch_dl(const GemmArgs &args, hipStream_t st) {
-    const size_t lds = (size_t)(4 * kStageFloats) * sizeof(float);
-    hipLaunchKernelGGL((gemm_dl_kernel<A_KC, B_KC>), dim3(args.units), dim3(kGemmThreads), lds, st, args);
+    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND>), dim3(args.units), dim3(kGemmThreads), lds, st, args);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -674,12 +519,11 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.vec_b = w8 ? (aligned(B, 4) && (ldb % 4 == 0)) : (aligned(B, 16) && (ldb % 4 == 0));
     a.scale = scale; a.table = ctx->table;
 
-    static const bool dl = []() { const char *e = getenv("CNHIP_GEMM_DL"); return !e || atoi(e) != 0; }();
-    if (w8)              s = launch<true, B_CODES_LDS>(a, st);
-    else if (!ta && !tb) s = dl ? launch_dl<true, false>(a, st) : launch<true, B_IC_LDS>(a, st);
-    else if (ta && !tb)  s = dl ? launch_dl<false, false>(a, st) : launch<false, B_IC_LDS>(a, st);
-    else if (!ta && tb)  s = dl ? launch_dl<true, true>(a, st) : launch<true, B_KC_LDS>(a, st);
-    else                 s = dl ? launch_dl<false, true>(a, st) : launch<false, B_KC_LDS>(a, st);
+    if (w8)              s = launch<true, B_CODES>(a, st);
+    else if (!ta && !tb) s = launch<true, B_IC>(a, st);
+    else if (ta && !tb)  s = launch<false, B_IC>(a, st);
+    else if (!ta && tb)  s = launch<true, B_KC>(a, st);
+    else                 s = launch<false, B_KC>(a, st);
     if (s != CN_OK) return s;
 
     if (plan.splits > 1) {
