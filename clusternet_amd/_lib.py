@@ -53,8 +53,10 @@ def lib():
     L.cn_decompress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
     L.cn_host_encode_lut_lookup.argtypes = [C.c_uint32, C.POINTER(C.c_int)]
     L.cn_host_encode_magnitude.argtypes = [f32]
-    L.cn_host_plan_gemm.argtypes = [i64, i64, i64, C.c_int, sz, C.POINTER(i64)]
+    L.cn_host_plan_gemm.argtypes = [i64, i64, i64, C.c_int, sz, C.c_int, C.POINTER(i64)]
     L.cn_host_plan_gemm.restype = None
+    L.cn_host_force_gemm_tile_n.argtypes = [C.c_int]
+    L.cn_host_force_gemm_tile_n.restype = None
     _lib = L
     return L
 

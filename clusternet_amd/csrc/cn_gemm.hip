@@ -1,9 +1,12 @@
 // fp32 GEMM for gfx950 on the matrix cores: C = op(A) op(B), row-major, alpha 1, beta 0, and the
 // fused variant whose B operand is 8-bit codes.
 //
-// One kernel template, gemm_kernel<A_KC, B_KIND>:
-//   * workgroup = 256 lanes = 4 wavefronts in a 2 x 2 arrangement, output tile 128 x 128, every
-//     wavefront owns 64 x 64 = 2 x 2 blocks of v_mfma_f32_32x32x2_f32 (64 accumulators per lane)
+// One kernel template, gemm_kernel<A_KC, B_KIND, TN>:
+//   * output tile 128 x TN; every wavefront owns 64 x 64 = 2 x 2 blocks of v_mfma_f32_32x32x2_f32
+//     (64 accumulators per lane).  TN = 128: 4 wavefronts (2 x 2), two workgroups per compute unit.
+//     TN = 256: 8 wavefronts (2 x 4), one workgroup per compute unit; the A tile is fetched once per
+//     256 output columns, which halves the L2 -> LDS traffic of the A operand.  Measured, the wide
+//     tile is the slower one on every shape tried, so the planner only uses it on request
 //   * K advances 32 at a time through two LDS stages with one barrier per stage; the global loads
 //     of stage i + 1 are issued before the MFMAs of stage i
 //   * fp32 tiles go from global memory straight into LDS with buffer_load_dwordx4 ... lds, 1 KiB
@@ -42,13 +45,19 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0xffffffff, 0x00020000);
 }
 
-constexpr int BM = kTileM, BN = kTileN, BK = kTileK;
-constexpr int kGemmThreads = 256;
-constexpr int kStageFloats = 128 * BK;  // one operand, one stage
+constexpr int BM = kTileM, BK = kTileK;
+constexpr int kAStage = BM * BK;  // floats of one A stage
 constexpr int kNumXcd = 8;
 
 // What the B operand is.
 enum BKind { B_IC = 0 /* fp32 [k][n] */, B_KC = 1 /* fp32 [n][k] */, B_CODES = 2 /* uint8 [k][n] */ };
+
+// LDS stages in flight.  The wide tile has its compute unit to itself, so nothing covers a stage
+// that arrives late; it keeps two stages in flight behind the one being consumed (3 x 48 KiB).  The
+// coded operand passes through registers and stays at two.
+__host__ __device__ constexpr int stages_of(int tile_n, int b_kind) {
+    return (tile_n == 256 && b_kind != B_CODES) ? 3 : 2;
+}
 
 struct GemmArgs {
     const float *A;
@@ -64,32 +73,34 @@ struct GemmArgs {
     const float *table;  // fused: 126-entry codebook
 };
 
-// LDS image of one operand tile (128 index values x 32 k, 16 KiB):
+// LDS image of one operand tile (ROWS index values x 32 k; ROWS = 128 for A, TN for B):
 //   KC (memory [index][k]): float offset lds_offset(index, k / 4) + k % 4   (swizzled 16-byte columns)
-//   IC (memory [k][index]): float offset k * 128 + index
+//   IC (memory [k][index]): float offset k * ROWS + index
 __device__ __forceinline__ int swizzle_of(int row) { return (row & 7) ^ ((row >> 3) & 3); }
 __device__ __forceinline__ int lds_offset(int row, int quad) {
     return row * BK + ((quad ^ swizzle_of(row)) << 2);
 }
 
 // ---- direct global -> LDS loads ------------------------------------------------------------------
-// A wavefront fills a tile 1 KiB at a time: block b = 4 j + wave (j = 0..3) is rows 8 b .. 8 b + 7 of
-// a KC tile or k rows 2 b, 2 b + 1 of an IC tile, lane l supplying bytes 16 l .. 16 l + 15 of the block.
-template <bool KC>
+// A wavefront fills a tile 1 KiB at a time: block b = NW j + wave is rows 8 b .. 8 b + 7 of a KC tile,
+// or 1024 / ROWS consecutive k rows of an IC tile; lane l supplies bytes 16 l .. 16 l + 15 of the block.
+template <bool KC, int ROWS, int NW>
 struct DirectLoader {
-    uint32_t off[4];  // byte offset of this lane's 16 bytes of block 4 j + wave from the tile corner
+    static constexpr int J = ROWS / 8 / NW;  // blocks per wavefront
+    uint32_t off[J];  // byte offset of this lane's 16 bytes of block NW j + wave from the tile corner
     __device__ __forceinline__ void init(int64_t ld, int wave) {
         const int lane = threadIdx.x & 63;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int blk = 4 * j + wave;
+        for (int j = 0; j < J; ++j) {
+            const int blk = NW * j + wave;
             if (KC) {
                 const int row = 8 * blk + (lane >> 3);
                 const int quad = (lane & 7) ^ swizzle_of(row);
                 off[j] = (uint32_t)((row * ld + 4 * quad) * 4);
             } else {
-                const int k = 2 * blk + (lane >> 5);
-                off[j] = (uint32_t)((k * ld + 4 * (lane & 31)) * 4);
+                constexpr int kLanesPerRow = ROWS / 4;  // 32 or 64
+                const int k = blk * (64 / kLanesPerRow) + lane / kLanesPerRow;
+                off[j] = (uint32_t)((k * ld + 4 * (lane % kLanesPerRow)) * 4);
             }
         }
     }
@@ -105,18 +116,20 @@ struct DirectLoader {
         const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(
             (__attribute__((address_space(3))) float *)lds_stage) + (uint32_t)wave * 1024u;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < J; ++j)
             asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                          :
-                         : "s"(lds0 + (uint32_t)j * 4096u), "v"(off[j]), "s"(rsrc)
+                         : "s"(lds0 + (uint32_t)(j * NW) * 1024u), "v"(off[j]), "s"(rsrc)
                          : "memory", "m0");
     }
 };
 
 // ---- predicated register paths (partial K stage, unaligned operands) ---------------------------------
-// KC operand: lane t covers k quad (t & 7) of rows (t >> 3) + 32 j, j = 0..3.
+// KC operand of ROWS rows, NT lanes: lane t covers k quad (t & 7) of rows (t >> 3) + (NT / 8) j.
+template <int ROWS, int NT>
 struct GuardedKC {
-    uint32_t off[4];
+    static constexpr int RB = NT / 8, J = ROWS / RB;
+    uint32_t off[J];
     uint32_t ok;  // bit j: row of load j is inside the matrix
     int kfirst;
     __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices) {
@@ -124,14 +137,14 @@ struct GuardedKC {
         kfirst = 4 * kq;
         ok = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            off[j] = (uint32_t)(((rb + 32 * j) * ld + 4 * kq) * 4);
-            if (index0 + rb + 32 * j < indices) ok |= 1u << j;
+        for (int j = 0; j < J; ++j) {
+            off[j] = (uint32_t)(((rb + RB * j) * ld + 4 * kq) * 4);
+            if (index0 + rb + RB * j < indices) ok |= 1u << j;
         }
     }
     __device__ __forceinline__ void load(rsrc_t base, int64_t kleft, f32x4 (&reg)[4]) const {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < J; ++j) {
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
             if (ok & (1u << j)) {
 #pragma unroll
@@ -145,29 +158,32 @@ struct GuardedKC {
     __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
         const int kq = threadIdx.x & 7, rb = threadIdx.x >> 3;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) *reinterpret_cast<f32x4 *>(lds + lds_offset(rb + 32 * j, kq)) = reg[j];
+        for (int j = 0; j < J; ++j) *reinterpret_cast<f32x4 *>(lds + lds_offset(rb + RB * j, kq)) = reg[j];
     }
 };
 
-// IC operand, fp32 or codes: lane t covers indices 4 (t & 31) .. +3 of k rows (t >> 5) + 8 r, r = 0..3.
+// IC operand of ROWS indices, fp32 or codes, NT lanes: lane t covers indices 4 (t % (ROWS / 4)) .. + 3 of
+// k rows t / (ROWS / 4) + KR r.
+template <int ROWS, int NT>
 struct GuardedIC {
-    uint32_t off[4];  // byte offsets for an element size of `elem`
+    static constexpr int CQ = ROWS / 4, KR = NT / CQ, R = BK / KR;
+    uint32_t off[R];  // byte offsets for an element size of `elem`
     uint32_t ok;      // bit e: index 4 cq + e is inside the matrix
     __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices, int elem) {
-        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
+        const int cq = threadIdx.x % CQ, kr = threadIdx.x / CQ;
         ok = 0;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) off[r] = (uint32_t)(((kr + 8 * r) * ld + 4 * cq) * elem);
+        for (int r = 0; r < R; ++r) off[r] = (uint32_t)(((kr + KR * r) * ld + 4 * cq) * elem);
 #pragma unroll
         for (int e = 0; e < 4; ++e)
             if (index0 + 4 * cq + e < indices) ok |= 1u << e;
     }
     __device__ __forceinline__ void load(rsrc_t base, int64_t kleft, f32x4 (&reg)[4]) const {
-        const int kr = threadIdx.x >> 5;
+        const int kr = threadIdx.x / CQ;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < R; ++r) {
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (kr + 8 * r < kleft) {
+            if (kr + KR * r < kleft) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                     if (ok & (1u << e))
@@ -177,20 +193,20 @@ struct GuardedIC {
         }
     }
     __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
-        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
+        const int cq = threadIdx.x % CQ, kr = threadIdx.x / CQ;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) *reinterpret_cast<f32x4 *>(lds + (kr + 8 * r) * 128 + 4 * cq) = reg[r];
+        for (int r = 0; r < R; ++r) *reinterpret_cast<f32x4 *>(lds + (kr + KR * r) * ROWS + 4 * cq) = reg[r];
     }
     // Codes: four per 32-bit word.  `whole` = aligned words inside the matrix and inside K.
     __device__ __forceinline__ void load_codes(rsrc_t base, int64_t kleft, bool whole, uint32_t (&reg)[4]) const {
-        const int kr = threadIdx.x >> 5;
+        const int kr = threadIdx.x / CQ;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < R; ++r) {
             if (whole) {
                 reg[r] = __builtin_amdgcn_raw_buffer_load_b32(base, off[r], 0, 0);
             } else {
                 uint32_t w = 0;
-                if (kr + 8 * r < kleft) {
+                if (kr + KR * r < kleft) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         if (ok & (1u << e))
@@ -204,26 +220,32 @@ struct GuardedIC {
     // code 0 decodes to; columns beyond N only reach outputs that are not stored.
     __device__ __forceinline__ void store_codes(float *__restrict__ lds, const float *__restrict__ lut,
                                                 const uint32_t (&reg)[4], int64_t kleft) const {
-        const int cq = threadIdx.x & 31, kr = threadIdx.x >> 5;
+        const int cq = threadIdx.x % CQ, kr = threadIdx.x / CQ;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int r = 0; r < R; ++r) {
             f32x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = lut[(reg[r] >> (8 * e)) & 0xffu];
-            if (kr + 8 * r >= kleft) v = f32x4{0.f, 0.f, 0.f, 0.f};
-            *reinterpret_cast<f32x4 *>(lds + (kr + 8 * r) * 128 + 4 * cq) = v;
+            if (kr + KR * r >= kleft) v = f32x4{0.f, 0.f, 0.f, 0.f};
+            *reinterpret_cast<f32x4 *>(lds + (kr + KR * r) * ROWS + 4 * cq) = v;
         }
     }
 };
 
-template <bool A_KC, int B_KIND>
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
+template <bool A_KC, int B_KIND, int TN>
+__global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmArgs g) {
     constexpr bool B_IS_KC = (B_KIND == B_KC);
     constexpr bool kCodes = (B_KIND == B_CODES);
+    constexpr int BN = TN;
+    constexpr int NW = TN / 32;      // wavefronts: 4 or 8
+    constexpr int NT = 64 * NW;      // lanes
+    constexpr int WN = TN / 64;      // wavefronts along n
+    constexpr int kBStage = TN * BK; // floats of one B stage
+    constexpr int NST = stages_of(TN, B_KIND);  // LDS stages
     extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *sA = smem;                       // [2][kStageFloats]
-    float *sB = smem + 2 * kStageFloats;    // [2][kStageFloats]
-    float *sLut = smem + 4 * kStageFloats;  // [256], fused only
+    float *sA = smem;                                  // [NST][kAStage]
+    float *sB = smem + NST * kAStage;                  // [NST][kBStage]
+    float *sLut = smem + NST * (kAStage + kBStage);    // [256], fused only
 
     // Work unit of this workgroup.  Hardware hands consecutive block ids to the XCDs round-robin;
     // give XCD x the x-th contiguous slice of the unit range.
@@ -262,7 +284,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int wave_m = wave / WN, wave_n = wave % WN;
     const int half = lane >> 5, l32 = lane & 31;
     int row_a[2], row_b[2];
 #pragma unroll
@@ -286,12 +308,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
     const int64_t end_a = A_KC ? (g.M - 1) * g.lda + g.K : (g.K - 1) * g.lda + ((g.M + 3) & ~(int64_t)3);
     const int64_t end_b = B_IS_KC ? (g.N - 1) * g.ldb + g.K : (g.K - 1) * g.ldb + ((g.N + 3) & ~(int64_t)3);
 
-    DirectLoader<A_KC> da;
-    DirectLoader<B_IS_KC> db;
+    DirectLoader<A_KC, BM, NW> da;
+    DirectLoader<B_IS_KC, TN, NW> db;
     da.init(g.lda, wave);
     if (!kCodes) db.init(g.ldb, wave);
-    GuardedKC ga_kc, gb_kc;
-    GuardedIC ga_ic, gb_ic;
+    GuardedKC<BM, NT> ga_kc;
+    GuardedKC<TN, NT> gb_kc;
+    GuardedIC<BM, NT> ga_ic;
+    GuardedIC<TN, NT> gb_ic;
     if (A_KC) ga_kc.init(g.lda, m0, g.M); else ga_ic.init(g.lda, m0, g.M, 4);
     if (B_IS_KC) gb_kc.init(g.ldb, n0, g.N); else gb_ic.init(g.ldb, n0, g.N, kCodes ? 1 : 4);
 
@@ -307,33 +331,41 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
     // One K stage of MFMAs.  Within each group of 8 k values, MFMA s (0..3) consumes
     // k = 8 g + 4 h + s from lane half h on both operands, i.e. the k order inside a stage is
     // permuted identically for A and B.
-    auto compute = [&](int buf) {
-        const float *pa = sA + buf * kStageFloats, *pb = sB + buf * kStageFloats;
+    auto load_frag = [&](const float *pa, const float *pb, int gq, f32x4 (&a)[2], f32x4 (&b)[2]) {
 #pragma unroll
-        for (int gq = 0; gq < BK / 8; ++gq) {
-            f32x4 a[2], b[2];
+        for (int i = 0; i < 2; ++i) {
+            if (A_KC) {
+                a[i] = *reinterpret_cast<const f32x4 *>(pa + lds_offset(row_a[i], 2 * gq + half));
+            } else {
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                if (A_KC) {
-                    a[i] = *reinterpret_cast<const f32x4 *>(pa + lds_offset(row_a[i], 2 * gq + half));
-                } else {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) a[i][s] = pa[(8 * gq + 4 * half + s) * 128 + row_a[i]];
-                }
-                if (B_IS_KC) {
-                    b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset(row_b[i], 2 * gq + half));
-                } else {
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) b[i][s] = pb[(8 * gq + 4 * half + s) * 128 + row_b[i]];
-                }
+                for (int s = 0; s < 4; ++s) a[i][s] = pa[(8 * gq + 4 * half + s) * 128 + row_a[i]];
             }
+            if (B_IS_KC) {
+                b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset(row_b[i], 2 * gq + half));
+            } else {
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
+                for (int s = 0; s < 4; ++s) b[i][s] = pb[(8 * gq + 4 * half + s) * TN + row_b[i]];
+            }
+        }
+    };
+    auto mfma_steps = [&](const f32x4 (&a)[2], const f32x4 (&b)[2], int s_begin, int s_end) {
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi)
+        for (int s = s_begin; s < s_end; ++s)
 #pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi][s], b[ni][s], acc[mi][ni], 0, 0, 0);
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi][s], b[ni][s], acc[mi][ni], 0, 0, 0);
+    };
+    // One stage, self-contained (used by the predicated path).
+    auto compute = [&](int buf) {
+        static_assert(BK == 32, "four groups of 8 k per stage");
+        const float *pa = sA + buf * kAStage, *pb = sB + buf * kBStage;
+        f32x4 a[2], b[2];
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+            load_frag(pa, pb, gq, a, b);
+            mfma_steps(a, b, 0, 4);
         }
     };
 
@@ -349,28 +381,52 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
     if (it0 < it_direct) {
         uint32_t rc[4];
         const bool whole_n = (n0 + BN <= g.N);
-        da.issue(corner_a(it0), limit_of(g.A, end_a, corner_a(it0)), sA, wave);
+        // vmcnt value that leaves exactly the newest stage's direct loads in flight
+        constexpr int kNewest = DirectLoader<A_KC, BM, NW>::J + DirectLoader<B_IS_KC, TN, NW>::J;
+        auto issue_stage = [&](int it, int slot) {
+            da.issue(corner_a(it), limit_of(g.A, end_a, corner_a(it)), sA + slot * kAStage, wave);
+            if (!kCodes) db.issue(corner_b(it), limit_of(Bf, end_b, corner_b(it)), sB + slot * kBStage, wave);
+        };
+        issue_stage(it0, 0);
         if (kCodes) {
             gb_ic.load_codes(make_rsrc(corner_c(it0)), BK, whole_n, rc);
             gb_ic.store_codes(sB, sLut, rc, BK);
-        } else {
-            db.issue(corner_b(it0), limit_of(Bf, end_b, corner_b(it0)), sB, wave);
         }
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
+        if (NST == 3 && it0 + 1 < it_direct) {
+            issue_stage(it0 + 1, 1);
+            __builtin_amdgcn_s_waitcnt(0x0f70 | kNewest);
+        } else {
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
+        }
         __syncthreads();
-        int buf = 0;
+        f32x4 a0[2], b0[2], a1[2], b1[2];
+        int slot = 0;
         for (int it = it0; it < it_direct; ++it) {
-            const bool more = (it + 1 < it_direct);
-            if (more) {  // lands in the other stage while this one is consumed
-                da.issue(corner_a(it + 1), limit_of(g.A, end_a, corner_a(it + 1)), sA + (buf ^ 1) * kStageFloats, wave);
-                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(it + 1)), BK, whole_n, rc);
-                else        db.issue(corner_b(it + 1), limit_of(Bf, end_b, corner_b(it + 1)), sB + (buf ^ 1) * kStageFloats, wave);
+            const int ahead = it + NST - 1;
+            const bool more = (ahead < it_direct);
+            const int slot_next = (slot + 1 == NST) ? 0 : slot + 1;
+            const int slot_ahead = (NST == 2) ? slot_next : ((slot == 0) ? 2 : slot - 1);
+            const float *pa = sA + slot * kAStage, *pb = sB + slot * kBStage;
+            if (more) {  // lands in a free stage while this one is consumed
+                issue_stage(ahead, slot_ahead);
+                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(ahead)), BK, whole_n, rc);
             }
-            compute(buf);
-            if (kCodes && more) gb_ic.store_codes(sB + (buf ^ 1) * kStageFloats, sLut, rc, BK);
-            __builtin_amdgcn_s_waitcnt(0x0f70);
+            // Fragment reads are left to the compiler's schedule (just ahead of their MFMAs; the other
+            // workgroup on the compute unit covers their latency).  The barrier that publishes the next
+            // stage sits eight MFMAs before the end of this one so that it is waited for in their shadow.
+            load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
+            load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, 4);
+            load_frag(pa, pb, 2, a0, b0); mfma_steps(a0, b0, 0, 4);
+            load_frag(pa, pb, 3, a1, b1); mfma_steps(a1, b1, 0, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kCodes && more) gb_ic.store_codes(sB + slot_ahead * kBStage, sLut, rc, BK);
+            // stage it + 1 must have landed; with three stages the loads just issued may stay in flight
+            if (NST == 3 && more) __builtin_amdgcn_s_waitcnt(0x0f70 | kNewest);
+            else                  __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();
-            buf ^= 1;
+            mfma_steps(a1, b1, 2, 4);
+            __builtin_amdgcn_sched_barrier(0);
+            slot = slot_next;
         }
     }
 
@@ -388,10 +444,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_kernel(GemmArgs g) {
         };
         auto stash = [&](int it, int buf) {
             const int64_t kleft = g.K - (int64_t)it * BK;
-            if (A_KC) ga_kc.store(sA + buf * kStageFloats, ra); else ga_ic.store(sA + buf * kStageFloats, ra);
-            if (kCodes)       gb_ic.store_codes(sB + buf * kStageFloats, sLut, rc, kleft);
-            else if (B_IS_KC) gb_kc.store(sB + buf * kStageFloats, rb);
-            else              gb_ic.store(sB + buf * kStageFloats, rb);
+            if (A_KC) ga_kc.store(sA + buf * kAStage, ra); else ga_ic.store(sA + buf * kAStage, ra);
+            if (kCodes)       gb_ic.store_codes(sB + buf * kBStage, sLut, rc, kleft);
+            else if (B_IS_KC) gb_kc.store(sB + buf * kBStage, rb);
+            else              gb_ic.store(sB + buf * kBStage, rb);
         };
         fetch(it_direct);
         stash(it_direct, 0);
@@ -461,19 +517,26 @@ __global__ __launch_bounds__(256) void zero_matrix_kernel(float *__restrict__ C,
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-template <bool A_KC, int B_KIND>
-static cn_status launch(const GemmArgs &args, hipStream_t st) {
-    const size_t lds = (size_t)(4 * kStageFloats + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
+template <bool A_KC, int B_KIND, int TN>
+static cn_status launch_tile(const GemmArgs &args, hipStream_t st) {
+    const size_t lds = (size_t)(stages_of(TN, B_KIND) * (BM + TN) * BK + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND>),
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         configured = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND>), dim3(args.units), dim3(kGemmThreads), lds, st, args);
+    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN>), dim3(args.units), dim3(TN * 2), lds, st, args);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
+
+template <bool A_KC, int B_KIND>
+static cn_status launch(const GemmArgs &args, int tile_n, hipStream_t st) {
+    return tile_n == 256 ? launch_tile<A_KC, B_KIND, 256>(args, st) : launch_tile<A_KC, B_KIND, 128>(args, st);
+}
+
+static int g_force_tile_n = 0;
 
 static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_t K, const float *A,
                            int64_t lda, const void *B, int64_t ldb, float scale, float *C, int64_t ldc,
@@ -500,7 +563,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
-    GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->workspace_bytes);
+    GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->workspace_bytes, g_force_tile_n);
     if (plan.units <= 0 || plan.units > 0x7fffffffLL) {
         set_error("%s: %lld work units exceed the launch limit", who, (long long)plan.units);
         return CN_ERR_SHAPE;
@@ -519,11 +582,11 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.vec_b = w8 ? (aligned(B, 4) && (ldb % 4 == 0)) : (aligned(B, 16) && (ldb % 4 == 0));
     a.scale = scale; a.table = ctx->table;
 
-    if (w8)              s = launch<true, B_CODES>(a, st);
-    else if (!ta && !tb) s = launch<true, B_IC>(a, st);
-    else if (ta && !tb)  s = launch<false, B_IC>(a, st);
-    else if (!ta && tb)  s = launch<true, B_KC>(a, st);
-    else                 s = launch<false, B_KC>(a, st);
+    if (w8)              s = launch<true, B_CODES>(a, plan.tile_n, st);
+    else if (!ta && !tb) s = launch<true, B_IC>(a, plan.tile_n, st);
+    else if (ta && !tb)  s = launch<false, B_IC>(a, plan.tile_n, st);
+    else if (!ta && tb)  s = launch<true, B_KC>(a, plan.tile_n, st);
+    else                 s = launch<false, B_KC>(a, plan.tile_n, st);
     if (s != CN_OK) return s;
 
     if (plan.splits > 1) {
@@ -543,6 +606,9 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
 using namespace cn;
 
 extern "C" {
+
+// Test and tuning hook: 0 = let the planner choose the tile width, 128 / 256 = force it.
+void cn_host_force_gemm_tile_n(int tile_n) { g_force_tile_n = (tile_n == 128 || tile_n == 256) ? tile_n : 0; }
 
 cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                       const float *B, int64_t ldb, float *C, int64_t ldc, void *stream) {

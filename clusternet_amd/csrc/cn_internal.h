@@ -65,13 +65,15 @@ cn_status current_context(Context **out);
 
 // ---- GEMM planning (host, pure function; exported for tests) ---------------------------------
 struct GemmPlan {
+    int tile_n;          // output tile is 128 x tile_n, tile_n = 128 (4 wavefronts) or 256 (8 wavefronts)
     int64_t tiles_m, tiles_n, k_iters;
     int splits;          // number of K chunks (1 = write C directly)
     int64_t iters_per_split;
     int64_t units;       // tiles_m * tiles_n * splits = grid size
 };
-GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes);
+// force_tile_n: 0 = choose, 128 or 256 = use that tile width.
+GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 
-constexpr int kTileM = 128, kTileN = 128, kTileK = 32;
+constexpr int kTileM = 128, kTileK = 32;
 
 }  // namespace cn

@@ -19,6 +19,16 @@ def dev():
     return torch.device("cuda:0")
 
 
+@pytest.fixture(autouse=True, params=[128, 256], ids=["tile128", "tile256"])
+def tile_width(request, dev):
+    """Every case runs on both kernel geometries (128 x 128 and 128 x 256 output tiles); other test
+    modules exercise the planner's own choice."""
+    import clusternet_amd as cn
+    cn.lib().cn_host_force_gemm_tile_n(request.param)
+    yield request.param
+    cn.lib().cn_host_force_gemm_tile_n(0)
+
+
 def _t(a, dev):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
