@@ -30,10 +30,10 @@ FLOP1 = 2.0 * M * N1 * K1
 FLOP2 = 2.0 * M * N2 * N1
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (profiles/gemm_kernel_128x40000x100000_hbm_traffic.txt): FETCH_SIZE 8178439 KiB x 2.0 (the factor
+# file (profiles/gemm_kernel_128x40000x100000_hbm_traffic.txt): FETCH_SIZE 8004218 KiB x 2.0 (the factor
 # that makes the same counter read 3276.8 MB on a 3276.8 MB device-to-device copy) + WRITE_SIZE
 # 260000 KiB x 1.0.  Algorithmic bytes of the same launch: 16.07e9.
-TRAFFIC_BYTES_GEMM1 = 8178439 * 1024 * 2.0 + 260000 * 1024 * 1.0
+TRAFFIC_BYTES_GEMM1 = 8004218 * 1024 * 2.0 + 260000 * 1024 * 1.0
 
 
 def log(*a):
@@ -225,7 +225,7 @@ def main():
         line["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                             "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                             "traffic": TRAFFIC_BYTES_GEMM1,
-                            "kernel": "gemm_kernel<true, 0> (13 K-chunks x 313 tiles) followed by "
+                            "kernel": "gemm_kernel<true, 0, 256> (13 K-chunks x 157 tiles of 128x256) followed by "
                                       "splitk_reduce_kernel, 128x40000x100000; both are inside the timed bracket",
                             "avg_ms": g["gemm1_ms"]}
         extra["gemm2_128x20000x40000"] = {"ms": g["gemm2_ms"], "TFLOPs": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12,

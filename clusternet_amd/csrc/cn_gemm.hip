@@ -1,14 +1,19 @@
 // fp32 GEMM for gfx950 on the matrix cores: C = op(A) op(B), row-major, alpha 1, beta 0, and the
 // fused variant whose B operand is 8-bit codes.
 //
-// One kernel template, gemm_kernel<A_KC, B_KIND, TN>:
-//   * output tile 128 x TN; every wavefront owns 64 x 64 = 2 x 2 blocks of v_mfma_f32_32x32x2_f32
-//     (64 accumulators per lane).  TN = 128: 4 wavefronts (2 x 2), two workgroups per compute unit.
-//     TN = 256: 8 wavefronts (2 x 4), one workgroup per compute unit; the A tile is fetched once per
-//     256 output columns, which halves the L2 -> LDS traffic of the A operand.  Measured, the wide
-//     tile is the slower one on every shape tried, so the planner only uses it on request
-//   * K advances 32 at a time through two LDS stages with one barrier per stage; the global loads
-//     of stage i + 1 are issued before the MFMAs of stage i
+// One kernel template, gemm_kernel<A_KC, B_KIND, TN>, 256 lanes = 4 wavefronts, two workgroups per
+// compute unit, in two geometries:
+//   TN = 128  output tile 128 x 128, wavefronts 2 x 2, each 64 x 64 = 2 x 2 blocks of
+//             v_mfma_f32_32x32x2_f32 (64 accumulators per lane); K advances 32 per stage through two
+//             LDS stages (64 KiB)
+//   TN = 256  output tile 128 x 256, wavefronts 1 x 4, each 128 x 64 = 4 x 2 blocks (128 accumulators
+//             per lane); K advances 16 per stage through two LDS stages (48 KiB).  The A
+//             tile is fetched once per 256 output columns and every B fragment read from LDS feeds four
+//             MFMAs instead of two: less L2 -> LDS and LDS -> register traffic per flop, which matters
+//             because the part runs power-limited on realistic data
+// Common to both:
+//   * one barrier per stage; the global loads of the next stage are issued before the MFMAs of the
+//     current one; the barrier sits eight MFMAs before the end of a stage
 //   * fp32 tiles go from global memory straight into LDS with buffer_load_dwordx4 ... lds, 1 KiB
 //     per wavefront instruction: no staging registers, no LDS store instructions.  An operand
 //     whose memory is contiguous along k (A of dot/dotT, B of dotT) sits in LDS as [index][k], its
@@ -45,19 +50,20 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0xffffffff, 0x00020000);
 }
 
-constexpr int BM = kTileM, BK = kTileK;
-constexpr int kAStage = BM * BK;  // floats of one A stage
+constexpr int BM = kTileM;
+constexpr int NT = 256;  // lanes per workgroup
+constexpr int NW = 4;    // wavefronts per workgroup
 constexpr int kNumXcd = 8;
 
 // What the B operand is.
 enum BKind { B_IC = 0 /* fp32 [k][n] */, B_KC = 1 /* fp32 [n][k] */, B_CODES = 2 /* uint8 [k][n] */ };
 
-// LDS stages in flight.  The wide tile has its compute unit to itself, so nothing covers a stage
-// that arrives late; it keeps two stages in flight behind the one being consumed (3 x 48 KiB).  The
-// coded operand passes through registers and stays at two.
-__host__ __device__ constexpr int stages_of(int tile_n, int b_kind) {
-    return (tile_n == 256 && b_kind != B_CODES) ? 3 : 2;
-}
+// Geometry of a tile width: wavefront grid WM x WN, FM x FN 32 x 32 blocks per wavefront, K depth
+// of a stage, LDS stages.
+template <int TN> struct Geo;
+template <> struct Geo<128> { static constexpr int WM = 2, WN = 2, FM = 2, FN = 2, BK = 32, NST = 2; };
+template <> struct Geo<256> { static constexpr int WM = 1, WN = 4, FM = 4, FN = 2, BK = 16, NST = 2; };
+static_assert(gemm_tile_k(128) == Geo<128>::BK && gemm_tile_k(256) == Geo<256>::BK, "planner and kernel disagree");
 
 struct GemmArgs {
     const float *A;
@@ -73,29 +79,36 @@ struct GemmArgs {
     const float *table;  // fused: 126-entry codebook
 };
 
-// LDS image of one operand tile (ROWS index values x 32 k; ROWS = 128 for A, TN for B):
+// LDS image of one operand tile (ROWS index values x BK k; ROWS = 128 for A, TN for B):
 //   KC (memory [index][k]): float offset lds_offset(index, k / 4) + k % 4   (swizzled 16-byte columns)
 //   IC (memory [k][index]): float offset k * ROWS + index
-__device__ __forceinline__ int swizzle_of(int row) { return (row & 7) ^ ((row >> 3) & 3); }
+// The swizzle makes the 16-byte reads of eight consecutive rows at one k quad hit eight different
+// 16-byte bank groups: rows are 128 bytes (BK 32) or 64 bytes (BK 16) apart.
+template <int BK>
+__device__ __forceinline__ int swizzle_of(int row) {
+    return BK == 32 ? ((row & 7) ^ ((row >> 3) & 3)) : ((row >> 1) & 3);
+}
+template <int BK>
 __device__ __forceinline__ int lds_offset(int row, int quad) {
-    return row * BK + ((quad ^ swizzle_of(row)) << 2);
+    return row * BK + ((quad ^ swizzle_of<BK>(row)) << 2);
 }
 
 // ---- direct global -> LDS loads ------------------------------------------------------------------
-// A wavefront fills a tile 1 KiB at a time: block b = NW j + wave is rows 8 b .. 8 b + 7 of a KC tile,
-// or 1024 / ROWS consecutive k rows of an IC tile; lane l supplies bytes 16 l .. 16 l + 15 of the block.
-template <bool KC, int ROWS, int NW>
+// A wavefront fills a tile 1 KiB at a time: block b = 4 j + wave is 256 / BK consecutive rows of a KC
+// tile or 256 / ROWS consecutive k rows of an IC tile; lane l supplies bytes 16 l .. 16 l + 15 of it.
+template <bool KC, int ROWS, int BK>
 struct DirectLoader {
-    static constexpr int J = ROWS / 8 / NW;  // blocks per wavefront
-    uint32_t off[J];  // byte offset of this lane's 16 bytes of block NW j + wave from the tile corner
+    static constexpr int J = ROWS * BK / 256 / NW;  // blocks per wavefront
+    uint32_t off[J];  // byte offset of this lane's 16 bytes of block 4 j + wave from the tile corner
     __device__ __forceinline__ void init(int64_t ld, int wave) {
         const int lane = threadIdx.x & 63;
 #pragma unroll
         for (int j = 0; j < J; ++j) {
             const int blk = NW * j + wave;
             if (KC) {
-                const int row = 8 * blk + (lane >> 3);
-                const int quad = (lane & 7) ^ swizzle_of(row);
+                constexpr int kQuads = BK / 4;  // lanes per row: 8 or 4
+                const int row = blk * (64 / kQuads) + lane / kQuads;
+                const int quad = (lane % kQuads) ^ swizzle_of<BK>(row);
                 off[j] = (uint32_t)((row * ld + 4 * quad) * 4);
             } else {
                 constexpr int kLanesPerRow = ROWS / 4;  // 32 or 64
@@ -107,7 +120,7 @@ struct DirectLoader {
     // The loads are written as inline assembly on purpose: the compiler's wait-count insertion
     // treats every LDS read that follows a compiler-visible LDS-writing load as dependent on it and
     // would wait for the whole next stage before the first MFMA of the current one.  Completion is
-    // awaited explicitly (vmcnt(0)) before the barrier that publishes the stage.
+    // awaited explicitly (vmcnt) before the barrier that publishes the stage.
     // `limit` = bytes from the corner to the end of the matrix: the descriptor's range check makes
     // every access at or beyond it return zero instead of touching memory.
     __device__ __forceinline__ void issue(const void *corner, uint32_t limit, float *lds_stage, int wave) const {
@@ -125,15 +138,16 @@ struct DirectLoader {
 };
 
 // ---- predicated register paths (partial K stage, unaligned operands) ---------------------------------
-// KC operand of ROWS rows, NT lanes: lane t covers k quad (t & 7) of rows (t >> 3) + (NT / 8) j.
-template <int ROWS, int NT>
+// KC operand of ROWS rows: lane t covers k quad t % (BK / 4) of rows t / (BK / 4) + RB j.
+template <int ROWS, int BK>
 struct GuardedKC {
-    static constexpr int RB = NT / 8, J = ROWS / RB;
+    static constexpr int KQ = BK / 4, RB = NT / KQ, J = ROWS / RB;
+    static_assert(J <= 4, "register staging holds four vectors");
     uint32_t off[J];
     uint32_t ok;  // bit j: row of load j is inside the matrix
     int kfirst;
     __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices) {
-        const int kq = threadIdx.x & 7, rb = threadIdx.x >> 3;
+        const int kq = threadIdx.x % KQ, rb = threadIdx.x / KQ;
         kfirst = 4 * kq;
         ok = 0;
 #pragma unroll
@@ -156,17 +170,18 @@ struct GuardedKC {
         }
     }
     __device__ __forceinline__ void store(float *__restrict__ lds, const f32x4 (&reg)[4]) const {
-        const int kq = threadIdx.x & 7, rb = threadIdx.x >> 3;
+        const int kq = threadIdx.x % KQ, rb = threadIdx.x / KQ;
 #pragma unroll
-        for (int j = 0; j < J; ++j) *reinterpret_cast<f32x4 *>(lds + lds_offset(rb + RB * j, kq)) = reg[j];
+        for (int j = 0; j < J; ++j) *reinterpret_cast<f32x4 *>(lds + lds_offset<BK>(rb + RB * j, kq)) = reg[j];
     }
 };
 
-// IC operand of ROWS indices, fp32 or codes, NT lanes: lane t covers indices 4 (t % (ROWS / 4)) .. + 3 of
+// IC operand of ROWS indices, fp32 or codes: lane t covers indices 4 (t % (ROWS / 4)) .. + 3 of
 // k rows t / (ROWS / 4) + KR r.
-template <int ROWS, int NT>
+template <int ROWS, int BK>
 struct GuardedIC {
     static constexpr int CQ = ROWS / 4, KR = NT / CQ, R = BK / KR;
+    static_assert(R <= 4, "register staging holds four vectors");
     uint32_t off[R];  // byte offsets for an element size of `elem`
     uint32_t ok;      // bit e: index 4 cq + e is inside the matrix
     __device__ __forceinline__ void init(int64_t ld, int64_t index0, int64_t indices, int elem) {
@@ -233,15 +248,15 @@ struct GuardedIC {
 };
 
 template <bool A_KC, int B_KIND, int TN>
-__global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmArgs g) {
+__global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
+    using G = Geo<TN>;
     constexpr bool B_IS_KC = (B_KIND == B_KC);
     constexpr bool kCodes = (B_KIND == B_CODES);
-    constexpr int BN = TN;
-    constexpr int NW = TN / 32;      // wavefronts: 4 or 8
-    constexpr int NT = 64 * NW;      // lanes
-    constexpr int WN = TN / 64;      // wavefronts along n
-    constexpr int kBStage = TN * BK; // floats of one B stage
-    constexpr int NST = stages_of(TN, B_KIND);  // LDS stages
+    constexpr int BN = TN, BK = G::BK, NST = G::NST, FM = G::FM, FN = G::FN;
+    constexpr int kGroups = BK / 8;      // groups of 8 k per stage, 4 FM FN MFMAs each
+    constexpr int kAStage = BM * BK;     // floats of one A stage
+    constexpr int kBStage = TN * BK;     // floats of one B stage
+    static_assert(G::WM * G::WN == NW && G::WM * FM * 32 == BM && G::WN * FN * 32 == TN, "geometry");
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float *sA = smem;                                  // [NST][kAStage]
     float *sB = smem + NST * kAStage;                  // [NST][kBStage]
@@ -284,20 +299,19 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int wave_m = wave / WN, wave_n = wave % WN;
+    const int wave_m = wave / G::WN, wave_n = wave % G::WN;
     const int half = lane >> 5, l32 = lane & 31;
-    int row_a[2], row_b[2];
+    int row_a[FM], row_b[FN];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        row_a[i] = wave_m * 64 + i * 32 + l32;
-        row_b[i] = wave_n * 64 + i * 32 + l32;
-    }
+    for (int i = 0; i < FM; ++i) row_a[i] = wave_m * (32 * FM) + i * 32 + l32;
+#pragma unroll
+    for (int i = 0; i < FN; ++i) row_b[i] = wave_n * (32 * FN) + i * 32 + l32;
 
-    f32x16 acc[2][2];
+    f32x16 acc[FM][FN];
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+        for (int ni = 0; ni < FN; ++ni)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
 
@@ -308,14 +322,14 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
     const int64_t end_a = A_KC ? (g.M - 1) * g.lda + g.K : (g.K - 1) * g.lda + ((g.M + 3) & ~(int64_t)3);
     const int64_t end_b = B_IS_KC ? (g.N - 1) * g.ldb + g.K : (g.K - 1) * g.ldb + ((g.N + 3) & ~(int64_t)3);
 
-    DirectLoader<A_KC, BM, NW> da;
-    DirectLoader<B_IS_KC, TN, NW> db;
+    DirectLoader<A_KC, BM, BK> da;
+    DirectLoader<B_IS_KC, TN, BK> db;
     da.init(g.lda, wave);
     if (!kCodes) db.init(g.ldb, wave);
-    GuardedKC<BM, NT> ga_kc;
-    GuardedKC<TN, NT> gb_kc;
-    GuardedIC<BM, NT> ga_ic;
-    GuardedIC<TN, NT> gb_ic;
+    GuardedKC<BM, BK> ga_kc;
+    GuardedKC<TN, BK> gb_kc;
+    GuardedIC<BM, BK> ga_ic;
+    GuardedIC<TN, BK> gb_ic;
     if (A_KC) ga_kc.init(g.lda, m0, g.M); else ga_ic.init(g.lda, m0, g.M, 4);
     if (B_IS_KC) gb_kc.init(g.ldb, n0, g.N); else gb_ic.init(g.ldb, n0, g.N, kCodes ? 1 : 4);
 
@@ -328,46 +342,39 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
         return bytes <= 0 ? 0u : (bytes > 0xffffffffLL ? 0xffffffffu : (uint32_t)bytes);
     };
 
-    // One K stage of MFMAs.  Within each group of 8 k values, MFMA s (0..3) consumes
-    // k = 8 g + 4 h + s from lane half h on both operands, i.e. the k order inside a stage is
-    // permuted identically for A and B.
-    auto load_frag = [&](const float *pa, const float *pb, int gq, f32x4 (&a)[2], f32x4 (&b)[2]) {
+    // Fragments of one group of 8 k.  MFMA s (0..3) of the group consumes k = 8 g + 4 h + s from lane
+    // half h on both operands, i.e. the k order inside a stage is permuted identically for A and B.
+    auto load_frag = [&](const float *pa, const float *pb, int gq, f32x4 (&a)[FM], f32x4 (&b)[FN]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < FM; ++i) {
             if (A_KC) {
-                a[i] = *reinterpret_cast<const f32x4 *>(pa + lds_offset(row_a[i], 2 * gq + half));
+                a[i] = *reinterpret_cast<const f32x4 *>(pa + lds_offset<BK>(row_a[i], 2 * gq + half));
             } else {
 #pragma unroll
-                for (int s = 0; s < 4; ++s) a[i][s] = pa[(8 * gq + 4 * half + s) * 128 + row_a[i]];
+                for (int s = 0; s < 4; ++s) a[i][s] = pa[(8 * gq + 4 * half + s) * BM + row_a[i]];
             }
+        }
+#pragma unroll
+        for (int i = 0; i < FN; ++i) {
             if (B_IS_KC) {
-                b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset(row_b[i], 2 * gq + half));
+                b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset<BK>(row_b[i], 2 * gq + half));
             } else {
 #pragma unroll
                 for (int s = 0; s < 4; ++s) b[i][s] = pb[(8 * gq + 4 * half + s) * TN + row_b[i]];
             }
         }
     };
-    auto mfma_steps = [&](const f32x4 (&a)[2], const f32x4 (&b)[2], int s_begin, int s_end) {
+    auto mfma_steps = [&](const f32x4 (&a)[FM], const f32x4 (&b)[FN], int s_begin, int s_end) {
 #pragma unroll
         for (int s = s_begin; s < s_end; ++s)
 #pragma unroll
-            for (int mi = 0; mi < 2; ++mi)
+            for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
+                for (int ni = 0; ni < FN; ++ni)
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi][s], b[ni][s], acc[mi][ni], 0, 0, 0);
     };
-    // One stage, self-contained (used by the predicated path).
-    auto compute = [&](int buf) {
-        static_assert(BK == 32, "four groups of 8 k per stage");
-        const float *pa = sA + buf * kAStage, *pb = sB + buf * kBStage;
-        f32x4 a[2], b[2];
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-            load_frag(pa, pb, gq, a, b);
-            mfma_steps(a, b, 0, 4);
-        }
-    };
+    // MFMA steps of the last group that are issued behind the barrier: eight MFMAs.
+    constexpr int kTailFrom = 4 - 8 / (FM * FN);
 
     // Stages [it0, it_direct) use the direct loads (operands allow 16-byte / 4-byte accesses and the
     // stage lies inside K); the rest, if any, goes through predicated registers.
@@ -381,8 +388,7 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
     if (it0 < it_direct) {
         uint32_t rc[4];
         const bool whole_n = (n0 + BN <= g.N);
-        // vmcnt value that leaves exactly the newest stage's direct loads in flight
-        constexpr int kNewest = DirectLoader<A_KC, BM, NW>::J + DirectLoader<B_IS_KC, TN, NW>::J;
+        static_assert(NST == 2, "the loop below double-buffers");
         auto issue_stage = [&](int it, int slot) {
             da.issue(corner_a(it), limit_of(g.A, end_a, corner_a(it)), sA + slot * kAStage, wave);
             if (!kCodes) db.issue(corner_b(it), limit_of(Bf, end_b, corner_b(it)), sB + slot * kBStage, wave);
@@ -392,39 +398,36 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
             gb_ic.load_codes(make_rsrc(corner_c(it0)), BK, whole_n, rc);
             gb_ic.store_codes(sB, sLut, rc, BK);
         }
-        if (NST == 3 && it0 + 1 < it_direct) {
-            issue_stage(it0 + 1, 1);
-            __builtin_amdgcn_s_waitcnt(0x0f70 | kNewest);
-        } else {
-            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
-        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
         __syncthreads();
-        f32x4 a0[2], b0[2], a1[2], b1[2];
+        f32x4 a0[FM], b0[FN], a1[FM], b1[FN];
         int slot = 0;
         for (int it = it0; it < it_direct; ++it) {
-            const int ahead = it + NST - 1;
-            const bool more = (ahead < it_direct);
-            const int slot_next = (slot + 1 == NST) ? 0 : slot + 1;
-            const int slot_ahead = (NST == 2) ? slot_next : ((slot == 0) ? 2 : slot - 1);
+            const bool more = (it + 1 < it_direct);
+            const int slot_next = slot ^ 1;
             const float *pa = sA + slot * kAStage, *pb = sB + slot * kBStage;
-            if (more) {  // lands in a free stage while this one is consumed
-                issue_stage(ahead, slot_ahead);
-                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(ahead)), BK, whole_n, rc);
+            if (more) {  // lands in the other stage while this one is consumed
+                issue_stage(it + 1, slot_next);
+                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(it + 1)), BK, whole_n, rc);
             }
             // Fragment reads are left to the compiler's schedule (just ahead of their MFMAs; the other
-            // workgroup on the compute unit covers their latency).  The barrier that publishes the next
-            // stage sits eight MFMAs before the end of this one so that it is waited for in their shadow.
-            load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
-            load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, 4);
-            load_frag(pa, pb, 2, a0, b0); mfma_steps(a0, b0, 0, 4);
-            load_frag(pa, pb, 3, a1, b1); mfma_steps(a1, b1, 0, 2);
+            // workgroup on the compute unit covers their latency); the register sets alternate.  The
+            // barrier that publishes the next stage sits eight MFMAs before the end of this one so
+            // that it is waited for in their shadow.
+            if (kGroups == 4) {
+                load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
+                load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, 4);
+                load_frag(pa, pb, 2, a0, b0); mfma_steps(a0, b0, 0, 4);
+                load_frag(pa, pb, 3, a1, b1); mfma_steps(a1, b1, 0, kTailFrom);
+            } else {
+                load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
+                load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, kTailFrom);
+            }
             __builtin_amdgcn_sched_barrier(0);
-            if (kCodes && more) gb_ic.store_codes(sB + slot_ahead * kBStage, sLut, rc, BK);
-            // stage it + 1 must have landed; with three stages the loads just issued may stay in flight
-            if (NST == 3 && more) __builtin_amdgcn_s_waitcnt(0x0f70 | kNewest);
-            else                  __builtin_amdgcn_s_waitcnt(0x0f70);
+            if (kCodes && more) gb_ic.store_codes(sB + slot_next * kBStage, sLut, rc, BK);
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // stage it + 1 has landed
             __syncthreads();
-            mfma_steps(a1, b1, 2, 4);
+            mfma_steps(a1, b1, kTailFrom, 4);
             __builtin_amdgcn_sched_barrier(0);
             slot = slot_next;
         }
@@ -432,7 +435,7 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
 
     if (it_direct < it1) {
         // Predicated path: global -> registers (zero-filled outside the matrix) -> LDS, stage in
-        // flight while the previous one is consumed.  Same LDS images as above.
+        // flight while the previous one is consumed.  Same LDS images as above, stages 0 and 1.
         f32x4 ra[4], rb[4];
         uint32_t rc[4];
         auto fetch = [&](int it) {
@@ -456,7 +459,13 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
         for (int it = it_direct; it < it1; ++it) {
             const bool more = (it + 1 < it1);
             if (more) fetch(it + 1);
-            compute(buf);
+            const float *pa = sA + buf * kAStage, *pb = sB + buf * kBStage;
+            f32x4 a[FM], b[FN];
+#pragma unroll
+            for (int gq = 0; gq < kGroups; ++gq) {
+                load_frag(pa, pb, gq, a, b);
+                mfma_steps(a, b, 0, 4);
+            }
             if (more) stash(it + 1, buf ^ 1);
             __syncthreads();
             buf ^= 1;
@@ -470,13 +479,13 @@ __global__ __launch_bounds__(TN * 2, (TN == 128 ? 2 : 1)) void gemm_kernel(GemmA
     if (g.splits > 1) { dst = g.partial + (int64_t)split * g.M * g.N; ldd = g.N; }
     else              { dst = g.C; ldd = g.ldc; }
 #pragma unroll
-    for (int mi = 0; mi < 2; ++mi)
+    for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const int64_t col = n0 + wave_n * 64 + ni * 32 + l32;
+        for (int ni = 0; ni < FN; ++ni) {
+            const int64_t col = n0 + wave_n * (32 * FN) + ni * 32 + l32;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int64_t row = m0 + wave_m * 64 + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const int64_t row = m0 + wave_m * (32 * FM) + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
                 if (row < g.M && col < g.N) dst[row * ldd + col] = acc[mi][ni][r];
             }
         }
@@ -519,14 +528,15 @@ static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<u
 
 template <bool A_KC, int B_KIND, int TN>
 static cn_status launch_tile(const GemmArgs &args, hipStream_t st) {
-    const size_t lds = (size_t)(stages_of(TN, B_KIND) * (BM + TN) * BK + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
+    using G = Geo<TN>;
+    const size_t lds = (size_t)(G::NST * (BM + TN) * G::BK + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
     static bool configured = false;
     if (!configured) {
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         configured = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN>), dim3(args.units), dim3(TN * 2), lds, st, args);
+    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN>), dim3(args.units), dim3(NT), lds, st, args);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

@@ -65,7 +65,7 @@ cn_status current_context(Context **out);
 
 // ---- GEMM planning (host, pure function; exported for tests) ---------------------------------
 struct GemmPlan {
-    int tile_n;          // output tile is 128 x tile_n, tile_n = 128 (4 wavefronts) or 256 (8 wavefronts)
+    int tile_n;          // output tile is 128 x tile_n, tile_n = 128 or 256
     int64_t tiles_m, tiles_n, k_iters;
     int splits;          // number of K chunks (1 = write C directly)
     int64_t iters_per_split;
@@ -74,6 +74,8 @@ struct GemmPlan {
 // force_tile_n: 0 = choose, 128 or 256 = use that tile width.
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 
-constexpr int kTileM = 128, kTileK = 32;
+constexpr int kTileM = 128;
+// K depth of one pipeline stage for a tile width (iters in a GemmPlan count these).
+constexpr int gemm_tile_k(int tile_n) { return tile_n == 256 ? 16 : 32; }
 
 }  // namespace cn

@@ -110,10 +110,10 @@ def test_gemm_plan_covers_k_and_fits_workspace():
                 L.cn_host_plan_gemm(M, N, K, 256, ws, force, out)
                 tm, tn, kit, splits, ips, units, tile_n = list(out)
                 assert tile_n in (128, 256) and (force == 0 or tile_n == force)
-                assert tm == -(-M // 128) and tn == -(-N // tile_n) and kit == max(1, -(-K // 32))
+                assert tm == -(-M // 128) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
                 assert splits >= 1 and units == tm * tn * splits
                 assert ips * splits >= kit and ips * (splits - 1) < kit  # every chunk non-empty
                 if splits > 1:
                     assert splits * M * N * 4 <= ws
-    L.cn_host_plan_gemm(128, 40000, 100000, 256, 1 << 30, 0, out)
+    L.cn_host_plan_gemm(128, 40000, 100000, 256, 1 << 30, 128, out)
     assert list(out)[:6] == [1, 313, 3125, 13, 241, 4069]
