@@ -155,6 +155,72 @@ def bench_fused(torch, cn, dev):
     return res
 
 
+def bench_step(torch, cn, dev):
+    """Maxout training step of the reference's benchmark network at its full sizes (batch 128,
+    100000 -> 8192 -> 8192 -> 10 with pool 2, 2 % dense input): forward, backward, 8-bit gradient round
+    trip and update, phase by phase."""
+    from clusternet_amd import maxout_step as ms
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    B, D, H, C, pool = 128, 100000, 8192, 10, 2
+    X = torch.rand((B, D), device=dev, generator=gen)
+    X = X * (torch.rand((B, D), device=dev, generator=gen) < 0.02)
+    W1 = make_uniform(torch, (D, H), (6.0 / (D + H)) ** 0.5, dev, gen)
+    W2 = make_uniform(torch, (H // pool, H), (6.0 / (H // pool + H)) ** 0.5, dev, gen)
+    W3 = make_uniform(torch, (H // pool, C), (6.0 / (H // pool + C)) ** 0.5, dev, gen)
+    b1 = torch.zeros(H, device=dev); b2 = torch.zeros(H, device=dev); b3 = torch.zeros(C, device=dev)
+    params = (W1, b1, W2, b2, W3, b3)
+    onehot = torch.zeros((B, C), device=dev)
+    onehot[torch.arange(B, device=dev), torch.randint(0, C, (B,), device=dev, generator=gen)] = 1.0
+    state = {}
+
+    def fwd():
+        state["p"], state["cache"] = ms.forward(X, params, pool)
+
+    def bwd():
+        state["grads"] = ms.backward(X, onehot, params, state["p"], state["cache"], pool)
+
+    def codec_update():
+        for w, g in zip((W1, W2, W3), state["grads"]):
+            ms.coded_update(w, g, 1e-3, fused=True)
+
+    def codec_update_unfused():
+        for w, g in zip((W1, W2, W3), state["grads"]):
+            ms.coded_update(w, g, 1e-3, fused=False, scratch=scratch[:g.numel()].view(g.shape))
+
+    rms = [torch.full_like(w, 1e-4) for w in (W1, W2, W3)]
+    scratch = torch.empty(W1.numel(), device=dev)  # where the unfused variants decode to
+
+    def codec_rmsprop():
+        for w, r, g in zip((W1, W2, W3), rms, state["grads"]):
+            ms.coded_rmsprop_update(w, r, g, 0.9, 1e-3, fused=True)
+
+    def codec_rmsprop_unfused():
+        for w, r, g in zip((W1, W2, W3), rms, state["grads"]):
+            ms.coded_rmsprop_update(w, r, g, 0.9, 1e-3, fused=False, scratch=scratch[:g.numel()].view(g.shape))
+
+    out = {}
+    for name, fn in (("forward", fwd), ("backward", bwd), ("codec_and_update", codec_update),
+                     ("codec_and_update_unfused", codec_update_unfused), ("codec_and_rmsprop", codec_rmsprop),
+                     ("codec_and_rmsprop_unfused", codec_rmsprop_unfused)):
+        out[name + "_ms"] = time_region(torch, fn, 5, 2)
+    flop_f = 2.0 * B * (D * H + (H // pool) * H + (H // pool) * C)
+    flop_b = flop_f + 2.0 * B * ((H // pool) * H + (H // pool) * C)
+    elems = D * H + (H // pool) * H + (H // pool) * C
+    out["forward_TFLOPs"] = flop_f / (out["forward_ms"] * 1e-3) / 1e12
+    out["backward_TFLOPs"] = flop_b / (out["backward_ms"] * 1e-3) / 1e12
+    out["codec_and_update_GBps"] = elems * (4 + 5 + 9) / (out["codec_and_update_ms"] * 1e-3) / 1e9
+    out["codec_and_update_unfused_GBps"] = elems * (4 + 5 + 5 + 12) / (out["codec_and_update_unfused_ms"] * 1e-3) / 1e9
+    out["codec_and_rmsprop_GBps"] = elems * (4 + 5 + 17) / (out["codec_and_rmsprop_ms"] * 1e-3) / 1e9
+    out["codec_and_rmsprop_unfused_GBps"] = elems * (4 + 5 + 5 + 20) / (out["codec_and_rmsprop_unfused_ms"] * 1e-3) / 1e9
+    out["step_ms"] = out["forward_ms"] + out["backward_ms"] + out["codec_and_update_ms"]
+    out["note"] = ("bytes per gradient element: absmax 4 + compress 5, then fused decode+update 9 (unfused: decompress 5 + "
+                   "update 12) or fused decode+RMSprop 17 (unfused 5 + 20); "
+                   "the gradient GEMM of layer 1 is 100000 x 8192 x 128")
+    return out
+
+
 def cpu_baseline(torch, tensors):
     """The CPU port (oracle/cpu_port.c, all OpenMP threads) on a column sample of the first dot,
     repeated until about ten seconds of CPU work have been timed."""
@@ -195,7 +261,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--only", choices=["gemm", "codec", "fused"], default=None,
+    ap.add_argument("--only", choices=["gemm", "codec", "fused", "step"], default=None,
                     help="run one part only (for profiling); prints a reduced JSON line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -242,6 +308,9 @@ def main():
             extra["codec"]["cpu_port"] = cpu_codec_baseline()
     if args.only in (None, "fused"):
         extra["fused_w8_gemm_4096x4096"] = bench_fused(torch, cn, dev)
+    if args.only in (None, "step"):
+        torch.cuda.empty_cache()
+        extra["maxout_step_128x100000_8192_8192_10"] = bench_step(torch, cn, dev)
     line["extra"] = extra
     print(json.dumps(line))
 

@@ -51,6 +51,11 @@ def lib():
     L.cn_compress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
     L.cn_decompress_8bit.argtypes = [vp, f32, sz, vp, vp]
     L.cn_decompress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
+    L.cn_decompress_8bit_axpy.argtypes = [vp, f32, f32, sz, vp, vp]
+    L.cn_decompress_8bit_axpy_dp.argtypes = [vp, vp, f32, sz, vp, vp]
+    L.cn_rmsprop_update_f32.argtypes = [vp, vp, vp, f32, f32, sz, vp]
+    L.cn_rmsprop_update_w8.argtypes = [vp, vp, f32, vp, f32, f32, sz, vp]
+    L.cn_rmsprop_update_w8_dp.argtypes = [vp, vp, vp, vp, f32, f32, sz, vp]
     L.cn_host_encode_lut_lookup.argtypes = [C.c_uint32, C.POINTER(C.c_int)]
     L.cn_host_encode_magnitude.argtypes = [f32]
     L.cn_host_plan_gemm.argtypes = [i64, i64, i64, C.c_int, sz, C.c_int, C.POINTER(i64)]
@@ -187,6 +192,49 @@ def decompression_8bit(codes, precision, out=None):
     else:
         check(lib().cn_decompress_8bit(codes.data_ptr(), float(precision), codes.numel(), out.data_ptr(), _stream()))
     return out
+
+
+def decompression_8bit_axpy(codes, precision, alpha, y):
+    """y += alpha * decode(codes), in place, one pass."""
+    import torch
+    _need(codes, torch.uint8, "codes")
+    _need(y, torch.float32, "y")
+    if not (codes.is_contiguous() and y.is_contiguous()) or codes.numel() != y.numel():
+        raise ValueError("codes and y must be contiguous and of equal size")
+    if isinstance(precision, torch.Tensor):
+        check(lib().cn_decompress_8bit_axpy_dp(codes.data_ptr(), precision.data_ptr(), float(alpha), codes.numel(),
+                                               y.data_ptr(), _stream()))
+    else:
+        check(lib().cn_decompress_8bit_axpy(codes.data_ptr(), float(precision), float(alpha), codes.numel(),
+                                            y.data_ptr(), _stream()))
+    return y
+
+
+def rmsprop_update(rms, grad, w, rms_multiplier, learning_rate, precision=None):
+    """RMSprop with weight update, in place on rms and w.  `grad` is fp32, or uint8 codes together
+    with their `precision` (a float or a one-element device tensor)."""
+    import torch
+    _need(rms, torch.float32, "rms")
+    _need(w, torch.float32, "w")
+    if not (rms.is_contiguous() and w.is_contiguous() and grad.is_contiguous()):
+        raise ValueError("operands must be contiguous")
+    if rms.numel() != w.numel() or grad.numel() != w.numel():
+        raise ValueError("operands must be of equal size")
+    n = w.numel()
+    if grad.dtype == torch.uint8:
+        if precision is None:
+            raise ValueError("coded gradient needs its precision")
+        if isinstance(precision, torch.Tensor):
+            check(lib().cn_rmsprop_update_w8_dp(rms.data_ptr(), grad.data_ptr(), precision.data_ptr(), w.data_ptr(),
+                                                float(rms_multiplier), float(learning_rate), n, _stream()))
+        else:
+            check(lib().cn_rmsprop_update_w8(rms.data_ptr(), grad.data_ptr(), float(precision), w.data_ptr(),
+                                             float(rms_multiplier), float(learning_rate), n, _stream()))
+    else:
+        _need(grad, torch.float32, "grad")
+        check(lib().cn_rmsprop_update_f32(rms.data_ptr(), grad.data_ptr(), w.data_ptr(), float(rms_multiplier),
+                                          float(learning_rate), n, _stream()))
+    return rms, w
 
 
 # ---- small kernels around the path (bias, maxout, softmax, ...) ---------------------------------

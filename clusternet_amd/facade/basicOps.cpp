@@ -261,6 +261,22 @@ void decompression_8bit(Matrix * /*tbl_flt*/, Matrix *A, float precision, Matrix
     cn_throw_on_error(cn_decompress_8bit(A->char_data, precision, (size_t)A->size, out->data, nullptr));
 }
 
+void RMSprop_with_weight_update(Matrix *RMS, Matrix *grad, Matrix *w, Matrix * /*m*/, float RMS_multiplier,
+                                float learning_rate, int /*batch_size*/, float /*momentum*/) {
+    cn_throw_on_error(cn_rmsprop_update_f32(RMS->data, grad->data, w->data, RMS_multiplier, learning_rate,
+                                            (size_t)RMS->size, nullptr));
+}
+
+void RMSprop_with_weight_update_from_8bit(Matrix *RMS, Matrix *grad8, float precision, Matrix *w,
+                                          float RMS_multiplier, float learning_rate) {
+    cn_throw_on_error(cn_rmsprop_update_w8(RMS->data, grad8->char_data, precision, w->data, RMS_multiplier,
+                                           learning_rate, (size_t)RMS->size, nullptr));
+}
+
+void decompression_8bit_axpy(Matrix *A, float precision, float alpha, Matrix *out) {
+    cn_throw_on_error(cn_decompress_8bit_axpy(A->char_data, precision, alpha, (size_t)A->size, out->data, nullptr));
+}
+
 // ---- shape checks: same rules and diagnostics as source/basicOps.cu:824-933 -------------------
 int blnFaultySizes(Matrix *A, Matrix *B, Matrix *C) {
     bool ok = A->rows == B->rows && A->cols == B->cols && C->rows == A->rows && C->cols == A->cols;

@@ -79,6 +79,18 @@ void expand_to_maxout_grad(Matrix *error, Matrix *idx, Matrix *grad);  // source
 void compression_8bit(Matrix *tbl_flt, Matrix *A, float precision, Matrix *out);
 void decompression_8bit(Matrix *tbl_flt, Matrix *A, float precision, Matrix *out);
 
+// ---- the passes that follow the 8-bit exchange of a gradient -----------------------------------
+// RMSprop_with_weight_update, source/basicOps.cu:1192-1197: same argument list; `m`, `batch_size`
+// and `momentum` are unused, as in the reference's kernel.
+void RMSprop_with_weight_update(Matrix *RMS, Matrix *grad, Matrix *w, Matrix *m, float RMS_multiplier,
+                                float learning_rate, int batch_size, float momentum);
+// Not in the reference: the same update reading the gradient as 8-bit codes (grad8->char_data), and
+// out += alpha * decode(A) as one pass (decompression_8bit followed by add / sub / a scaled step,
+// source/Layer.cpp:430-431, source/DeepNeuralNetwork.cpp:338-339).
+void RMSprop_with_weight_update_from_8bit(Matrix *RMS, Matrix *grad8, float precision, Matrix *w,
+                                          float RMS_multiplier, float learning_rate);
+void decompression_8bit_axpy(Matrix *A, float precision, float alpha, Matrix *out);
+
 // ---- shape checks (source/basicOps.cu:824-933) ----------------------------------------------
 int blnFaultySizes(Matrix *A, Matrix *B, Matrix *C);
 int blnFaultyMatrixProductSizes(Matrix *A, Matrix *B, Matrix *C, MatrixOp T1, MatrixOp T2);

@@ -7,7 +7,8 @@ into libcnhip.
     z1 = X W1 + b1;  h1, a1 = maxout(z1);  z2 = h1 W2 + b2;  h2, a2 = maxout(z2)
     p  = softmax(h2 W3 + b3);  e3 = p - onehot(y)
     gW3 = h2^T e3;  e2 = expand(e3 W3^T, a2);  gW2 = h1^T e2;  e1 = expand(e2 W2^T, a1);  gW1 = X^T e1
-    each gW -> absmax -> compression_8bit -> decompression_8bit -> W -= rate * gW'
+    each gW -> absmax -> compression_8bit -> W -= rate * decode(codes)   (one fused pass, identical
+    bit for bit to decompression_8bit followed by the update)
 Biases are inputs and are not updated.
 """
 from . import _lib as L
@@ -42,11 +43,34 @@ def codec_round_trip(grad):
     return L.decompression_8bit(codes, prec, out=grad), codes, prec
 
 
+def coded_update(w, grad, rate, fused=True, scratch=None):
+    """W -= rate * decode(encode(grad)).  `fused` picks the one-pass kernel; the unfused sequence
+    (decompression_8bit into `scratch`, or over `grad` itself, then the update) gives the same bits."""
+    prec = L.absmax(grad)
+    codes = L.compression_8bit(grad, prec)
+    if fused:
+        L.decompression_8bit_axpy(codes, prec, -rate, w)
+    else:
+        L.sgd_update(w, L.decompression_8bit(codes, prec, out=grad if scratch is None else scratch), rate)
+    return codes, prec
+
+
+def coded_rmsprop_update(w, rms, grad, rms_multiplier, rate, fused=True, scratch=None):
+    """RMSprop with weight update (source/basicOps.cu:1192-1197) on the 8-bit round trip of `grad`."""
+    prec = L.absmax(grad)
+    codes = L.compression_8bit(grad, prec)
+    if fused:
+        L.rmsprop_update(rms, codes, w, rms_multiplier, rate, precision=prec)
+    else:
+        L.rmsprop_update(rms, L.decompression_8bit(codes, prec, out=grad if scratch is None else scratch), w,
+                         rms_multiplier, rate)
+    return codes, prec
+
+
 def step(X, onehot, params, rate, pool=2):
     p, cache = forward(X, params, pool)
     grads = backward(X, onehot, params, p, cache, pool)
     W = (params[0], params[2], params[4])
     for w, g in zip(W, grads):
-        g8, _, _ = codec_round_trip(g)
-        L.sgd_update(w, g8, rate)
+        coded_update(w, g, rate)
     return p

@@ -113,6 +113,37 @@ cn_status cn_decompress_8bit(const uint8_t *codes_device, float precision, size_
 cn_status cn_decompress_8bit_dp(const uint8_t *codes_device, const float *precision_device,
                                 size_t n, float *out_device, void *stream);
 
+/* ---- fused passes that follow the 8-bit exchange of a gradient ------------------------------- */
+
+/* y[i] = y[i] + alpha * decode(codes[i]) in one pass (9 bytes per element instead of 17), decode as
+ * in cn_decompress_8bit.  alpha = 1 replaces decompression_8bit followed by add, the accumulation of
+ * the peers' gradients (source/Layer.cpp:430-431); alpha = -1 replaces decompression_8bit followed by
+ * sub (source/DeepNeuralNetwork.cpp:338-339); alpha = -rate is a plain gradient step on coded
+ * gradients.  The product alpha * decode is rounded before the addition, so the result equals
+ * cn_decompress_8bit followed by cn_sgd_update_f32 / add / sub bit for bit. */
+cn_status cn_decompress_8bit_axpy(const uint8_t *codes_device, float precision, float alpha, size_t n,
+                                  float *y_device, void *stream);
+cn_status cn_decompress_8bit_axpy_dp(const uint8_t *codes_device, const float *precision_device,
+                                     float alpha, size_t n, float *y_device, void *stream);
+
+/* RMSprop with weight update, RMSprop_with_weight_update (source/basicOps.cu:1192-1197, kernel
+ * source/clusterKernels.cu:1305-1325), per element:
+ *   rms = rms_multiplier * rms + grad * grad * (1 - rms_multiplier)
+ *   w   = w - learning_rate * (grad / (sqrtf(rms) + 1e-8f))
+ * every operation rounded to fp32 in that order.  The reference divides with fdividef, which CUDA
+ * documents as accurate to 2 ulp; here the division is correctly rounded.  (The batch_size, momentum
+ * and m arguments of the reference routine are unused by its kernel.) */
+cn_status cn_rmsprop_update_f32(float *rms_device, const float *grad_device, float *w_device,
+                                float rms_multiplier, float learning_rate, size_t n, void *stream);
+/* Same with the gradient given as 8-bit codes (decode as in cn_decompress_8bit): one pass of 17
+ * bytes per element instead of decompression (5) followed by the update (20). */
+cn_status cn_rmsprop_update_w8(float *rms_device, const uint8_t *codes_device, float precision,
+                               float *w_device, float rms_multiplier, float learning_rate, size_t n,
+                               void *stream);
+cn_status cn_rmsprop_update_w8_dp(float *rms_device, const uint8_t *codes_device,
+                                  const float *precision_device, float *w_device, float rms_multiplier,
+                                  float learning_rate, size_t n, void *stream);
+
 /* ---- small kernels used around the path by its callers (row-major, flat where no shape is given).
  * They are not on the measured hot path; each names the reference routine it stands in for. */
 

@@ -34,6 +34,8 @@ def _load():
         getattr(lib, name).argtypes = [_f32p, _c.c_float, _c.c_size_t, _u8p, _c.c_int]
     lib.cn_oracle_decode_lut.argtypes = [_c.c_float, _f32p]
     lib.cn_oracle_decompress.argtypes = [_u8p, _c.c_float, _c.c_size_t, _f32p]
+    lib.cn_oracle_decompress_axpy.argtypes = [_u8p, _c.c_float, _c.c_float, _c.c_size_t, _f32p]
+    lib.cn_oracle_rmsprop_update.argtypes = [_f32p, _f32p, _f32p, _c.c_float, _c.c_float, _c.c_size_t]
     lib.cn_oracle_absmax.argtypes = [_f32p, _c.c_size_t]
     lib.cn_oracle_absmax.restype = _c.c_float
     g = [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _f32p, _c.c_int64, _f32p,
@@ -97,6 +99,24 @@ def decompress(codes, precision):
     out = np.empty(codes.shape, np.float32)
     _lib.cn_oracle_decompress(codes.reshape(-1), float(precision), codes.size, out.reshape(-1))
     return out
+
+
+def decompress_axpy(codes, precision, alpha, y):
+    """Returns y + alpha * decode(codes) (y is not modified)."""
+    codes = np.ascontiguousarray(codes, dtype=np.uint8)
+    out = np.array(y, dtype=np.float32, order="C", copy=True)
+    _lib.cn_oracle_decompress_axpy(codes.reshape(-1), float(precision), float(alpha), codes.size, out.reshape(-1))
+    return out
+
+
+def rmsprop_update(rms, grad, w, rms_multiplier, learning_rate):
+    """Returns (rms', w') of one RMSprop-with-weight-update pass (inputs are not modified)."""
+    r = np.array(rms, dtype=np.float32, order="C", copy=True)
+    ww = np.array(w, dtype=np.float32, order="C", copy=True)
+    g = _f32(grad)
+    _lib.cn_oracle_rmsprop_update(r.reshape(-1), g.reshape(-1), ww.reshape(-1), float(rms_multiplier),
+                                  float(learning_rate), g.size)
+    return r, ww
 
 
 def absmax(x):

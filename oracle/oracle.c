@@ -10,6 +10,15 @@
  *   cn_oracle_compress_closed    same kernel, second independent formulation (count of odd
  *                                table entries below the input, then a two-candidate pick)
  *   cn_oracle_decompress         source/clusterKernels.cu:1135-1160 (kDecompression_8bit)
+ *   cn_oracle_decompress_axpy    cn_oracle_decompress followed by y = y + alpha * g with the product
+ *                                rounded first: decompression_8bit then add (source/Layer.cpp:430-431),
+ *                                sub (source/DeepNeuralNetwork.cpp:338-339) or a scaled step
+ *   cn_oracle_rmsprop_update     source/clusterKernels.cu:1305-1325 (kRMSprop_with_weight_update),
+ *                                powf(g, 2) as g * g, fdividef as IEEE division (CUDA documents
+ *                                fdividef as accurate to 2 ulp, so the reference itself is only
+ *                                defined to that accuracy).  Pinned by its closed forms: multiplier
+ *                                0 and 1, zero gradient, and an fp64 evaluation of the same formula
+ *                                (tests/test_oracle_codec.py)
  *   cn_oracle_absmax             source/basicOps.cu:810-822 + source/clusterKernels.cu:429-436
  *                                (abs) followed by source/basicOps.cu:1076-1081 (max)
  *   cn_oracle_gemm_*             source/clusterNet.cpp:404-461: C = op(A) op(B), alpha 1, beta 0,
@@ -133,6 +142,32 @@ void cn_oracle_decompress(const uint8_t *codes, float precision, size_t n, float
     float lut[256];
     cn_oracle_decode_lut(precision, lut);
     for (size_t i = 0; i < n; ++i) out[i] = lut[codes[i]];
+}
+
+void cn_oracle_decompress_axpy(const uint8_t *codes, float precision, float alpha, size_t n, float *y) {
+    float lut[256];
+    cn_oracle_decode_lut(precision, lut);
+    for (size_t i = 0; i < n; ++i) {
+        volatile float scaled = alpha * lut[codes[i]];
+        y[i] = y[i] + scaled;
+    }
+}
+
+void cn_oracle_rmsprop_update(float *rms, const float *grad, float *w, float rms_multiplier,
+                              float learning_rate, size_t n) {
+    const float one_minus = 1.0f - rms_multiplier;
+    for (size_t i = 0; i < n; ++i) {
+        const float g = grad[i];
+        volatile float a = rms_multiplier * rms[i];
+        volatile float sq = g * g;
+        volatile float b = sq * one_minus;
+        const float r = a + b;
+        volatile float den = sqrtf(r) + 1.0e-08f;
+        volatile float q = g / den;
+        volatile float step = learning_rate * q;
+        rms[i] = r;
+        w[i] = w[i] - step;
+    }
 }
 
 /* max_i |x_i|, start value -1 as in the reference's reduction; NaN propagates. */

@@ -18,6 +18,9 @@
 extern "C" {
 void cn_oracle_compress_literal(const float *x, float precision, size_t n, uint8_t *codes, int sliver_rule);
 void cn_oracle_decompress(const uint8_t *codes, float precision, size_t n, float *out);
+void cn_oracle_decompress_axpy(const uint8_t *codes, float precision, float alpha, size_t n, float *y);
+void cn_oracle_rmsprop_update(float *rms, const float *grad, float *w, float rms_multiplier, float learning_rate,
+                              size_t n);
 }
 
 static int failures = 0;
@@ -193,6 +196,31 @@ static void run_codec_test(ClusterNet gpu) {
     Matrix *back2 = empty(128, 4000);
     gpu.decompression_8bit(codes2, precision, back2);
     CHECK(memcmp(to_host(back2)->data, want_f.data(), back_host->bytes) == 0, "decompression_8bit(out)");
+
+    // the passes behind the exchange: decode + accumulate, RMSprop on fp32 and on coded gradients
+    {
+        Matrix *acc = gpu.randn(128, 4000, 0.0f, 1.0f);
+        std::vector<float> acc_want(a_host->size);
+        memcpy(acc_want.data(), to_host(acc)->data, acc->bytes);
+        cn_oracle_decompress_axpy(want.data(), precision, 1.0f, want.size(), acc_want.data());
+        decompression_8bit_axpy(codes, precision, 1.0f, acc);
+        CHECK(memcmp(to_host(acc)->data, acc_want.data(), acc->bytes) == 0, "decompression_8bit_axpy == decompress then add");
+
+        Matrix *rms = gpu.rand(128, 4000);
+        Matrix *w = gpu.randn(128, 4000, 0.0f, 0.1f);
+        Matrix *rms_b = to_gpu(to_host(rms));
+        Matrix *w_b = to_gpu(to_host(w));
+        std::vector<float> rms_want(a_host->size), w_want(a_host->size);
+        memcpy(rms_want.data(), to_host(rms)->data, rms->bytes);
+        memcpy(w_want.data(), to_host(w)->data, w->bytes);
+        cn_oracle_rmsprop_update(rms_want.data(), want_f.data(), w_want.data(), 0.9f, 0.003f, want_f.size());
+        RMSprop_with_weight_update(rms, back, w, w, 0.9f, 0.003f, 128, 0.5f);
+        CHECK(memcmp(to_host(rms)->data, rms_want.data(), rms->bytes) == 0, "RMSprop_with_weight_update: RMS");
+        CHECK(memcmp(to_host(w)->data, w_want.data(), w->bytes) == 0, "RMSprop_with_weight_update: weights");
+        RMSprop_with_weight_update_from_8bit(rms_b, codes, precision, w_b, 0.9f, 0.003f);
+        CHECK(memcmp(to_host(rms_b)->data, rms_want.data(), rms->bytes) == 0, "RMSprop on codes: RMS");
+        CHECK(memcmp(to_host(w_b)->data, w_want.data(), w->bytes) == 0, "RMSprop on codes: weights");
+    }
 
     // fused product on coded weights against dot on the decoded weights
     Matrix *W = gpu.randn(4000, 96, 0.0f, 0.05f);

@@ -1,0 +1,115 @@
+"""Parity of the fused update passes with the CPU checker and with the unfused kernels they replace,
+through the C-ABI.  Everything here is bit-exact: each pass performs the same fp32 operations in
+the same order as decompression followed by the element-wise step."""
+import numpy as np
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    import clusternet_amd as cn
+    cn.init(0)
+    return torch.device("cuda:0")
+
+
+def _t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 1023, 4096, 4097, 1_000_003])
+@pytest.mark.parametrize("alpha", [1.0, -1.0, -0.01])
+def test_decompress_axpy_matches_checker(dev, n, alpha):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(n + 7)
+    codes = rng.integers(0, 256, n, dtype=np.uint8)
+    y = rng.normal(0, 1, n).astype(np.float32)
+    prec = 0.0371
+    want = oracle.decompress_axpy(codes, prec, alpha, y)
+    got = cn.decompression_8bit_axpy(_t(codes, dev), prec, alpha, _t(y, dev)).cpu().numpy()
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+def test_decompress_axpy_equals_the_unfused_kernels_and_takes_device_precision(dev):
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(11)
+    n = 8_388_608 + 5
+    x = torch.randn(n, device=dev, generator=gen) * 0.02
+    w = torch.randn(n, device=dev, generator=gen)
+    prec = cn.absmax(x)                              # one-element device tensor
+    codes = cn.compression_8bit(x, prec)
+    rate = 0.0125
+    w_ref = w.clone()
+    L.sgd_update(w_ref, cn.decompression_8bit(codes, prec), rate)
+    w_fused = cn.decompression_8bit_axpy(codes, prec, -rate, w.clone())
+    assert torch.equal(w_ref.view(torch.int32), w_fused.view(torch.int32))
+    acc = w.clone()
+    acc_ref = acc + cn.decompression_8bit(codes, prec)   # accumulation of a peer's gradient
+    cn.decompression_8bit_axpy(codes, float(prec.cpu()[0]), 1.0, acc)
+    assert torch.equal(acc_ref.view(torch.int32), acc.view(torch.int32))
+    # unaligned views take the scalar path
+    w2 = w.clone()
+    cn.decompression_8bit_axpy(codes[1:], prec, -rate, w2[1:])
+    assert torch.equal(w2[1:].view(torch.int32), w_ref[1:].view(torch.int32)) and w2[0] == w[0]
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 4099, 1_000_003])
+def test_rmsprop_update_matches_checker(dev, n):
+    import clusternet_amd as cn
+    rng = np.random.default_rng(n + 3)
+    g = (rng.normal(0, 0.05, n) * (rng.random(n) < 0.9)).astype(np.float32)
+    rms = rng.uniform(0, 0.01, n).astype(np.float32)
+    rms[::7] = 0.0
+    w = rng.normal(0, 0.05, n).astype(np.float32)
+    for mult, lr in ((0.9, 0.003), (0.0, 0.1), (1.0, 0.01)):
+        r_want, w_want = oracle.rmsprop_update(rms, g, w, mult, lr)
+        r_t, w_t = _t(rms, dev), _t(w, dev)
+        cn.rmsprop_update(r_t, _t(g, dev), w_t, mult, lr)
+        assert np.array_equal(_bits(r_t.cpu().numpy()), _bits(r_want))
+        assert np.array_equal(_bits(w_t.cpu().numpy()), _bits(w_want))
+
+
+def test_rmsprop_update_on_codes_equals_decompress_then_update(dev):
+    import torch
+    import clusternet_amd as cn
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(12)
+    n = 4_194_304 + 3
+    x = torch.randn(n, device=dev, generator=gen) * 0.02
+    w = torch.randn(n, device=dev, generator=gen) * 0.05
+    rms = torch.rand(n, device=dev, generator=gen) * 0.01
+    prec = cn.absmax(x)
+    codes = cn.compression_8bit(x, prec)
+    r_ref, w_ref = rms.clone(), w.clone()
+    cn.rmsprop_update(r_ref, cn.decompression_8bit(codes, prec), w_ref, 0.9, 0.003)
+    for p in (prec, float(prec.cpu()[0])):
+        r_f, w_f = rms.clone(), w.clone()
+        cn.rmsprop_update(r_f, codes, w_f, 0.9, 0.003, precision=p)
+        assert torch.equal(r_ref.view(torch.int32), r_f.view(torch.int32))
+        assert torch.equal(w_ref.view(torch.int32), w_f.view(torch.int32))
+    # and against the checker on a slice
+    k = 100_000
+    r_want, w_want = oracle.rmsprop_update(rms[:k].cpu().numpy(), oracle.decompress(codes[:k].cpu().numpy(), float(prec.cpu()[0])),
+                                           w[:k].cpu().numpy(), 0.9, 0.003)
+    assert np.array_equal(_bits(r_ref[:k].cpu().numpy()), _bits(r_want))
+    assert np.array_equal(_bits(w_ref[:k].cpu().numpy()), _bits(w_want))
+
+
+def test_null_and_size_errors(dev):
+    import clusternet_amd as cn
+    L = cn.lib()
+    assert L.cn_decompress_8bit_axpy(None, 1.0, 1.0, 4, None, None) == 1
+    assert L.cn_rmsprop_update_f32(None, None, None, 0.9, 0.1, 4, None) == 1
+    assert L.cn_decompress_8bit_axpy(None, 1.0, 1.0, 0, None, None) == 0
