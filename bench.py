@@ -181,6 +181,15 @@ def bench_step(torch, cn, dev):
     def bwd():
         state["grads"] = ms.backward(X, onehot, params, state["p"], state["cache"], pool)
 
+    maxima = [torch.empty(1, device=dev) for _ in range(3)]
+
+    def bwd_absmax():  # the gradient products also deliver max|gW|
+        state["grads"] = ms.backward(X, onehot, params, state["p"], state["cache"], pool, absmax_out=maxima)
+
+    def codec_update_given_max():
+        for w, g, m in zip((W1, W2, W3), state["grads"], maxima):
+            ms.coded_update(w, g, 1e-3, fused=True, prec=m)
+
     def codec_update():
         for w, g in zip((W1, W2, W3), state["grads"]):
             ms.coded_update(w, g, 1e-3, fused=True)
@@ -201,7 +210,9 @@ def bench_step(torch, cn, dev):
             ms.coded_rmsprop_update(w, r, g, 0.9, 1e-3, fused=False, scratch=scratch[:g.numel()].view(g.shape))
 
     out = {}
-    for name, fn in (("forward", fwd), ("backward", bwd), ("codec_and_update", codec_update),
+    for name, fn in (("forward", fwd), ("backward_with_absmax", bwd_absmax),
+                     ("compress_and_update_given_absmax", codec_update_given_max),
+                     ("backward", bwd), ("codec_and_update", codec_update),
                      ("codec_and_update_unfused", codec_update_unfused), ("codec_and_rmsprop", codec_rmsprop),
                      ("codec_and_rmsprop_unfused", codec_rmsprop_unfused)):
         out[name + "_ms"] = time_region(torch, fn, 5, 2)
@@ -214,7 +225,8 @@ def bench_step(torch, cn, dev):
     out["codec_and_update_unfused_GBps"] = elems * (4 + 5 + 5 + 12) / (out["codec_and_update_unfused_ms"] * 1e-3) / 1e9
     out["codec_and_rmsprop_GBps"] = elems * (4 + 5 + 17) / (out["codec_and_rmsprop_ms"] * 1e-3) / 1e9
     out["codec_and_rmsprop_unfused_GBps"] = elems * (4 + 5 + 5 + 20) / (out["codec_and_rmsprop_unfused_ms"] * 1e-3) / 1e9
-    out["step_ms"] = out["forward_ms"] + out["backward_ms"] + out["codec_and_update_ms"]
+    out["step_ms"] = out["forward_ms"] + out["backward_with_absmax_ms"] + out["compress_and_update_given_absmax_ms"]
+    out["step_unfused_ms"] = out["forward_ms"] + out["backward_ms"] + out["codec_and_update_unfused_ms"]
     out["note"] = ("bytes per gradient element: absmax 4 + compress 5, then fused decode+update 9 (unfused: decompress 5 + "
                    "update 12) or fused decode+RMSprop 17 (unfused 5 + 20); "
                    "the gradient GEMM of layer 1 is 100000 x 8192 x 128")

@@ -45,6 +45,7 @@ def lib():
     L.cn_synchronize.argtypes = [vp]
     L.cn_table_get.argtypes = [C.POINTER(f32)]
     L.cn_gemm_f32.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp]
+    L.cn_gemm_f32_absmax.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, vp]
     L.cn_gemm_f32_w8.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, vp, i64, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
@@ -104,8 +105,9 @@ def _ld(t):
     return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
 
 
-def gemm(A, B, trans_a=False, trans_b=False, out=None):
-    """out = op(A) op(B) on row-major fp32 matrices; mirrors ClusterNet::dot(A,B,out,T1,T2)."""
+def gemm(A, B, trans_a=False, trans_b=False, out=None, absmax_out=None):
+    """out = op(A) op(B) on row-major fp32 matrices; mirrors ClusterNet::dot(A,B,out,T1,T2).
+    `absmax_out` (one-element fp32 device tensor) additionally receives max|out|."""
     import torch
     _need(A, torch.float32, "A")
     _need(B, torch.float32, "B")
@@ -117,17 +119,22 @@ def gemm(A, B, trans_a=False, trans_b=False, out=None):
     if K != K2 or tuple(out.shape) != (M, N):
         raise CnError(2, "Matrix size error: op(A) %dx%d, op(B) %dx%d, out %dx%d"
                       % (M, K, K2, N, out.shape[0], out.shape[1]))
-    check(lib().cn_gemm_f32(int(trans_a), int(trans_b), M, N, K, A.data_ptr(), _ld(A), B.data_ptr(),
-                            _ld(B), out.data_ptr(), _ld(out), _stream()))
+    if absmax_out is not None:
+        _need(absmax_out, torch.float32, "absmax_out")
+        check(lib().cn_gemm_f32_absmax(int(trans_a), int(trans_b), M, N, K, A.data_ptr(), _ld(A), B.data_ptr(),
+                                       _ld(B), out.data_ptr(), _ld(out), absmax_out.data_ptr(), _stream()))
+    else:
+        check(lib().cn_gemm_f32(int(trans_a), int(trans_b), M, N, K, A.data_ptr(), _ld(A), B.data_ptr(),
+                                _ld(B), out.data_ptr(), _ld(out), _stream()))
     return out
 
 
-def dot(A, B, out=None):
-    return gemm(A, B, False, False, out)
+def dot(A, B, out=None, absmax_out=None):
+    return gemm(A, B, False, False, out, absmax_out)
 
 
-def Tdot(A, B, out=None):
-    return gemm(A, B, True, False, out)
+def Tdot(A, B, out=None, absmax_out=None):
+    return gemm(A, B, True, False, out, absmax_out)
 
 
 def dotT(A, B, out=None):

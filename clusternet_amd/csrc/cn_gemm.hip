@@ -77,7 +77,20 @@ struct GemmArgs {
     int vec_a, vec_b;    // operand base and leading dimension allow 16-byte (fp32) / 4-byte (codes) loads
     float scale;         // fused: decode scale
     const float *table;  // fused: 126-entry codebook
+    uint32_t *amax;      // optional: receives max |C| as the bit pattern of a non-negative float
 };
+
+// max over the wavefront of a non-negative float's bit pattern, then one atomic per wavefront.
+// Bit patterns of non-negative floats order like the floats, so the unsigned maximum is exact and
+// independent of the order of the updates.
+__device__ __forceinline__ void publish_absmax(uint32_t v, uint32_t *amax) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)v, off, 64);
+        v = o > v ? o : v;
+    }
+    if ((threadIdx.x & 63) == 0) atomicMax(amax, v);
+}
 
 // LDS image of one operand tile (ROWS index values x BK k; ROWS = 128 for A, TN for B):
 //   KC (memory [index][k]): float offset lds_offset(index, k / 4) + k % 4   (swizzled 16-byte columns)
@@ -478,6 +491,8 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
     int64_t ldd;
     if (g.splits > 1) { dst = g.partial + (int64_t)split * g.M * g.N; ldd = g.N; }
     else              { dst = g.C; ldd = g.ldc; }
+    const bool want_amax = (g.amax != nullptr) && (g.splits == 1);  // with chunks the reduction does it
+    uint32_t amax = 0;
 #pragma unroll
     for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
@@ -486,16 +501,22 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int64_t row = m0 + wave_m * (32 * FM) + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (row < g.M && col < g.N) dst[row * ldd + col] = acc[mi][ni][r];
+                if (row < g.M && col < g.N) {
+                    dst[row * ldd + col] = acc[mi][ni][r];
+                    const uint32_t bits = __float_as_uint(acc[mi][ni][r]) & 0x7fffffffu;
+                    amax = bits > amax ? bits : amax;
+                }
             }
         }
+    if (want_amax) publish_absmax(amax, g.amax);
 }
 
 // C[m][n] = sum over chunks of partial[chunk][m][n], chunks added in ascending order.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partial, int splits,
                                                             int64_t M, int64_t N, float *__restrict__ C,
-                                                            int64_t ldc, int vec) {
+                                                            int64_t ldc, int vec, uint32_t *amax_out) {
     const int64_t plane = M * N;
+    uint32_t amax = 0;
     if (vec) {
         const int64_t nq = N / 4, total = M * nq;
         for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
@@ -505,6 +526,11 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
             f32x4 s = *reinterpret_cast<const f32x4 *>(src);
             for (int c = 1; c < splits; ++c) s += *reinterpret_cast<const f32x4 *>(src + c * plane);
             *reinterpret_cast<f32x4 *>(C + m * ldc + 4 * q) = s;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t bits = __float_as_uint(s[e]) & 0x7fffffffu;
+                amax = bits > amax ? bits : amax;
+            }
         }
     } else {
         for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < plane;
@@ -513,8 +539,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
             float s = partial[i];
             for (int c = 1; c < splits; ++c) s += partial[i + c * plane];
             C[m * ldc + n] = s;
+            const uint32_t bits = __float_as_uint(s) & 0x7fffffffu;
+            amax = bits > amax ? bits : amax;
         }
     }
+    if (amax_out) publish_absmax(amax, amax_out);
+}
+
+__global__ void set_word_kernel(uint32_t *p, uint32_t value) {
+    if (threadIdx.x == 0) *p = value;
 }
 
 __global__ __launch_bounds__(256) void zero_matrix_kernel(float *__restrict__ C, int64_t M, int64_t N, int64_t ldc) {
@@ -550,7 +583,7 @@ static int g_force_tile_n = 0;
 
 static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_t K, const float *A,
                            int64_t lda, const void *B, int64_t ldb, float scale, float *C, int64_t ldc,
-                           void *stream) {
+                           float *absmax_out, void *stream) {
     const char *who = w8 ? "gemm_f32_w8" : "gemm_f32";
     if (M < 0 || N < 0 || K < 0) { set_error("%s: negative dimension", who); return CN_ERR_SHAPE; }
     if (lda < (ta ? M : K) || ldb < (tb ? K : N) || ldc < N) {
@@ -562,12 +595,20 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         set_error("%s: leading dimensions above 2^22 elements are not supported", who);
         return CN_ERR_SHAPE;
     }
-    if (M == 0 || N == 0) return CN_OK;
-    if (!C || (K > 0 && (!A || !B))) { set_error("%s: NULL operand", who); return CN_ERR_NULL; }
+    if ((M == 0 || N == 0) && !absmax_out) return CN_OK;
+    if ((M > 0 && N > 0) && (!C || (K > 0 && (!A || !B)))) { set_error("%s: NULL operand", who); return CN_ERR_NULL; }
     Context *ctx;
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
+    // The maximum is accumulated with atomics from +0.0 (|C| >= 0); an empty C reports -1.0f, the start
+    // value of the reference's reduction, like cn_absmax_f32.
+    uint32_t *amax = reinterpret_cast<uint32_t *>(absmax_out);
+    if (amax) {
+        hipLaunchKernelGGL(set_word_kernel, dim3(1), dim3(64), 0, st, amax, (M == 0 || N == 0) ? 0xbf800000u : 0u);
+        CN_HIP(hipGetLastError());
+    }
+    if (M == 0 || N == 0) return CN_OK;
     if (K == 0) {
         hipLaunchKernelGGL(zero_matrix_kernel, dim3(ctx->num_cu * 4), dim3(256), 0, st, C, M, N, ldc);
         CN_HIP(hipGetLastError());
@@ -591,6 +632,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.vec_a = aligned(A, 16) && (lda % 4 == 0);
     a.vec_b = w8 ? (aligned(B, 4) && (ldb % 4 == 0)) : (aligned(B, 16) && (ldb % 4 == 0));
     a.scale = scale; a.table = ctx->table;
+    a.amax = amax;
 
     if (w8)              s = launch<true, B_CODES>(a, plan.tile_n, st);
     else if (!ta && !tb) s = launch<true, B_IC>(a, plan.tile_n, st);
@@ -605,7 +647,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         int64_t blocks = (work + 255) / 256;
         int64_t cap = (int64_t)ctx->num_cu * 8;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, st,
-                           (const float *)ctx->workspace, plan.splits, M, N, C, ldc, vec);
+                           (const float *)ctx->workspace, plan.splits, M, N, C, ldc, vec, amax);
         CN_HIP(hipGetLastError());
     }
     return CN_OK;
@@ -622,12 +664,19 @@ void cn_host_force_gemm_tile_n(int tile_n) { g_force_tile_n = (tile_n == 128 || 
 
 cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                       const float *B, int64_t ldb, float *C, int64_t ldc, void *stream) {
-    return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, C, ldc, stream);
+    return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, C, ldc, nullptr, stream);
+}
+
+cn_status cn_gemm_f32_absmax(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A,
+                             int64_t lda, const float *B, int64_t ldb, float *C, int64_t ldc, float *absmax_out,
+                             void *stream) {
+    if (!absmax_out) { set_error("gemm_f32_absmax: NULL output for the maximum"); return CN_ERR_NULL; }
+    return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, C, ldc, absmax_out, stream);
 }
 
 cn_status cn_gemm_f32_w8(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W,
                          int64_t ldw, float scale, float *C, int64_t ldc, void *stream) {
-    return gemm_impl(0, 0, true, M, N, K, A, lda, W, ldw, scale, C, ldc, stream);
+    return gemm_impl(0, 0, true, M, N, K, A, lda, W, ldw, scale, C, ldc, nullptr, stream);
 }
 
 }  // extern "C"

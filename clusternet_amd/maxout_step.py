@@ -24,15 +24,18 @@ def forward(X, params, pool=2):
     return p, (h1, a1, h2, a2)
 
 
-def backward(X, onehot, params, p, cache, pool=2):
+def backward(X, onehot, params, p, cache, pool=2, absmax_out=None):
+    """Weight gradients.  `absmax_out` = three one-element device tensors: the gradient products then
+    also deliver max|gW|, which saves the abs-max pass in front of compression_8bit."""
     W1, b1, W2, b2, W3, b3 = params
     h1, a1, h2, a2 = cache
+    m1, m2, m3 = absmax_out if absmax_out is not None else (None, None, None)
     e3 = L.sub(p, onehot)
-    gW3 = L.Tdot(h2, e3)
+    gW3 = L.Tdot(h2, e3, absmax_out=m3)
     e2 = L.expand_to_maxout_grad(L.dotT(e3, W3), a2, pool)
-    gW2 = L.Tdot(h1, e2)
+    gW2 = L.Tdot(h1, e2, absmax_out=m2)
     e1 = L.expand_to_maxout_grad(L.dotT(e2, W2), a1, pool)
-    gW1 = L.Tdot(X, e1)
+    gW1 = L.Tdot(X, e1, absmax_out=m1)
     return gW1, gW2, gW3
 
 
@@ -43,10 +46,12 @@ def codec_round_trip(grad):
     return L.decompression_8bit(codes, prec, out=grad), codes, prec
 
 
-def coded_update(w, grad, rate, fused=True, scratch=None):
+def coded_update(w, grad, rate, fused=True, scratch=None, prec=None):
     """W -= rate * decode(encode(grad)).  `fused` picks the one-pass kernel; the unfused sequence
-    (decompression_8bit into `scratch`, or over `grad` itself, then the update) gives the same bits."""
-    prec = L.absmax(grad)
+    (decompression_8bit into `scratch`, or over `grad` itself, then the update) gives the same bits.
+    `prec` = max|grad| on the device if the caller already has it."""
+    if prec is None:
+        prec = L.absmax(grad)
     codes = L.compression_8bit(grad, prec)
     if fused:
         L.decompression_8bit_axpy(codes, prec, -rate, w)
@@ -68,9 +73,11 @@ def coded_rmsprop_update(w, rms, grad, rms_multiplier, rate, fused=True, scratch
 
 
 def step(X, onehot, params, rate, pool=2):
+    import torch
     p, cache = forward(X, params, pool)
-    grads = backward(X, onehot, params, p, cache, pool)
+    maxima = [torch.empty(1, dtype=torch.float32, device=X.device) for _ in range(3)]
+    grads = backward(X, onehot, params, p, cache, pool, absmax_out=maxima)
     W = (params[0], params[2], params[4])
-    for w, g in zip(W, grads):
-        coded_update(w, g, rate)
+    for w, g, m in zip(W, grads, maxima):
+        coded_update(w, g, rate, prec=m)
     return p

@@ -76,6 +76,15 @@ cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
                       const float *A_device, int64_t lda, const float *B_device, int64_t ldb,
                       float *C_device, int64_t ldc, void *stream);
 
+/* cn_gemm_f32 that also writes max |C[i][j]| to *absmax_out_device, taken in the kernel's write-out
+ * (or in the addition of the K chunks): the value equals cn_absmax_f32 over the result bit for bit
+ * (-1.0f for an empty C) and saves that pass over C.  It fuses dot / Tdot with the max(abs(grad)) that
+ * precedes every compression_8bit of a gradient (source/DeepNeuralNetwork.cpp:334-337,
+ * source/basicOps.cu:810-822,1076-1081). */
+cn_status cn_gemm_f32_absmax(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
+                             const float *A_device, int64_t lda, const float *B_device, int64_t ldb,
+                             float *C_device, int64_t ldc, float *absmax_out_device, void *stream);
+
 /* C[M x N] = A[M x K] decode(W[K x N], scale): W holds 8-bit codes (row-major, ldw >= N) that are
  * expanded inside the kernel with exactly the table of cn_decompress_8bit(scale).  No counterpart
  * in the reference; its relatives are dot8bit / dot8bit_shared (source/clusterNet.cpp:1409-1431,

@@ -253,3 +253,42 @@ def test_fused_w8_ragged(dev, shape):
     Cref, Cabs = oracle.gemm_with_abs(A, oracle.decompress(W, 0.25))
     e1, e2 = gemm_errors(got, Cref, Cabs)
     assert e1 <= 1e-4 and e2 <= 1e-4, (e1, e2)
+
+
+@pytest.mark.parametrize("shape,ta,tb", [((128, 300, 64), False, False), ((1000, 257, 128), True, False),
+                                          ((37, 1029, 515), False, True), ((128, 512, 8192), False, False),
+                                          ((3, 5, 7), True, True), ((64, 64, 1), False, False)])
+def test_gemm_with_absmax_output(dev, shape, ta, tb):
+    """The maximum delivered by the product's write-out (or by the addition of K chunks) equals the
+    stand-alone abs-max kernel over the result bit for bit, and the product itself is unchanged."""
+    import torch
+    import clusternet_amd as cn
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N)
+    A = rng.normal(0, 1, (K, M) if ta else (M, K)).astype(np.float32)
+    B = rng.normal(0, 0.05, (N, K) if tb else (K, N)).astype(np.float32)
+    At, Bt = _t(A, dev), _t(B, dev)
+    plain = cn.gemm(At, Bt, ta, tb)
+    m = torch.full((1,), 123.0, device=dev)
+    fused = cn.gemm(At, Bt, ta, tb, absmax_out=m)
+    assert torch.equal(plain.view(torch.int32), fused.view(torch.int32))
+    want = cn.absmax(plain)
+    assert torch.equal(m.view(torch.int32), want.view(torch.int32)), (float(m), float(want))
+    assert float(m) == float(np.abs(plain.cpu().numpy()).max()) if plain.numel() else True
+
+
+def test_gemm_with_absmax_output_strided_and_empty(dev):
+    import torch
+    import clusternet_amd as cn
+    L = cn.lib()
+    rng = np.random.default_rng(4)
+    A = _t(rng.normal(0, 1, (128, 96)).astype(np.float32), dev)
+    B = _t(rng.normal(0, 1, (96, 200)).astype(np.float32), dev)
+    big = torch.full((128, 256), 1e9, device=dev)      # columns 200.. must not enter the maximum
+    m = torch.empty(1, device=dev)
+    cn.gemm(A, B, False, False, out=big[:, :200], absmax_out=m)
+    assert float(m) == float(big[:, :200].abs().max()) and float(big[0, 200]) == 1e9
+    assert L.cn_gemm_f32_absmax(0, 0, 0, 5, 3, None, 3, None, 5, None, 5, m.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    assert float(m) == -1.0
+    assert L.cn_gemm_f32_absmax(0, 0, 4, 4, 4, A.data_ptr(), 96, B.data_ptr(), 200, big.data_ptr(), 256, None, None) == 1
