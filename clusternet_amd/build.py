@@ -68,7 +68,7 @@ def build_facade(verbose=False):
     cxx = shutil.which("g++") or "g++"
     inc = ["-I" + os.path.join(ROOT, "include"), "-I" + FACADE]
     _run([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-o", FACADE_LIB, src,
-          os.path.join(FACADE, "basicOps.cpp")] + inc +
+          os.path.join(FACADE, "basicOps.cpp"), os.path.join(FACADE, "util.cpp")] + inc +
          ["-L" + HERE, "-lcnhip", "-Wl,-rpath,$ORIGIN"])
     test_src = os.path.join(ROOT, "tests", "cpp", "facade_test.cpp")
     oracle_dir = os.path.join(ROOT, "oracle")

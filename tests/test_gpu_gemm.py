@@ -94,6 +94,26 @@ def test_config1_mlp_layer(dev):
     assert E.shape == (128, 784)
 
 
+def test_config1_on_the_reference_mnist_batch(dev):
+    """First layer of the reference's MNIST network on its own data file (tests/mnist_mini_X.hdf5 of
+    the reference, 500 x 784 fp32 at byte 2144): real pixel rows are mostly exact zeros with runs of
+    values in (0, 1], unlike the synthetic uniform batch."""
+    import os
+    import clusternet_amd as cn
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "hdf5", "mnist_mini_X.hdf5")
+    X = np.fromfile(path, dtype=np.float32, offset=2144, count=500 * 784).reshape(500, 784)
+    rng = np.random.default_rng(6)
+    lim = np.sqrt(6.0 / (784 + 1024))
+    W = rng.uniform(-lim, lim, (784, 1024)).astype(np.float32)
+    for lo in (0, 128, 372):                       # 372: the last, 128-row batch of the 500
+        A = X[lo:lo + 128]
+        C = _check(cn, dev, A, W)
+        dC = (C * 0.01).astype(np.float32)
+        _check(cn, dev, A, dC, ta=True)            # Tdot -> 784 x 1024
+        _check(cn, dev, dC, W, tb=True)            # dotT -> 128 x 784
+    _check(cn, dev, X, W)                          # all 500 rows: ragged in M
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (2, 2, 3), (128, 128, 32), (129, 130, 33),
                                    (64, 200, 31), (257, 100, 64), (100, 10, 4096), (200, 300, 1000),
                                    (128, 512, 8192), (37, 1029, 515), (1000, 4, 128)])
