@@ -57,8 +57,7 @@ def lib():
     L.cn_rmsprop_update_f32.argtypes = [vp, vp, vp, f32, f32, sz, vp]
     L.cn_rmsprop_update_w8.argtypes = [vp, vp, f32, vp, f32, f32, sz, vp]
     L.cn_rmsprop_update_w8_dp.argtypes = [vp, vp, vp, vp, f32, f32, sz, vp]
-    L.cn_host_encode_lut_lookup.argtypes = [C.c_uint32, C.POINTER(C.c_int)]
-    L.cn_host_encode_magnitude.argtypes = [f32]
+    L.cn_host_encode_exact.argtypes = [f32, f32]
     L.cn_host_plan_gemm.argtypes = [i64, i64, i64, C.c_int, sz, C.c_int, C.POINTER(i64)]
     L.cn_host_plan_gemm.restype = None
     L.cn_host_force_gemm_tile_n.argtypes = [C.c_int]

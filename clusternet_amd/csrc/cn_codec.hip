@@ -5,91 +5,68 @@
 // Each lane moves 16-byte vectors laid out so that one wavefront instruction touches one
 // contiguous 1 KiB (fp32 side) / 256 B (code side) span.
 #include "cn_internal.h"
+#include "cn_xlut.h"
 
 namespace cn {
 
 constexpr int kThreads = 256;
 constexpr int kVecPerThread = 4;                         // float4 per lane per tile
 constexpr int kTileVec = kThreads * kVecPerThread;       // float4 per workgroup tile (4096 floats)
-constexpr uint32_t kLutCapacity = (127 - 107 + 1) * (1 << kMantBits) + 2;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// ---- exact encoder: the reference procedure, element by element --------------------------------
-// Follows kCompression_8bit (source/clusterKernels.cu:1163-1232): IEEE division, sign split,
-// two threshold exits, 6-step pivot search over the table, two-candidate pick.  `slot` is the
-// 128-entry LDS copy of the table whose entry 126 holds 1.0f.
-__device__ __forceinline__ uint32_t encode_exact(float x, float precision, const float *slot) {
-    float a = x / precision;
-    uint32_t neg = 0;
-    if (a < 0.0f) { neg = 0x80u; a = -a; }
-    if (a < 0.0000015f) return 254u;
-    if (a > 0.995703f) return 127u | neg;
-    int lo = 0, hi = 125, p = 63;
-#pragma unroll
-    for (int step = 32; step > 0; step >>= 1) {
-        if (a > slot[p]) { lo = p; p += step; }
-        else             { hi = p; p -= step; }
-    }
-    int c;
-    if (lo == p) c = (fabsf(slot[p] - a) < (slot[hi] - a)) ? p : hi;
-    else         c = ((slot[p] - a) < fabsf(slot[lo] - a)) ? p : lo;
-    return (uint32_t)c | neg;
+// ---- encoder ---------------------------------------------------------------------------------------
+// compression_8bit is two launches: a 20-workgroup kernel that derives the table of cn_xlut.h for the
+// call's precision from the literal procedure, and the streaming kernel that looks every element up
+// in an LDS copy of it (shift, clamp, one 8-byte LDS read, one compare, one byte select).
+
+// One thread per table entry.  flags[block] != 0 tells the encoder not to trust the table.
+__global__ __launch_bounds__(kThreads) void build_xlut_kernel(float precision_value,
+                                                              const float *__restrict__ precision_ptr,
+                                                              const float *__restrict__ table,
+                                                              XEntry *__restrict__ out, uint32_t *__restrict__ flags) {
+    __shared__ float slot[128];
+    if (threadIdx.x < 126) slot[threadIdx.x] = table[threadIdx.x];
+    if (threadIdx.x == 126) slot[126] = 1.0f;
+    if (threadIdx.x == 127) slot[127] = 0.0f;
+    __syncthreads();
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    bool unusable = false;
+    if (i < kXEntries) out[i] = xlut_entry(i, precision, slot, &unusable);
+    const int any = __syncthreads_or(unusable ? 1 : 0);
+    if (threadIdx.x == 0) flags[blockIdx.x] = (uint32_t)any;
 }
+constexpr int kXBuildBlocks = (kXEntries + kThreads - 1) / kThreads;
 
 struct EncodeShared {
-    EncodeBucket lut[kLutCapacity];
+    XEntry lut[kXEntries];
     float slot[128];
 };
-
-__device__ __forceinline__ void stage_encoder(EncodeShared &sh, const EncodeBucket *lut,
-                                              uint32_t lut_count, const float *table) {
-    const uint2 *src = reinterpret_cast<const uint2 *>(lut);
-    uint2 *dst = reinterpret_cast<uint2 *>(sh.lut);
-    for (uint32_t i = threadIdx.x; i < lut_count; i += blockDim.x) dst[i] = src[i];
-    if (threadIdx.x < 126) sh.slot[threadIdx.x] = table[threadIdx.x];
-    if (threadIdx.x == 126) sh.slot[126] = 1.0f;
-    if (threadIdx.x == 127) sh.slot[127] = 0.0f;
-    __syncthreads();
-}
-
-// Fast path for one element: approximate quotient x * (1/precision), bucket lookup, one compare.
-// The approximate quotient is within kGuard bit patterns of the correctly rounded one; `near`
-// collects whether any element sits within kGuard of its bucket's boundary, in which case the
-// caller recomputes with encode_exact.
-__device__ __forceinline__ uint32_t encode_fast(float x, float recip, const EncodeBucket *lut,
-                                                uint32_t first, uint32_t last, uint32_t &near,
-                                                uint32_t &magmax) {
-    float a0 = x * recip;
-    uint32_t bits = __float_as_uint(a0);
-    uint32_t mag = bits & 0x7fffffffu;
-    magmax = max(magmax, mag);
-    uint32_t b = min(max(mag >> kBucketShift, first), last) - first;
-    EncodeBucket e = lut[b];
-    int32_t d = (int32_t)(mag - e.boundary_minus_guard);
-    near |= ((uint32_t)d <= 2u * kGuard) ? 1u : 0u;
-    uint32_t c = (d >= (int32_t)kGuard) ? (e.codes >> 8) : e.codes;
-    return (c & 0xffu) | ((bits >> 24) & 0x80u);
-}
-
-// The approximation x * (1/p) is trusted only when 1/p is a normal number with full precision.
-__device__ __forceinline__ bool precision_allows_fast_path(float p) {
-    float ap = fabsf(p);
-    return ap >= 8.67361738e-19f /* 2^-60 */ && ap <= 1.15292150e18f /* 2^60 */;
-}
 
 template <bool kVector>
 __global__ __launch_bounds__(kThreads) void compress_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr,
-    size_t n, uint8_t *__restrict__ codes, const EncodeBucket *__restrict__ lut,
-    uint32_t lut_first, uint32_t lut_count, const float *__restrict__ table) {
-    __shared__ EncodeShared sh;
-    stage_encoder(sh, lut, lut_count, table);
+    size_t n, uint8_t *__restrict__ codes, const XEntry *__restrict__ xlut,
+    const uint32_t *__restrict__ xflags, const float *__restrict__ table) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    {
+        const uint2 *src = reinterpret_cast<const uint2 *>(xlut);
+        uint2 *dst = reinterpret_cast<uint2 *>(sh.lut);
+        for (int i = threadIdx.x; i < kXEntries; i += kThreads) dst[i] = src[i];
+        if (threadIdx.x < 126) sh.slot[threadIdx.x] = table[threadIdx.x];
+        if (threadIdx.x == 126) sh.slot[126] = 1.0f;
+        if (threadIdx.x == 127) sh.slot[127] = 0.0f;
+    }
+    const bool exact_only = __syncthreads_or((threadIdx.x < kXBuildBlocks && xflags[threadIdx.x] != 0) ? 1 : 0) != 0;
     const float precision = precision_ptr ? *precision_ptr : precision_value;
-    const bool fast_ok = precision_allows_fast_path(precision);
-    const float recip = 1.0f / precision;
-    const uint32_t first = lut_first, last = lut_first + lut_count - 1;
+    const uint32_t first = xlut_first(precision);
+    auto encode = [&](float v) -> uint32_t {
+        const uint32_t bits = __float_as_uint(v);
+        return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
+    };
 
     if (kVector) {
         const size_t nvec = n / 4;
@@ -107,24 +84,16 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
         auto encode_tile = [&](size_t tile, const f32x4 (&v)[kVecPerThread]) {
             const size_t base = tile * kTileVec + threadIdx.x;
             uint32_t packed[kVecPerThread];
-            uint32_t near = 0, magmax = 0;
+            if (!exact_only) {
 #pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
-                uint32_t c0 = encode_fast(v[j].x, recip, sh.lut, first, last, near, magmax);
-                uint32_t c1 = encode_fast(v[j].y, recip, sh.lut, first, last, near, magmax);
-                uint32_t c2 = encode_fast(v[j].z, recip, sh.lut, first, last, near, magmax);
-                uint32_t c3 = encode_fast(v[j].w, recip, sh.lut, first, last, near, magmax);
-                packed[j] = c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
-            }
-            if (!fast_ok || near != 0 || magmax > 0x7f800000u) {
+                for (int j = 0; j < kVecPerThread; ++j)
+                    packed[j] = encode(v[j].x) | (encode(v[j].y) << 8) | (encode(v[j].z) << 16) | (encode(v[j].w) << 24);
+            } else {
 #pragma unroll
-                for (int j = 0; j < kVecPerThread; ++j) {
-                    uint32_t c0 = encode_exact(v[j].x, precision, sh.slot);
-                    uint32_t c1 = encode_exact(v[j].y, precision, sh.slot);
-                    uint32_t c2 = encode_exact(v[j].z, precision, sh.slot);
-                    uint32_t c3 = encode_exact(v[j].w, precision, sh.slot);
-                    packed[j] = c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
-                }
+                for (int j = 0; j < kVecPerThread; ++j)
+                    packed[j] = encode_exact(v[j].x, precision, sh.slot) | (encode_exact(v[j].y, precision, sh.slot) << 8) |
+                                (encode_exact(v[j].z, precision, sh.slot) << 16) |
+                                (encode_exact(v[j].w, precision, sh.slot) << 24);
             }
 #pragma unroll
             for (int j = 0; j < kVecPerThread; ++j) {
@@ -152,11 +121,11 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
         // ragged tail (n % 4 elements)
         if (blockIdx.x == 0) {
             size_t i = nvec * 4 + threadIdx.x;
-            if (i < n) codes[i] = (uint8_t)encode_exact(x[i], precision, sh.slot);
+            if (i < n) codes[i] = (uint8_t)(exact_only ? encode_exact(x[i], precision, sh.slot) : encode(x[i]));
         }
     } else {
         for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
-            codes[i] = (uint8_t)encode_exact(x[i], precision, sh.slot);
+            codes[i] = (uint8_t)(exact_only ? encode_exact(x[i], precision, sh.slot) : encode(x[i]));
     }
 }
 
@@ -338,15 +307,26 @@ static cn_status compress_impl(const float *x, float precision, const float *pre
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(build_xlut_kernel, dim3(kXBuildBlocks), dim3(kThreads), 0, st, precision, precision_dev,
+                       ctx->table, ctx->xlut, ctx->xflags);
+    CN_HIP(hipGetLastError());
     // two workgroups per CU: mixed read/write streams run fastest on this part with few wavefronts
     // in flight, and the kernel keeps its own next tile in flight to stay busy at that occupancy
     int grid = stream_grid(ctx, n, 2);
+    static bool configured = false;
+    if (!configured) {
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
+        configured = true;
+    }
     if (aligned(x, 16) && aligned(codes, 4))
-        hipLaunchKernelGGL(compress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, x, precision,
-                           precision_dev, n, codes, ctx->encode_lut, ctx->lut_first, ctx->lut_count, ctx->table);
+        hipLaunchKernelGGL(compress_kernel<true>, dim3(grid), dim3(kThreads), sizeof(EncodeShared), st, x, precision,
+                           precision_dev, n, codes, ctx->xlut, ctx->xflags, ctx->table);
     else
-        hipLaunchKernelGGL(compress_kernel<false>, dim3(grid), dim3(kThreads), 0, st, x, precision,
-                           precision_dev, n, codes, ctx->encode_lut, ctx->lut_first, ctx->lut_count, ctx->table);
+        hipLaunchKernelGGL(compress_kernel<false>, dim3(grid), dim3(kThreads), sizeof(EncodeShared), st, x, precision,
+                           precision_dev, n, codes, ctx->xlut, ctx->xflags, ctx->table);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

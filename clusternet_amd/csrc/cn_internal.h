@@ -19,30 +19,8 @@ cn_status hip_fail(hipError_t e, const char *what, const char *file, int line);
         if (cn_e_ != hipSuccess) return cn::hip_fail(cn_e_, #call, __FILE__, __LINE__); \
     } while (0)
 
-// ---- encoder bucket table --------------------------------------------------------------------
-// The encoder maps |x / precision| to a code through a direct-indexed table over the leading bits
-// of the fp32 pattern.  Each bucket holds at most one code boundary.
-constexpr int kMantBits = 7;                       // mantissa bits used for the bucket index
-constexpr int kBucketShift = 23 - kMantBits;       // pattern >> shift = bucket number
-constexpr uint32_t kGuard = 6;                     // |approx - exact| quotient distance bound, in ulps
-constexpr uint32_t kNoBoundary = 0x7ffffff0u;
-
-struct EncodeBucket {
-    uint32_t boundary_minus_guard;  // first pattern that takes `above`, minus kGuard
-    uint32_t codes;                 // below | (above << 8), magnitude codes without the sign bit
-};
-
-struct EncodeLut {
-    uint32_t first_bucket;  // bucket number of entry 0
-    uint32_t count;         // number of entries (last one = everything above the saturation bound)
-    EncodeBucket entry[(127 - 107 + 1) * (1 << kMantBits) + 2];
-};
-
-// Magnitude code (0..127, 254) of a non-negative, non-NaN scaled magnitude by the reference
-// procedure; host-side evaluator used to derive the bucket table.
-uint8_t host_encode_magnitude(float a);
-// Fills `lut`; returns false (with set_error) if some bucket would need two boundaries.
-bool build_encode_lut(EncodeLut *lut);
+// The 126-entry codebook (exact bit patterns of the reference's table file).
+void host_table(float out[126]);
 
 // ---- per-device state ------------------------------------------------------------------------
 struct Context {
@@ -50,8 +28,8 @@ struct Context {
     int device = -1;
     int num_cu = 0;
     float *table = nullptr;          // 126 floats
-    EncodeBucket *encode_lut = nullptr;
-    uint32_t lut_first = 0, lut_count = 0;
+    struct XEntry *xlut = nullptr;   // encoder table of the compression call in flight (cn_xlut.h)
+    uint32_t *xflags = nullptr;      // its "do not trust" flags, one per build workgroup
     void *workspace = nullptr;       // split-K partial sums
     size_t workspace_bytes = 0;
     uint32_t *reduce_scratch = nullptr;  // per-workgroup partial maxima + ticket counters

@@ -7,6 +7,7 @@
 #include <mutex>
 
 #include "cn_internal.h"
+#include "cn_xlut.h"
 
 namespace cn {
 
@@ -57,12 +58,8 @@ static cn_status init_device(int device) {
     CN_HIP(hipMalloc((void **)&c.table, sizeof(table)));
     CN_HIP(hipMemcpy(c.table, table, sizeof(table), hipMemcpyHostToDevice));
 
-    static EncodeLut lut;
-    if (!build_encode_lut(&lut)) return CN_ERR_ARG;
-    c.lut_first = lut.first_bucket;
-    c.lut_count = lut.count;
-    CN_HIP(hipMalloc((void **)&c.encode_lut, lut.count * sizeof(EncodeBucket)));
-    CN_HIP(hipMemcpy(c.encode_lut, lut.entry, lut.count * sizeof(EncodeBucket), hipMemcpyHostToDevice));
+    CN_HIP(hipMalloc((void **)&c.xlut, (size_t)kXEntries * sizeof(XEntry)));
+    CN_HIP(hipMalloc((void **)&c.xflags, 64 * sizeof(uint32_t)));
 
     size_t mib = 1024;
     if (const char *env = getenv("CNHIP_WORKSPACE_MB")) {
@@ -137,7 +134,8 @@ cn_status cn_shutdown(void) {
         CN_HIP(hipSetDevice(d));
         CN_HIP(hipDeviceSynchronize());
         CN_HIP(hipFree(c.table));
-        CN_HIP(hipFree(c.encode_lut));
+        CN_HIP(hipFree(c.xlut));
+        CN_HIP(hipFree(c.xflags));
         CN_HIP(hipFree(c.workspace));
         CN_HIP(hipFree(c.reduce_scratch));
         CN_HIP(hipFree(c.sum_scratch));

@@ -45,55 +45,89 @@ def test_product_table_equals_fixture():
     assert cn.table().tobytes() == raw
 
 
-def _lookup(mags):
+def _encode_host(x, precision):
+    """The encoder as the device runs it (per-call table, or the literal procedure where the table
+    reports itself unusable), evaluated by the library's host build."""
     L = cn.lib()
-    mags = np.ascontiguousarray(mags, np.uint32)
-    codes = np.empty(mags.size, np.uint8)
-    near = np.empty(mags.size, np.uint8)
-    L.cn_host_encode_lut_lookup_many.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
-    assert L.cn_host_encode_lut_lookup_many(mags.ctypes.data, mags.size, codes.ctypes.data, near.ctypes.data) == 0
-    return codes, near
+    x = np.ascontiguousarray(x, np.float32)
+    codes = np.empty(x.size, np.uint8)
+    L.cn_host_xlut_encode_many.argtypes = [C.c_float, C.c_void_p, C.c_size_t, C.c_void_p]
+    used_table = L.cn_host_xlut_encode_many(float(precision), x.ctypes.data, x.size, codes.ctypes.data)
+    return codes, bool(used_table)
 
 
-def test_bucket_table_exhaustive_over_all_patterns_in_range():
+def test_encoder_table_exhaustive_at_precision_one():
+    """Every fp32 pattern from 1e-6 to 1.01 and, sparsely strided, from 0 to NaN, both signs."""
     lo = int(np.array([1.0e-6], np.float32).view(np.uint32)[0])
     hi = int(np.array([1.01], np.float32).view(np.uint32)[0])
     step = 1 << 24
     for start in range(lo, hi, step):
         mags = np.arange(start, min(start + step, hi), dtype=np.uint32)
-        codes, _ = _lookup(mags)
-        want = oracle.compress(mags.view(np.float32), 1.0, 0)
-        assert np.array_equal(codes, want), hex(start)
-    # far outside the table: zero code below, saturation above (including infinity)
-    far = np.array([0, 1, 0x00800000, lo - 1, hi + 5, 0x7f000000, 0x7f800000], np.uint32)
-    codes, _ = _lookup(far)
-    assert codes.tolist() == [254, 254, 254, 254, 127, 127, 127]
+        for sign in (0, 0x80000000):
+            x = (mags | np.uint32(sign)).view(np.float32)
+            codes, used = _encode_host(x, 1.0)
+            assert used
+            assert np.array_equal(codes, oracle.port_compress(x, 1.0)), (hex(start), sign)
+    with np.errstate(all="ignore"):
+        sweep = np.arange(0, 1 << 32, 4099, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        codes, used = _encode_host(sweep, 1.0)
+        assert used and np.array_equal(codes, oracle.compress(sweep, 1.0, 0))
+    far = np.array([0, 1, 0x00800000, lo - 1, hi + 5, 0x7f000000, 0x7f800000, 0x7f800001, 0x7fc00000,
+                    0x80000000, 0xff800000, 0xffc00000], np.uint32).view(np.float32)
+    codes, _ = _encode_host(far, 1.0)
+    assert codes.tolist() == [254, 254, 254, 254, 127, 127, 127, 1, 1, 254, 255, 1]
 
 
-def test_fast_path_is_exact_wherever_it_is_trusted():
-    """x * (1/p) stands in for x / p; wherever the table does not flag the element as near a
-    boundary the code must equal the reference procedure's on the exact quotient."""
+def test_encoder_table_over_precisions_and_step_neighbourhoods():
+    """For ordinary, negative, tiny, huge and degenerate precisions: random inputs over the whole
+    coded range, every pattern within 40 ulps of every step of the code function, and a strided
+    sweep over all bit patterns.  Where the table is trusted it must equal the literal procedure;
+    where it is not, the encoder must say so (and then runs the literal procedure itself)."""
     rng = np.random.default_rng(123)
     t = oracle.table()
     edges = np.concatenate([t, (t[:-1] + t[1:]) / 2, [1.5e-6, 0.995703, 1.0]]).astype(np.float32)
-    trusted = 0
-    for p in [1.0, 0.1, 0.0234375, 3.0, 1e-5, 7.7e4] + list(rng.uniform(1e-3, 10, 6)):
-        p = np.float32(p)
-        r = np.float32(1.0) / p
-        x = np.concatenate([
-            np.exp(rng.uniform(np.log(1e-7), np.log(1.5), 400_000)).astype(np.float32) * p,
-            # inputs whose quotient sits within a few ulps of every boundary candidate
-            (np.repeat(edges, 41).view(np.uint32).astype(np.int64)
-             + np.tile(np.arange(-20, 21), edges.size)).astype(np.uint32).view(np.float32) * p,
-        ]).astype(np.float32)
-        a0 = (x * r).astype(np.float32)
-        codes, near = _lookup(a0.view(np.uint32) & np.uint32(0x7fffffff))
-        want = oracle.compress(x, float(p), 0)
-        ok = near == 0
-        assert np.array_equal(codes[ok], want[ok]), float(p)
-        trusted += int(ok.sum())
-        assert near.mean() < 0.02
-    assert trusted > 1_000_000
+    trusted_precisions = 0
+    with np.errstate(all="ignore"):
+        sweep = np.arange(0, 1 << 32, 16411, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        precisions = [1.0, 0.1, 0.0234375, 3.0, 1e-5, 7.7e4, -1.0, -0.37, 2.0 ** -60, 2.0 ** 60, 1e-30, 1e30,
+                      3e38, 1.2e-38, 1e-42, 0.0, -0.0, float("inf"), float("-inf"), float("nan")]
+        precisions += list(rng.uniform(1e-3, 10, 6))
+        for p in precisions:
+            p32 = np.float32(p)
+            scale = p32 if np.isfinite(p32) and p32 != 0 else np.float32(1.0)
+            near = (np.repeat(edges, 81).view(np.uint32).astype(np.int64)
+                    + np.tile(np.arange(-40, 41), edges.size)).astype(np.uint32).view(np.float32)
+            x = np.concatenate([
+                np.exp(rng.uniform(np.log(1e-7), np.log(1.5), 200_000)).astype(np.float32) * scale,
+                -np.exp(rng.uniform(np.log(1e-7), np.log(1.5), 50_000)).astype(np.float32) * scale,
+                near * scale, -near * scale, sweep,
+            ]).astype(np.float32)
+            codes, used = _encode_host(x, p)
+            want = oracle.compress(x, float(p), 0)
+            bad = np.nonzero(codes != want)[0]
+            assert bad.size == 0, (p, used, x[bad[:4]], codes[bad[:4]], want[bad[:4]])
+            trusted_precisions += int(used)
+            if np.isfinite(p32) and 1e-30 <= abs(float(p32)) <= 1e30:
+                assert used, p          # the table serves every precision a gradient can have
+    assert trusted_precisions >= 18
+
+
+def test_encoder_table_shape():
+    L = cn.lib()
+    n = L.cn_host_xlut_entries()
+    entries = np.zeros((n, 2), np.uint32)
+    first = C.c_uint32()
+    L.cn_host_xlut_build.argtypes = [C.c_float, C.c_void_p, C.POINTER(C.c_uint32)]
+    assert L.cn_host_xlut_build(1.0, entries.ctypes.data, C.byref(first)) == 0
+    assert n * 8 <= 48 * 1024                                  # two workgroups per CU keep it in LDS
+    codes = entries[1:-1, 1]
+    below, above = codes & 0xff, (codes >> 8) & 0xff
+    steps = int((below != above).sum())
+    assert 100 <= steps <= 260                                 # 254 -> 0 -> ... -> 125 -> 127 (a few codes never occur)
+    assert entries[0, 1] == 0xfefefefe and (entries[-1, 1] & 0xff) == 127
+    # negative side: same steps, sign bit on every code but 254
+    nb, pb = (codes >> 16) & 0xff, below
+    assert np.all(np.where(pb == 254, nb == 254, nb == (pb | 0x80)))
 
 
 def test_gemm_plan_covers_k_and_fits_workspace():
