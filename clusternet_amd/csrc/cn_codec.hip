@@ -17,51 +17,78 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // ---- encoder ---------------------------------------------------------------------------------------
-// compression_8bit is two launches: a 20-workgroup kernel that derives the table of cn_xlut.h for the
-// call's precision from the literal procedure, and the streaming kernel that looks every element up
-// in an LDS copy of it (shift, clamp, one 8-byte LDS read, one compare, one byte select).
-
-// One thread per table entry.  flags[block] != 0 tells the encoder not to trust the table.
-__global__ __launch_bounds__(kThreads) void build_xlut_kernel(float precision_value,
-                                                              const float *__restrict__ precision_ptr,
-                                                              const float *__restrict__ table,
-                                                              XEntry *__restrict__ out, uint32_t *__restrict__ flags) {
-    __shared__ float slot[128];
-    if (threadIdx.x < 126) slot[threadIdx.x] = table[threadIdx.x];
-    if (threadIdx.x == 126) slot[126] = 1.0f;
-    if (threadIdx.x == 127) slot[127] = 0.0f;
-    __syncthreads();
-    const float precision = precision_ptr ? *precision_ptr : precision_value;
-    const int i = blockIdx.x * kThreads + threadIdx.x;
-    bool unusable = false;
-    if (i < kXEntries) out[i] = xlut_entry(i, precision, slot, &unusable);
-    const int any = __syncthreads_or(unusable ? 1 : 0);
-    if (threadIdx.x == 0) flags[blockIdx.x] = (uint32_t)any;
-}
-constexpr int kXBuildBlocks = (kXEntries + kThreads - 1) / kThreads;
+// Every workgroup builds the table of cn_xlut.h for the call's precision in LDS (one thread per step
+// of the code function: nine evaluations of the literal procedure and a run of LDS stores), then
+// looks every element up: shift, clamp, one 8-byte LDS read, one compare, one byte select.
 
 struct EncodeShared {
     XEntry lut[kXEntries];
     float slot[128];
+    int step_index[kXMaxSteps];
+    XEntry step_entry[kXMaxSteps];
 };
+
+// Returns true when the table in sh.lut may be used.
+__device__ __forceinline__ bool build_table(EncodeShared &sh, const XStep *__restrict__ steps, int count,
+                                            float precision, const float *__restrict__ table) {
+    const int t = threadIdx.x;
+    if (t < 126) sh.slot[t] = table[t];
+    if (t == 126) sh.slot[126] = 1.0f;
+    if (t == 127) sh.slot[127] = 0.0f;
+    __syncthreads();
+    const uint32_t first = xlut_first(precision);
+    bool bad = false;
+    XEntry e{};
+    int index = 0;
+    if (t < count) {
+        bad = !xlut_locate_step(steps[t], precision, sh.slot, &e);
+        index = (int)(e.boundary >> kXShift) - (int)first + 1;
+        if (bad || index < 1 || index > kXBuckets) { bad = true; index = 0; }
+        sh.step_index[t] = index;
+    } else if (t == count) {
+        sh.lut[0] = xlut_entry(0, precision, sh.slot, &bad);
+    } else if (t == count + 1) {
+        sh.lut[kXEntries - 1] = xlut_entry(kXEntries - 1, precision, sh.slot, &bad);
+        if ((uint64_t)first + kXBuckets > 0xff00u) bad = true;  // infinity / NaN inside the window
+    }
+    if (t < count) sh.step_entry[t] = e;
+    if (__syncthreads_or(bad ? 1 : 0)) return false;
+    // the steps must come in ascending buckets, one per bucket
+    bad = (t > 0 && t < count) ? (index <= sh.step_index[t - 1]) : false;
+    if (__syncthreads_or(bad ? 1 : 0)) return false;
+    // Every thread fills a run of consecutive entries: the step whose bucket it is, else the codes
+    // below the next step (above the last one).
+    constexpr int kRun = (kXBuckets + kThreads - 1) / kThreads;
+    const int i0 = 1 + t * kRun;
+    const int i1 = (i0 + kRun < kXBuckets + 1) ? i0 + kRun : kXBuckets + 1;
+    int k = 0;  // first step at or above entry i0
+    for (int width = 128; width > 0; width >>= 1)
+        if (k + width <= count && sh.step_index[k + width - 1] < i0) k += width;
+    int next_index = k < count ? sh.step_index[k] : 0x7fffffff;
+    XEntry next_entry = sh.step_entry[k < count ? k : count - 1];
+    for (int i = i0; i < i1; ++i) {
+        if (i == next_index) {
+            sh.lut[i] = next_entry;
+            ++k;
+            next_index = k < count ? sh.step_index[k] : 0x7fffffff;
+            if (k < count) next_entry = sh.step_entry[k];
+            continue;
+        }
+        sh.lut[i] = xlut_flat_entry(next_entry, k >= count);
+    }
+    __syncthreads();
+    return true;
+}
 
 template <bool kVector>
 __global__ __launch_bounds__(kThreads) void compress_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr,
-    size_t n, uint8_t *__restrict__ codes, const XEntry *__restrict__ xlut,
-    const uint32_t *__restrict__ xflags, const float *__restrict__ table) {
+    size_t n, uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count,
+    const float *__restrict__ table) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
-    {
-        const uint2 *src = reinterpret_cast<const uint2 *>(xlut);
-        uint2 *dst = reinterpret_cast<uint2 *>(sh.lut);
-        for (int i = threadIdx.x; i < kXEntries; i += kThreads) dst[i] = src[i];
-        if (threadIdx.x < 126) sh.slot[threadIdx.x] = table[threadIdx.x];
-        if (threadIdx.x == 126) sh.slot[126] = 1.0f;
-        if (threadIdx.x == 127) sh.slot[127] = 0.0f;
-    }
-    const bool exact_only = __syncthreads_or((threadIdx.x < kXBuildBlocks && xflags[threadIdx.x] != 0) ? 1 : 0) != 0;
     const float precision = precision_ptr ? *precision_ptr : precision_value;
+    const bool exact_only = !build_table(sh, steps, step_count, precision, table);
     const uint32_t first = xlut_first(precision);
     auto encode = [&](float v) -> uint32_t {
         const uint32_t bits = __float_as_uint(v);
@@ -307,9 +334,6 @@ static cn_status compress_impl(const float *x, float precision, const float *pre
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(build_xlut_kernel, dim3(kXBuildBlocks), dim3(kThreads), 0, st, precision, precision_dev,
-                       ctx->table, ctx->xlut, ctx->xflags);
-    CN_HIP(hipGetLastError());
     // two workgroups per CU: mixed read/write streams run fastest on this part with few wavefronts
     // in flight, and the kernel keeps its own next tile in flight to stay busy at that occupancy
     int grid = stream_grid(ctx, n, 2);
@@ -323,10 +347,10 @@ static cn_status compress_impl(const float *x, float precision, const float *pre
     }
     if (aligned(x, 16) && aligned(codes, 4))
         hipLaunchKernelGGL(compress_kernel<true>, dim3(grid), dim3(kThreads), sizeof(EncodeShared), st, x, precision,
-                           precision_dev, n, codes, ctx->xlut, ctx->xflags, ctx->table);
+                           precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
     else
         hipLaunchKernelGGL(compress_kernel<false>, dim3(grid), dim3(kThreads), sizeof(EncodeShared), st, x, precision,
-                           precision_dev, n, codes, ctx->xlut, ctx->xflags, ctx->table);
+                           precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

@@ -33,21 +33,26 @@ extern "C" {
 
 int cn_host_xlut_entries(void) { return cn::kXEntries; }
 
-// Fills entries[kXEntries] (8 bytes each: boundary, codes) and *first for `precision`; returns 1 if
+int cn_host_xlut_step_count(void) {
+    float slot[128];
+    host_slot(slot);
+    static cn::XStep steps[cn::kXMaxSteps];
+    return cn::xlut_collect_steps(slot, steps);
+}
+
+// Fills entries[kXEntries] (8 bytes each: boundary, codes) and *first for `precision`, from the list
+// of steps, the way a workgroup of the encoder does; returns 1 if
 // the table must not be trusted for this precision (the encoder then evaluates every element
 // literally), else 0.
 int cn_host_xlut_build(float precision, void *entries, uint32_t *first) {
     float slot[128];
     host_slot(slot);
-    cn::XEntry *out = static_cast<cn::XEntry *>(entries);
-    int unusable = 0;
-    for (int i = 0; i < cn::kXEntries; ++i) {
-        bool bad = false;
-        out[i] = cn::xlut_entry(i, precision, slot, &bad);
-        unusable |= bad ? 1 : 0;
-    }
+    static cn::XStep steps[cn::kXMaxSteps];
+    static int count = -2;
+    if (count == -2) count = cn::xlut_collect_steps(slot, steps);
     if (first) *first = cn::xlut_first(precision);
-    return unusable;
+    if (count <= 0) return 1;
+    return cn::xlut_build_from_steps(steps, count, precision, slot, static_cast<cn::XEntry *>(entries)) ? 0 : 1;
 }
 
 // The encoder as the device runs it: table lookup, or the literal procedure when the table is

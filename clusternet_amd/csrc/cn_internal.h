@@ -28,8 +28,8 @@ struct Context {
     int device = -1;
     int num_cu = 0;
     float *table = nullptr;          // 126 floats
-    struct XEntry *xlut = nullptr;   // encoder table of the compression call in flight (cn_xlut.h)
-    uint32_t *xflags = nullptr;      // its "do not trust" flags, one per build workgroup
+    struct XStep *xsteps = nullptr;  // the steps of the code function (cn_xlut.h), found once at init
+    int xstep_count = 0;
     void *workspace = nullptr;       // split-K partial sums
     size_t workspace_bytes = 0;
     uint32_t *reduce_scratch = nullptr;  // per-workgroup partial maxima + ticket counters

@@ -58,8 +58,18 @@ static cn_status init_device(int device) {
     CN_HIP(hipMalloc((void **)&c.table, sizeof(table)));
     CN_HIP(hipMemcpy(c.table, table, sizeof(table), hipMemcpyHostToDevice));
 
-    CN_HIP(hipMalloc((void **)&c.xlut, (size_t)kXEntries * sizeof(XEntry)));
-    CN_HIP(hipMalloc((void **)&c.xflags, 64 * sizeof(uint32_t)));
+    {
+        float slot[128];
+        host_table(slot);
+        slot[126] = 1.0f;
+        slot[127] = 0.0f;
+        static XStep steps[kXMaxSteps];
+        const int count = xlut_collect_steps(slot, steps);
+        if (count <= 0 || count + 2 > 256) { set_error("init: the encoder's step list could not be derived"); return CN_ERR_ARG; }
+        c.xstep_count = count;
+        CN_HIP(hipMalloc((void **)&c.xsteps, sizeof(steps)));
+        CN_HIP(hipMemcpy(c.xsteps, steps, sizeof(steps), hipMemcpyHostToDevice));
+    }
 
     size_t mib = 1024;
     if (const char *env = getenv("CNHIP_WORKSPACE_MB")) {
@@ -134,8 +144,7 @@ cn_status cn_shutdown(void) {
         CN_HIP(hipSetDevice(d));
         CN_HIP(hipDeviceSynchronize());
         CN_HIP(hipFree(c.table));
-        CN_HIP(hipFree(c.xlut));
-        CN_HIP(hipFree(c.xflags));
+        CN_HIP(hipFree(c.xsteps));
         CN_HIP(hipFree(c.workspace));
         CN_HIP(hipFree(c.reduce_scratch));
         CN_HIP(hipFree(c.sum_scratch));

@@ -1,17 +1,18 @@
-// Per-call encoder table of compression_8bit, shared by the device build kernel and a host build
-// used by the CPU tests (plain inline C++, compiled by hipcc for both sides and by nothing else).
+// Encoder table of compression_8bit: construction and lookup, shared by the device kernel (every
+// workgroup builds the table for the call's precision in LDS) and by a host build used by the CPU
+// tests.  Plain inline C++.
 //
 // For a fixed precision the code of x is a step function of |x| (IEEE division and the reference's
 // search are both monotone in |x|) with the sign of x / precision on top.  The table is indexed by
 // the leading 17 bits of |x| (exponent and 8 mantissa bits): every bucket stores the code below and
 // above the one step it can contain, for either sign of x, and the first bit pattern that takes
-// the upper code.  All entries come from the literal procedure (encode_exact), evaluated at the
-// bucket ends and, where they differ, at the points of a binary search, so the table reproduces
-// the literal procedure for every input by construction: no approximate quotient, no guard band,
-// no restriction on the precision.  Buckets of the logarithmic range are 0.4 % wide and the
-// codebook's steps are at least 0.8 % apart, so a bucket holds at most one step; where that fails
-// (denormal inputs under a tiny precision) or the fixed-size table does not cover the code range,
-// the build reports it and the encoder evaluates the literal procedure for every element.
+// the upper code.  All entries come from evaluations of the literal procedure (encode_exact), so the
+// table reproduces the literal procedure for every input by construction: no approximate quotient,
+// no guard band, no restriction on the precision.  Buckets of the logarithmic range are 0.4 % wide
+// and the codebook's steps are at least 0.8 % apart, so a bucket holds at most one step; where that
+// fails (denormal inputs under a tiny precision), where a step cannot be pinned down or where the
+// fixed-size table does not cover the coded range, the build says so and the encoder evaluates the
+// literal procedure for every element instead.
 #pragma once
 
 #include <stdint.h>
@@ -41,21 +42,67 @@ CN_HD uint32_t x_to_bits(float f) { uint32_t b; memcpy(&b, &f, 4); return b; }
 // IEEE division, sign split, two threshold exits, 6-step pivot search over the table, two-candidate
 // pick.  `slot` is a 128-entry copy of the table whose entry 126 holds 1.0f.
 CN_HD uint32_t encode_exact(float x, float precision, const float *slot) {
+    // Written without branches (selects only) so that independent evaluations overlap on the device;
+    // the two threshold exits of the reference are applied last, which gives the same result because
+    // the search itself has no side effects.
     float a = x / precision;
-    uint32_t neg = 0;
-    if (a < 0.0f) { neg = 0x80u; a = -a; }
-    if (a < 0.0000015f) return 254u;
-    if (a > 0.995703f) return 127u | neg;
+    const uint32_t neg = (a < 0.0f) ? 0x80u : 0u;
+    a = (a < 0.0f) ? -a : a;
     int lo = 0, hi = 125, p = 63;
+#if defined(__HIPCC__)
+#pragma unroll
+#endif
     for (int step = 32; step > 0; step >>= 1) {
-        if (a > slot[p]) { lo = p; p += step; }
-        else             { hi = p; p -= step; }
+        const bool up = a > slot[p];
+        lo = up ? p : lo;
+        hi = up ? hi : p;
+        p = up ? p + step : p - step;
     }
-    const float dp = slot[p] - a;
-    int c;
-    if (lo == p) c = ((dp < 0 ? -dp : dp) < (slot[hi] - a)) ? p : hi;
-    else { const float dl = slot[lo] - a; c = (dp < (dl < 0 ? -dl : dl)) ? p : lo; }
-    return (uint32_t)c | neg;
+    const float dp = slot[p] - a, dh = slot[hi] - a, dl = slot[lo] - a;
+    const float adp = dp < 0 ? -dp : dp, adl = dl < 0 ? -dl : dl;
+    const int c_first = (adp < dh) ? p : hi;   // lo == p
+    const int c_other = (dp < adl) ? p : lo;
+    uint32_t code = (uint32_t)((lo == p) ? c_first : c_other) | neg;
+    code = (a > 0.995703f) ? (127u | neg) : code;
+    code = (a < 0.0000015f) ? 254u : code;
+    return code;
+}
+
+// N evaluations of encode_exact, written level by level so that the N table reads of a search level
+// are independent of each other (a single evaluation is a chain of seven dependent reads).
+template <int N>
+CN_HD void encode_exact_many(const uint32_t (&bits)[N], float precision, const float *slot, uint32_t (&code)[N]) {
+    float a[N];
+    uint32_t neg[N];
+    int lo[N], hi[N], p[N];
+    for (int j = 0; j < N; ++j) {
+        const float q = x_from_bits(bits[j]) / precision;
+        neg[j] = (q < 0.0f) ? 0x80u : 0u;
+        a[j] = (q < 0.0f) ? -q : q;
+        lo[j] = 0; hi[j] = 125; p[j] = 63;
+    }
+    for (int step = 32; step > 0; step >>= 1) {
+        float t[N];
+        for (int j = 0; j < N; ++j) t[j] = slot[p[j]];
+        for (int j = 0; j < N; ++j) {
+            const bool up = a[j] > t[j];
+            lo[j] = up ? p[j] : lo[j];
+            hi[j] = up ? hi[j] : p[j];
+            p[j] = up ? p[j] + step : p[j] - step;
+        }
+    }
+    float tp[N], th[N], tl[N];
+    for (int j = 0; j < N; ++j) { tp[j] = slot[p[j]]; th[j] = slot[hi[j]]; tl[j] = slot[lo[j]]; }
+    for (int j = 0; j < N; ++j) {
+        const float dp = tp[j] - a[j], dh = th[j] - a[j], dl = tl[j] - a[j];
+        const float adp = dp < 0 ? -dp : dp, adl = dl < 0 ? -dl : dl;
+        const int c_first = (adp < dh) ? p[j] : hi[j];
+        const int c_other = (dp < adl) ? p[j] : lo[j];
+        uint32_t c = (uint32_t)((lo[j] == p[j]) ? c_first : c_other) | neg[j];
+        c = (a[j] > 0.995703f) ? (127u | neg[j]) : c;
+        c = (a[j] < 0.0000015f) ? 254u : c;
+        code[j] = c;
+    }
 }
 
 // Bucket number of table entry 1 for this precision: one bucket below the bucket of 1.4e-6 |p|
@@ -81,22 +128,23 @@ CN_HD XEntry xlut_entry(int index, float precision, const float *slot, bool *unu
         // everything below bucket `first`: must be code 254 throughout, i.e. at its largest pattern
         if (first > 0) {
             const uint32_t top = (first << kXShift) - 1;
-            if (encode_exact(x_from_bits(top), precision, slot) != 254u ||
-                encode_exact(x_from_bits(top | kSign), precision, slot) != 254u) *unusable = true;
+            const uint32_t in[2] = {top, top | kSign};
+            uint32_t c[2];
+            encode_exact_many<2>(in, precision, slot, c);
+            if (c[0] != 254u || c[1] != 254u) *unusable = true;
         }
         return XEntry{0xffffffffu, pack_codes(254, 254, 254, 254)};
     }
     if (index == kXEntries - 1) {
         // everything above the last bucket: one code up to infinity, then the code of a NaN
-        const uint64_t start = ((uint64_t)first + kXBuckets) << kXShift;
-        const uint32_t c_nan = encode_exact(x_from_bits(0x7fc00000u), precision, slot);
-        const uint32_t n_nan = encode_exact(x_from_bits(0xffc00000u), precision, slot);
-        if (start > 0x7f800000u) return XEntry{0u, pack_codes(c_nan, c_nan, n_nan, n_nan)};  // only NaNs left
-        const uint32_t c0 = encode_exact(x_from_bits((uint32_t)start), precision, slot);
-        const uint32_t n0 = encode_exact(x_from_bits((uint32_t)start | kSign), precision, slot);
-        if (c0 != encode_exact(x_from_bits(0x7f800000u), precision, slot) ||
-            n0 != encode_exact(x_from_bits(0xff800000u), precision, slot)) *unusable = true;
-        return XEntry{0x7f800001u, pack_codes(c0, c_nan, n0, n_nan)};
+        const uint64_t start64 = ((uint64_t)first + kXBuckets) << kXShift;
+        const uint32_t start = start64 > 0x7f800000u ? 0x7f800000u : (uint32_t)start64;
+        const uint32_t in[6] = {0x7fc00000u, 0xffc00000u, start, start | kSign, 0x7f800000u, 0xff800000u};
+        uint32_t c[6];
+        encode_exact_many<6>(in, precision, slot, c);
+        if (start64 > 0x7f800000u) return XEntry{0u, pack_codes(c[0], c[0], c[1], c[1])};  // only NaNs left
+        if (c[2] != c[4] || c[3] != c[5]) *unusable = true;
+        return XEntry{0x7f800001u, pack_codes(c[2], c[0], c[3], c[1])};
     }
     const uint64_t bucket = (uint64_t)first + (uint32_t)(index - 1);
     if (bucket > 0xffffu) return XEntry{0xffffffffu, 0u};  // beyond the last bit pattern: never indexed
@@ -119,6 +167,118 @@ CN_HD XEntry xlut_entry(int index, float precision, const float *slot, bool *unu
         encode_exact(x_from_bits(below | kSign), precision, slot) != n_lo ||
         encode_exact(x_from_bits(above | kSign), precision, slot) != n_hi) *unusable = true;
     return XEntry{above, pack_codes(c_lo, c_hi, n_lo, n_hi)};
+}
+
+// ---- building the table from the list of steps --------------------------------------------------
+// At precision 1 the table above is built bucket by bucket (on the host, once).  Its steps - the
+// smallest quotient pattern S that takes the upper code, with the two magnitude codes - are the same
+// for every precision, because the code depends on x only through fl(|x| / |p|).  For another
+// precision the step sits at the smallest |x| with fl(|x| / |p|) >= S, within two patterns of
+// fl(S |p|): a workgroup finds all steps with nine literal evaluations each and fills the buckets
+// between them, which is cheap enough to do in every workgroup instead of sharing a table.
+struct XStep {
+    uint32_t boundary;  // S: smallest quotient pattern that takes `above`
+    uint32_t codes;     // below | above << 8, magnitude codes (0 .. 127 or 254)
+};
+constexpr int kXMaxSteps = 160;
+
+CN_HD uint32_t magnitude_code(uint32_t c) { return c == 254u ? 254u : (c & 0x7fu); }
+
+// Step `s` under `precision`: its entry (boundary in |x| patterns, the four codes).  False when the
+// step cannot be pinned down (estimate out of range, or the neighbourhood is not below ... above).
+CN_HD bool xlut_locate_step(XStep s, float precision, const float *slot, XEntry *entry) {
+    const uint32_t kSign = 0x80000000u;
+    const float ap = precision < 0 ? -precision : precision;
+    const uint32_t est = x_to_bits(x_from_bits(s.boundary) * ap);
+    if (!(est >= 16u && est <= 0x7f800000u - 16u)) return false;  // also false for a NaN estimate
+    const uint32_t below = s.codes & 0xffu, above = (s.codes >> 8) & 0xffu;
+    // ten independent evaluations around the estimate (independent so that they overlap), then the
+    // position of the step among them
+    uint32_t probe[10], code[10];
+    for (int j = 0; j < 10; ++j) probe[j] = est - 5 + (uint32_t)j;
+    encode_exact_many<10>(probe, precision, slot, code);
+    if (magnitude_code(code[0]) != below) return false;
+    int at = 0;  // first j whose code is `above`
+    bool clean = true;
+    for (int j = 1; j < 10; ++j) {
+        const uint32_t m = magnitude_code(code[j]);
+        if (at == 0) {
+            if (m == above) at = j; else if (m != below) clean = false;
+        } else if (m != above) {
+            clean = false;
+        }
+    }
+    if (at == 0 || !clean) return false;
+    const uint32_t found = est - 5 + (uint32_t)at;
+    uint32_t bp = code[0], tp = code[1];
+    for (int j = 1; j < 10; ++j)
+        if (j == at) { bp = code[j - 1]; tp = code[j]; }
+    const uint32_t mirrored[2] = {(found - 1) | kSign, found | kSign};
+    uint32_t mirror_code[2];
+    encode_exact_many<2>(mirrored, precision, slot, mirror_code);
+    const uint32_t bn = mirror_code[0], tn = mirror_code[1];
+    if (magnitude_code(bn) != below || magnitude_code(tn) != above) return false;
+    *entry = XEntry{found, pack_codes(bp, tp, bn, tn)};
+    return true;
+}
+
+// Entry of a bucket without a step, given the entry of the nearest step below (`from_above` false)
+// ... or the codes above the last step (`from_above` true).
+CN_HD XEntry xlut_flat_entry(XEntry step, bool above) {
+    const uint32_t c = step.codes;
+    const uint32_t pos = above ? ((c >> 8) & 0xffu) : (c & 0xffu);
+    const uint32_t neg = above ? ((c >> 24) & 0xffu) : ((c >> 16) & 0xffu);
+    return XEntry{0xffffffffu, pack_codes(pos, pos, neg, neg)};
+}
+
+// Host: the steps of the precision-1 table, in ascending order.  A step can sit inside a bucket or
+// exactly on its first pattern (then neither neighbour bucket shows two codes).  Returns their
+// number, or -1 if the table is unusable or the codes do not run from 254 up to 127.
+inline int xlut_collect_steps(const float *slot, XStep *out) {
+    int count = 0;
+    uint32_t current = 254u;  // code below the first bucket
+    for (int i = 1; i < kXEntries - 1; ++i) {
+        bool bad = false;
+        const XEntry e = xlut_entry(i, 1.0f, slot, &bad);
+        if (bad) return -1;
+        const uint32_t below = magnitude_code(e.codes & 0xffu), above = magnitude_code((e.codes >> 8) & 0xffu);
+        const uint32_t lo = (xlut_first(1.0f) + (uint32_t)(i - 1)) << kXShift;
+        if (below != current) {
+            if (count == kXMaxSteps) return -1;
+            out[count++] = XStep{lo, current | (below << 8)};
+        }
+        if (above != below) {
+            if (count == kXMaxSteps) return -1;
+            out[count++] = XStep{e.boundary, below | (above << 8)};
+        }
+        current = above;
+    }
+    return current == 127u ? count : -1;
+}
+
+// Host: the whole table for `precision` from the steps, the way a workgroup builds it.  Returns
+// false when the table must not be trusted.
+inline bool xlut_build_from_steps(const XStep *steps, int count, float precision, const float *slot, XEntry *lut) {
+    const uint32_t first = xlut_first(precision);
+    bool bad = false, unusable = false;
+    lut[0] = xlut_entry(0, precision, slot, &bad);
+    unusable |= bad;
+    lut[kXEntries - 1] = xlut_entry(kXEntries - 1, precision, slot, &bad);
+    unusable |= bad;
+    if ((uint64_t)first + kXBuckets > 0xff00u) unusable = true;  // infinity / NaN inside the window
+    int previous = 0;
+    XEntry e{};
+    for (int k = 0; k < count && !unusable; ++k) {
+        if (!xlut_locate_step(steps[k], precision, slot, &e)) { unusable = true; break; }
+        const int64_t index = (int64_t)(e.boundary >> kXShift) - (int64_t)first + 1;
+        if (index <= previous || index > kXBuckets) { unusable = true; break; }
+        for (int i = previous + 1; i < index; ++i) lut[i] = xlut_flat_entry(e, false);
+        lut[index] = e;
+        previous = (int)index;
+    }
+    if (unusable || count == 0) return false;
+    for (int i = previous + 1; i <= kXBuckets; ++i) lut[i] = xlut_flat_entry(e, true);
+    return true;
 }
 
 // Table index of a bit pattern.
