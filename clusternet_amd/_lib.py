@@ -47,6 +47,9 @@ def lib():
     L.cn_gemm_f32.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp]
     L.cn_gemm_f32_absmax.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, vp]
     L.cn_gemm_f32_w8.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, vp, i64, vp]
+    L.cn_csr_from_dense_f32.argtypes = [vp, i64, i64, i64, C.c_int, vp, vp, vp, i64, C.POINTER(i64), vp]
+    L.cn_csr_gemm_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp]
+    L.cn_csr_gemm_tn_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, C.c_int, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
     L.cn_compress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
@@ -154,6 +157,67 @@ def gemm_w8(A, W, scale, out=None):
         raise CnError(2, "Matrix size error")
     check(lib().cn_gemm_f32_w8(M, N, K, A.data_ptr(), _ld(A), W.data_ptr(), _ld(W), float(scale),
                                out.data_ptr(), _ld(out), _stream()))
+    return out
+
+
+class Csr:
+    """Device CSR matrix: rows x cols, row_ptr (int32, rows + 1), col_idx (int32), vals (fp32)."""
+
+    def __init__(self, rows, cols, row_ptr, col_idx, vals):
+        self.rows, self.cols, self.row_ptr, self.col_idx, self.vals = rows, cols, row_ptr, col_idx, vals
+
+    @property
+    def nnz(self):
+        return self.vals.numel()
+
+
+def csr_from_dense(A, transpose=False):
+    """CSR of the dense row-major A, or of its transpose (the CSC arrays of A)."""
+    import torch
+    _need(A, torch.float32, "A")
+    rows, cols = A.shape
+    R, Cc = (cols, rows) if transpose else (rows, cols)
+    row_ptr = torch.empty(R + 1, dtype=torch.int32, device=A.device)
+    nnz = C.c_int64(0)
+    status = lib().cn_csr_from_dense_f32(A.data_ptr(), rows, cols, _ld(A), int(transpose), row_ptr.data_ptr(), None,
+                                         None, 0, C.byref(nnz), _stream())
+    if status not in (0, 5):
+        check(status)
+    col_idx = torch.empty(max(nnz.value, 1), dtype=torch.int32, device=A.device)
+    vals = torch.empty(max(nnz.value, 1), dtype=torch.float32, device=A.device)
+    if nnz.value:
+        check(lib().cn_csr_from_dense_f32(A.data_ptr(), rows, cols, _ld(A), int(transpose), row_ptr.data_ptr(),
+                                          col_idx.data_ptr(), vals.data_ptr(), nnz.value, C.byref(nnz), _stream()))
+    return Csr(R, Cc, row_ptr, col_idx[:nnz.value], vals[:nnz.value])
+
+
+def csr_gemm(S, B, out=None):
+    """out = S B (S: Csr of shape R x C, B dense C x N)."""
+    import torch
+    _need(B, torch.float32, "B")
+    if B.shape[0] != S.cols:
+        raise CnError(2, "Matrix size error: S %dx%d, B %dx%d" % (S.rows, S.cols, B.shape[0], B.shape[1]))
+    N = B.shape[1]
+    if out is None:
+        out = torch.empty((S.rows, N), dtype=torch.float32, device=B.device)
+    _need(out, torch.float32, "out")
+    check(lib().cn_csr_gemm_f32(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                B.data_ptr(), _ld(B), out.data_ptr(), _ld(out), _stream()))
+    return out
+
+
+def csr_gemm_tn(S, B, out=None, splits=0):
+    """out = S^T B (S: Csr of shape R x C, B dense R x N; out C x N)."""
+    import torch
+    _need(B, torch.float32, "B")
+    if B.shape[0] != S.rows:
+        raise CnError(2, "Matrix size error: S^T %dx%d, B %dx%d" % (S.cols, S.rows, B.shape[0], B.shape[1]))
+    N = B.shape[1]
+    if out is None:
+        out = torch.empty((S.cols, N), dtype=torch.float32, device=B.device)
+    _need(out, torch.float32, "out")
+    check(lib().cn_csr_gemm_tn_f32(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                   B.data_ptr(), _ld(B), out.data_ptr(), _ld(out), int(splits), _stream()))
     return out
 
 

@@ -559,6 +559,20 @@ __global__ __launch_bounds__(256) void zero_matrix_kernel(float *__restrict__ C,
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// C = sum of the `splits` M x N planes at the start of the workspace, added in ascending order;
+// optionally also max |C| (see publish_absmax).
+cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float *C, int64_t ldc, uint32_t *amax,
+                           hipStream_t st) {
+    int vec = (N % 4 == 0) && (ldc % 4 == 0) && aligned(C, 16);
+    int64_t work = vec ? M * (N / 4) : M * N;
+    int64_t blocks = (work + 255) / 256;
+    int64_t cap = (int64_t)ctx->num_cu * 8;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, st,
+                       (const float *)ctx->workspace, splits, M, N, C, ldc, vec, amax);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
 template <bool A_KC, int B_KIND, int TN>
 static cn_status launch_tile(const GemmArgs &args, hipStream_t st) {
     using G = Geo<TN>;
@@ -641,15 +655,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     else                 s = launch<false, B_KC>(a, plan.tile_n, st);
     if (s != CN_OK) return s;
 
-    if (plan.splits > 1) {
-        int vec = (N % 4 == 0) && (ldc % 4 == 0) && aligned(C, 16);
-        int64_t work = vec ? M * (N / 4) : M * N;
-        int64_t blocks = (work + 255) / 256;
-        int64_t cap = (int64_t)ctx->num_cu * 8;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, st,
-                           (const float *)ctx->workspace, plan.splits, M, N, C, ldc, vec, amax);
-        CN_HIP(hipGetLastError());
-    }
+    if (plan.splits > 1) return add_chunk_planes(ctx, plan.splits, M, N, C, ldc, amax, st);
     return CN_OK;
 }
 

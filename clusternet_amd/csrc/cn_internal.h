@@ -50,6 +50,10 @@ struct GemmPlan {
     int64_t units;       // tiles_m * tiles_n * splits = grid size
 };
 // force_tile_n: 0 = choose, 128 or 256 = use that tile width.
+// C = sum of `splits` M x N planes held at the start of the workspace (ascending order); optional max |C|.
+cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float *C, int64_t ldc, uint32_t *amax,
+                           hipStream_t st);
+
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 
 constexpr int kTileM = 128;

@@ -153,6 +153,35 @@ cn_status cn_rmsprop_update_w8_dp(float *rms_device, const uint8_t *codes_device
                                   const float *precision_device, float *w_device, float rms_multiplier,
                                   float learning_rate, size_t n, void *stream);
 
+/* ---- sparse (CSR) operands ----------------------------------------------------------------------
+ * 32-bit zero-based indices, column indices ascending within a row: the layout of the reference's
+ * sparse Matrix (ptr_rows, idx_cols, data; source/basicOps.cuh:25-42) and of cusparseSdense2csr. */
+
+/* CSR of A (transpose = 0) or of A^T (transpose != 0; i.e. the CSC arrays of A), A row-major rows x cols.
+ * row_ptr has rows + 1 (cols + 1) entries; col_idx and vals have room for `capacity` nonzeros.
+ * *nnz_host receives the number of nonzeros (values that compare unequal to zero); the call
+ * synchronises the stream to deliver it.  If it exceeds `capacity`, row_ptr is valid, nothing else is
+ * written and the status is CN_ERR_WORKSPACE: call once with capacity 0 to size the arrays.
+ * dense_to_sparse, source/clusterNet.cpp:1004-1032 (cusparseSnnz + cusparseSdense2csr). */
+cn_status cn_csr_from_dense_f32(const float *A_device, int64_t rows, int64_t cols, int64_t lda, int transpose,
+                                int32_t *row_ptr_device, int32_t *col_idx_device, float *vals_device,
+                                int64_t capacity, int64_t *nnz_host, void *stream);
+
+/* out[R x N] = S B with S an R x C CSR matrix and B a dense C x N matrix: every output row gathers the
+ * rows of B named by its nonzeros, in ascending order, each term as a rounded product added to the
+ * running sum.  dot_sparse, source/clusterNet.cpp:301-401 (cusparseScsrmm2, non-transposed A). */
+cn_status cn_csr_gemm_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
+                          const int32_t *col_idx_device, const float *vals_device, const float *B_device,
+                          int64_t ldb, float *out_device, int64_t ldo, void *stream);
+
+/* out[C x N] = S^T B with S an R x C CSR matrix and B a dense R x N matrix: B is read once, row k of B is
+ * added, scaled, into the output rows named by row k of S.  Tdot_sparse (transposed A of
+ * cusparseScsrmm2), source/clusterNet.cpp:304,307.  `splits` > 0 fixes the number of chunks the R rows
+ * are cut into (partial outputs are added in ascending order; 1 = none), 0 lets the library choose. */
+cn_status cn_csr_gemm_tn_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
+                             const int32_t *col_idx_device, const float *vals_device, const float *B_device,
+                             int64_t ldb, float *out_device, int64_t ldo, int splits, void *stream);
+
 /* ---- small kernels used around the path by its callers (row-major, flat where no shape is given).
  * They are not on the measured hot path; each names the reference routine it stands in for. */
 

@@ -36,6 +36,11 @@ def _load():
     lib.cn_oracle_decompress.argtypes = [_u8p, _c.c_float, _c.c_size_t, _f32p]
     lib.cn_oracle_decompress_axpy.argtypes = [_u8p, _c.c_float, _c.c_float, _c.c_size_t, _f32p]
     lib.cn_oracle_rmsprop_update.argtypes = [_f32p, _f32p, _f32p, _c.c_float, _c.c_float, _c.c_size_t]
+    _i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+    lib.cn_oracle_csr_from_dense.argtypes = [_f32p, _c.c_int64, _c.c_int64, _c.c_int, _i32p, _c.c_void_p, _c.c_void_p]
+    lib.cn_oracle_csr_from_dense.restype = _c.c_int64
+    lib.cn_oracle_csr_gemm.argtypes = [_c.c_int64, _c.c_int64, _i32p, _i32p, _f32p, _f32p, _f32p]
+    lib.cn_oracle_csr_gemm_tn.argtypes = [_c.c_int64, _c.c_int64, _c.c_int64, _i32p, _i32p, _f32p, _f32p, _f32p, _c.c_int]
     lib.cn_oracle_absmax.argtypes = [_f32p, _c.c_size_t]
     lib.cn_oracle_absmax.restype = _c.c_float
     g = [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _f32p, _c.c_int64, _f32p,
@@ -117,6 +122,43 @@ def rmsprop_update(rms, grad, w, rms_multiplier, learning_rate):
     _lib.cn_oracle_rmsprop_update(r.reshape(-1), g.reshape(-1), ww.reshape(-1), float(rms_multiplier),
                                   float(learning_rate), g.size)
     return r, ww
+
+
+def csr_from_dense(A, transpose=False):
+    """(row_ptr, col_idx, vals) of A, or of A^T when `transpose`."""
+    A = _f32(A)
+    rows, cols = A.shape
+    R = cols if transpose else rows
+    row_ptr = np.zeros(R + 1, np.int32)
+    nnz = _lib.cn_oracle_csr_from_dense(A, rows, cols, int(transpose), row_ptr, None, None)
+    col_idx = np.zeros(max(nnz, 1), np.int32)
+    vals = np.zeros(max(nnz, 1), np.float32)
+    _lib.cn_oracle_csr_from_dense(A, rows, cols, int(transpose), row_ptr, col_idx.ctypes.data, vals.ctypes.data)
+    return row_ptr, col_idx[:nnz], vals[:nnz]
+
+
+def _csr_arrays(csr):
+    row_ptr, col_idx, vals = csr
+    pad = lambda a, t: np.ascontiguousarray(a if a.size else np.zeros(1, t), t)
+    return np.ascontiguousarray(row_ptr, np.int32), pad(col_idx, np.int32), pad(vals, np.float32)
+
+
+def csr_gemm(csr, B):
+    """S B for S = (row_ptr, col_idx, vals)."""
+    row_ptr, col_idx, vals = _csr_arrays(csr)
+    B = _f32(B)
+    out = np.empty((row_ptr.size - 1, B.shape[1]), np.float32)
+    _lib.cn_oracle_csr_gemm(row_ptr.size - 1, B.shape[1], row_ptr, col_idx, vals, B, out)
+    return out
+
+
+def csr_gemm_tn(csr, cols, B, splits=1):
+    """S^T B for the R x cols matrix S = (row_ptr, col_idx, vals) and B with R rows."""
+    row_ptr, col_idx, vals = _csr_arrays(csr)
+    B = _f32(B)
+    out = np.empty((cols, B.shape[1]), np.float32)
+    _lib.cn_oracle_csr_gemm_tn(row_ptr.size - 1, cols, B.shape[1], row_ptr, col_idx, vals, B, out, int(splits))
+    return out
 
 
 def absmax(x):

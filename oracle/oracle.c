@@ -19,6 +19,14 @@
  *                                defined to that accuracy).  Pinned by its closed forms: multiplier
  *                                0 and 1, zero gradient, and an fp64 evaluation of the same formula
  *                                (tests/test_oracle_codec.py)
+ *   cn_oracle_csr_from_dense     dense_to_sparse, source/clusterNet.cpp:1004-1032 (cusparseSnnz +
+ *   cn_oracle_csr_gemm(_tn)      cusparseSdense2csr) and dot_sparse / Tdot_sparse, :301-401
+ *                                (cusparseScsrmm2).  cuSPARSE is closed source; what it computes is the
+ *                                textbook CSR layout and product, restated here with sums in ascending
+ *                                index order.  Pinned by scipy.sparse (layout) and by the dense
+ *                                product of the densified operand (tests/test_oracle_sparse.py); the
+ *                                reference's own tests only ask for agreement with the dense product
+ *                                within 0.1 (tests/clusterNet_test.cu:396-463)
  *   cn_oracle_absmax             source/basicOps.cu:810-822 + source/clusterKernels.cu:429-436
  *                                (abs) followed by source/basicOps.cu:1076-1081 (max)
  *   cn_oracle_gemm_*             source/clusterNet.cpp:404-461: C = op(A) op(B), alpha 1, beta 0,
@@ -168,6 +176,64 @@ void cn_oracle_rmsprop_update(float *rms, const float *grad, float *w, float rms
         rms[i] = r;
         w[i] = w[i] - step;
     }
+}
+
+/* CSR of A (transpose 0) or of A^T; returns the number of nonzeros (values != 0).  col_idx / vals may
+ * be NULL to count only. */
+int64_t cn_oracle_csr_from_dense(const float *A, int64_t rows, int64_t cols, int transpose, int32_t *row_ptr,
+                                 int32_t *col_idx, float *vals) {
+    const int64_t R = transpose ? cols : rows, C = transpose ? rows : cols;
+    int64_t n = 0;
+    for (int64_t i = 0; i < R; ++i) {
+        row_ptr[i] = (int32_t)n;
+        for (int64_t j = 0; j < C; ++j) {
+            const float v = transpose ? A[j * cols + i] : A[i * cols + j];
+            if (v != 0.0f) {
+                if (col_idx) col_idx[n] = (int32_t)j;
+                if (vals) vals[n] = v;
+                ++n;
+            }
+        }
+    }
+    row_ptr[R] = (int32_t)n;
+    return n;
+}
+
+/* out[R x N] = S B, every row summed over its nonzeros in ascending order, product rounded first. */
+void cn_oracle_csr_gemm(int64_t R, int64_t N, const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                        const float *B, float *out) {
+    for (int64_t r = 0; r < R; ++r)
+        for (int64_t n = 0; n < N; ++n) {
+            float acc = 0.0f;
+            for (int32_t j = row_ptr[r]; j < row_ptr[r + 1]; ++j) {
+                volatile float term = vals[j] * B[(int64_t)col_idx[j] * N + n];
+                acc = acc + term;
+            }
+            out[r * N + n] = acc;
+        }
+}
+
+/* out[C x N] = S^T B, the rows of S taken in ascending order within each of `splits` equal chunks,
+ * chunk sums added in ascending order (splits = 1: one running sum). */
+void cn_oracle_csr_gemm_tn(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                           const float *vals, const float *B, float *out, int splits) {
+    const int64_t per = (R + splits - 1) / (splits > 0 ? splits : 1);
+    float *part = (float *)malloc((size_t)(C * N ? C * N : 1) * sizeof(float));
+    for (int64_t i = 0; i < C * N; ++i) out[i] = 0.0f;
+    for (int64_t k0 = 0, chunk = 0; k0 < R || chunk == 0; k0 += per, ++chunk) {
+        const int64_t k1 = k0 + per < R ? k0 + per : R;
+        for (int64_t i = 0; i < C * N; ++i) part[i] = 0.0f;
+        for (int64_t k = k0; k < k1; ++k)
+            for (int32_t j = row_ptr[k]; j < row_ptr[k + 1]; ++j)
+                for (int64_t n = 0; n < N; ++n) {
+                    volatile float term = vals[j] * B[k * N + n];
+                    part[(int64_t)col_idx[j] * N + n] = part[(int64_t)col_idx[j] * N + n] + term;
+                }
+        if (chunk == 0) memcpy(out, part, (size_t)(C * N) * sizeof(float));
+        else for (int64_t i = 0; i < C * N; ++i) out[i] = out[i] + part[i];
+        if (per <= 0) break;
+    }
+    free(part);
 }
 
 /* max_i |x_i|, start value -1 as in the reference's reduction; NaN propagates. */

@@ -1,0 +1,139 @@
+"""Parity of the sparse (CSR) path with the CPU checker through the C-ABI: layout bit for bit, the
+gather product bit for bit (same summation order), the scatter product bit for bit when the chunking
+is given and within the GEMM tolerance of the fp64 dense product otherwise."""
+import numpy as np
+import pytest
+
+import oracle
+from util import gemm_tolerance
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    import torch
+    import clusternet_amd as cn
+    cn.init(0)
+    return torch.device("cuda:0")
+
+
+def _t(a, dev):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def _sparse(rng, rows, cols, density):
+    A = rng.uniform(0, 1, (rows, cols)).astype(np.float32)
+    return A * (rng.random((rows, cols)) < density)
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint32)
+
+
+@pytest.mark.parametrize("shape,density", [((1, 1), 1.0), ((7, 11), 0.3), ((128, 5000), 0.02), ((300, 257), 0.1),
+                                           ((5, 1000), 0.0), ((128, 1024), 1.0), ((1000, 3), 0.5)])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_csr_from_dense_matches_checker(dev, shape, density, transpose):
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(shape[0] * 31 + shape[1])
+    A = _sparse(rng, *shape, density)
+    if A.size > 3:
+        A.flat[1] = -0.0
+    S = L.csr_from_dense(_t(A, dev), transpose)
+    row_ptr, col_idx, vals = oracle.csr_from_dense(A, transpose)
+    assert (S.rows, S.cols) == ((shape[1], shape[0]) if transpose else shape)
+    assert np.array_equal(S.row_ptr.cpu().numpy(), row_ptr)
+    assert np.array_equal(S.col_idx.cpu().numpy(), col_idx)
+    assert np.array_equal(_bits(S.vals.cpu().numpy()), _bits(vals))
+
+
+def test_csr_from_dense_of_a_strided_view_and_capacity_error(dev):
+    import ctypes as C
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(5)
+    big = _sparse(rng, 64, 300, 0.2)
+    view = _t(big, dev)[:, 10:210]
+    S = L.csr_from_dense(view)
+    row_ptr, col_idx, vals = oracle.csr_from_dense(np.ascontiguousarray(big[:, 10:210]))
+    assert np.array_equal(S.row_ptr.cpu().numpy(), row_ptr) and np.array_equal(S.col_idx.cpu().numpy(), col_idx)
+    nnz = C.c_int64()
+    rp = torch.empty(65, dtype=torch.int32, device=dev)
+    ci = torch.empty(4, dtype=torch.int32, device=dev)
+    va = torch.empty(4, dtype=torch.float32, device=dev)
+    status = L.lib().cn_csr_from_dense_f32(view.data_ptr(), 64, 200, 300, 0, rp.data_ptr(), ci.data_ptr(), va.data_ptr(), 4,
+                                           C.byref(nnz), None)
+    assert status == 5 and nnz.value == vals.size and np.array_equal(rp.cpu().numpy(), row_ptr)
+
+
+@pytest.mark.parametrize("R,Cc,N,density", [(37, 211, 19, 0.05), (1000, 128, 1024, 0.02), (300, 64, 4100, 0.1),
+                                            (5, 9, 1, 0.5), (2048, 128, 8192, 0.02), (16, 40, 7, 0.0)])
+def test_gather_product_is_bit_exact(dev, R, Cc, N, density):
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(R + N)
+    S_dense = _sparse(rng, R, Cc, density)
+    B = rng.normal(0, 1, (Cc, N)).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    got = L.csr_gemm(S, _t(B, dev)).cpu().numpy()
+    want = oracle.csr_gemm(oracle.csr_from_dense(S_dense), B)
+    assert np.array_equal(_bits(got), _bits(want))
+
+
+@pytest.mark.parametrize("R,Cc,N,density", [(211, 37, 19, 0.05), (5000, 128, 1024, 0.02), (3000, 64, 300, 0.1),
+                                            (9, 5, 1, 0.5), (1000, 300, 520, 0.05), (40, 16, 7, 0.0)])
+def test_scatter_product(dev, R, Cc, N, density):
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(R + N + 1)
+    S_dense = _sparse(rng, R, Cc, density)
+    B = rng.normal(0, 1, (R, N)).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    csr = oracle.csr_from_dense(S_dense)
+    for splits in (1, 3):
+        got = L.csr_gemm_tn(S, _t(B, dev), splits=splits).cpu().numpy()
+        eff = -(-R // -(-R // splits))             # chunks actually formed
+        want = oracle.csr_gemm_tn(csr, Cc, B, eff)
+        assert np.array_equal(_bits(got), _bits(want)), splits
+    got = L.csr_gemm_tn(S, _t(B, dev)).cpu().numpy()      # library's own chunking
+    ref = S_dense.T.astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(S_dense.T.astype(np.float64)) @ np.abs(B.astype(np.float64))
+    tol = gemm_tolerance(R)
+    assert np.max(np.abs(got - ref)) <= tol * max(np.max(np.abs(ref)), 1e-30)
+    assert np.all(np.abs(got - ref) <= tol * np.maximum(scale, 1e-30))
+
+
+def test_batch_products_through_the_transposed_csr(dev):
+    """The two products of the training step on a 2 % dense batch: X W = S^T W and X^T E = S E with
+    S = CSR(X^T); against the dense kernels of this library and the fp64 product."""
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(8)
+    X = _sparse(rng, 128, 6000, 0.02)
+    W = rng.uniform(-0.01, 0.01, (6000, 2048)).astype(np.float32)
+    E = rng.normal(0, 0.01, (128, 2048)).astype(np.float32)
+    Xt, Wt, Et = _t(X, dev), _t(W, dev), _t(E, dev)
+    S = L.csr_from_dense(Xt, transpose=True)
+    assert (S.rows, S.cols) == (6000, 128)
+    fwd = L.csr_gemm_tn(S, Wt).cpu().numpy()
+    ref = X.astype(np.float64) @ W.astype(np.float64)
+    assert np.max(np.abs(fwd - ref)) <= gemm_tolerance(6000) * np.max(np.abs(ref))
+    assert np.max(np.abs(fwd - cn.dot(Xt, Wt).cpu().numpy())) <= 2 * gemm_tolerance(6000) * np.max(np.abs(ref))
+    grad = L.csr_gemm(S, Et).cpu().numpy()
+    ref_g = X.T.astype(np.float64) @ E.astype(np.float64)
+    assert np.max(np.abs(grad - ref_g)) <= gemm_tolerance(128) * np.max(np.abs(ref_g))
+    assert np.array_equal(_bits(grad), _bits(oracle.csr_gemm(oracle.csr_from_dense(X, True), E)))
+
+
+def test_shape_errors(dev):
+    import torch
+    from clusternet_amd import _lib as L
+    S = L.csr_from_dense(torch.zeros((4, 5), device=dev))
+    assert S.nnz == 0
+    with pytest.raises(L.CnError):
+        L.csr_gemm(S, torch.zeros((4, 3), device=dev))
+    with pytest.raises(L.CnError):
+        L.csr_gemm_tn(S, torch.zeros((5, 3), device=dev))
+    assert torch.equal(L.csr_gemm(S, torch.ones((5, 3), device=dev)), torch.zeros((4, 3), device=dev))
+    assert torch.equal(L.csr_gemm_tn(S, torch.ones((4, 3), device=dev)), torch.zeros((5, 3), device=dev))
