@@ -49,7 +49,7 @@ def lib():
     L.cn_gemm_f32_w8.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, vp, i64, vp]
     L.cn_csr_from_dense_f32.argtypes = [vp, i64, i64, i64, C.c_int, vp, vp, vp, i64, C.POINTER(i64), vp]
     L.cn_csr_gemm_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp]
-    L.cn_csr_gemm_tn_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, C.c_int, vp]
+    L.cn_csr_transpose.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
     L.cn_compress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
@@ -206,19 +206,18 @@ def csr_gemm(S, B, out=None):
     return out
 
 
-def csr_gemm_tn(S, B, out=None, splits=0):
-    """out = S^T B (S: Csr of shape R x C, B dense R x N; out C x N)."""
+def csr_transpose(S):
+    """CSR of S^T."""
     import torch
-    _need(B, torch.float32, "B")
-    if B.shape[0] != S.rows:
-        raise CnError(2, "Matrix size error: S^T %dx%d, B %dx%d" % (S.cols, S.rows, B.shape[0], B.shape[1]))
-    N = B.shape[1]
-    if out is None:
-        out = torch.empty((S.cols, N), dtype=torch.float32, device=B.device)
-    _need(out, torch.float32, "out")
-    check(lib().cn_csr_gemm_tn_f32(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
-                                   B.data_ptr(), _ld(B), out.data_ptr(), _ld(out), int(splits), _stream()))
-    return out
+    dev = S.row_ptr.device
+    t_row_ptr = torch.empty(S.cols + 1, dtype=torch.int32, device=dev)
+    t_col_idx = torch.empty(max(S.nnz, 1), dtype=torch.int32, device=dev)
+    t_vals = torch.empty(max(S.nnz, 1), dtype=torch.float32, device=dev)
+    scratch = torch.empty(max(S.cols, 1), dtype=torch.int32, device=dev)
+    check(lib().cn_csr_transpose(S.rows, S.cols, S.nnz, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                 t_row_ptr.data_ptr(), t_col_idx.data_ptr(), t_vals.data_ptr(), scratch.data_ptr(),
+                                 _stream()))
+    return Csr(S.cols, S.rows, t_row_ptr, t_col_idx[:S.nnz], t_vals[:S.nnz])
 
 
 def absmax(x, out=None):

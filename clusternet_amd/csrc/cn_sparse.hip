@@ -5,16 +5,15 @@
 // the same stream (or by writing the result) and do no wasted arithmetic.  S is an R x C matrix in
 // CSR form (row_ptr[R + 1], col_idx[nnz] ascending within a row, vals[nnz]), 32-bit indices.
 //
-//   csr_gemm      out[R x N] = S B     every output row gathers the B rows of its nonzeros
-//                                       (bound by writing out; B should be small enough to stay in L2)
-//   csr_gemm_tn   out[C x N] = S^T B   B is streamed once, row k of B is scattered into the output rows
-//                                       named by row k of S; the output (C <= 128 rows per pass) is
-//                                       accumulated in LDS; the R rows may be split into chunks whose
-//                                       partial outputs are added in a fixed order
+//   csr_gemm        out[R x N] = S B: every output row gathers the B rows of its nonzeros, four columns
+//                   per lane, accumulators in registers.  Rows are processed by workgroups that run
+//                   side by side and walk their nonzeros in ascending order, so a B row needed by
+//                   several output rows is fetched from HBM once and served from L2 afterwards
+//   csr_transpose   CSR(S) -> CSR(S^T), for the products with the transposed sparse operand
 //
-// With X the 128 x 100000 batch and S = CSR(X^T):  X W = S^T W (csr_gemm_tn) and X^T E = S E (csr_gemm).
+// With X the 128 x 100000 batch:  X W = CSR(X) W and X^T E = CSR(X^T) E, both through csr_gemm.
 // Sums run over the nonzeros in ascending order with a rounded product and a rounded addition per
-// term, so csr_gemm is reproducible to the bit and csr_gemm_tn is once the chunking is fixed.
+// term, so the results are reproducible to the bit.
 #include "cn_internal.h"
 
 namespace cn {
@@ -127,7 +126,11 @@ __global__ __launch_bounds__(kT) void fill_cols_kernel(const float *__restrict__
 }
 
 // ---- out = S B (gather) ---------------------------------------------------------------------------------
-// A workgroup owns a block of 1024 columns (4 per lane) and walks a range of output rows.
+// A workgroup owns a block of 1024 columns (4 per lane) and walks a range of output rows.  The
+// nonzeros of a row are taken eight at a time: indices and values first, then the eight B rows, then
+// the eight multiply-adds in order.
+constexpr int kGather = 8;
+
 template <bool kVector>
 __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, const int32_t *__restrict__ row_ptr,
                                                       const int32_t *__restrict__ col_idx,
@@ -141,10 +144,21 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
         if (kVector) {
             if (n >= N) continue;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            for (int32_t j = j0; j < j1; ++j) {
-                const float v = vals[j];
-                const f32x4 b = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + n);
-                acc = acc + v * b;
+            for (int32_t j = j0; j < j1; j += kGather) {
+                int32_t c[kGather];
+                float v[kGather];
+                f32x4 b[kGather];
+#pragma unroll
+                for (int u = 0; u < kGather; ++u) {
+                    const int32_t at = (j + u < j1) ? j + u : j1 - 1;  // past the end: a valid, unused address
+                    c[u] = col_idx[at];
+                    v[u] = vals[at];
+                }
+#pragma unroll
+                for (int u = 0; u < kGather; ++u) b[u] = *reinterpret_cast<const f32x4 *>(B + (int64_t)c[u] * ldb + n);
+#pragma unroll
+                for (int u = 0; u < kGather; ++u)
+                    if (j + u < j1) acc = acc + v[u] * b[u];
             }
             __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(out + r * ldo + n));
         } else {
@@ -161,55 +175,47 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
     }
 }
 
-// ---- out = S^T B (scatter into LDS) -----------------------------------------------------------------------
-// A workgroup owns 256 output columns (one per lane), up to 128 output rows [c0, c0 + 128) and a range
-// of S rows.  acc[c][lane] lives in LDS; lane t only ever touches column t, so no atomics are needed.
-constexpr int kScatterRows = 128;
-constexpr int kScatterCols = 256;
+// ---- CSR(S) -> CSR(S^T) ------------------------------------------------------------------------------------
+// Histogram of the column indices, prefix sums, a fill in arbitrary order, then every row of the
+// result is sorted by its (few) column indices: the result does not depend on the order of the fill.
+__global__ __launch_bounds__(kT) void histogram_kernel(const int32_t *__restrict__ col_idx, int64_t nnz,
+                                                       int32_t *__restrict__ counts) {
+    for (int64_t j = (int64_t)blockIdx.x * kT + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kT)
+        atomicAdd(&counts[col_idx[j]], 1);
+}
 
-__global__ __launch_bounds__(kT) void csr_gemm_tn_kernel(int64_t R, int64_t Cc, int64_t N,
-                                                         const int32_t *__restrict__ row_ptr,
-                                                         const int32_t *__restrict__ col_idx,
-                                                         const float *__restrict__ vals, const float *__restrict__ B,
-                                                         int64_t ldb, float *__restrict__ out, int64_t ldo,
-                                                         float *__restrict__ partial, int64_t col_blocks,
-                                                         int64_t row_blocks, int splits, int64_t rows_per_split) {
-    extern __shared__ __attribute__((aligned(16))) float acc[];  // [kScatterRows][kScatterCols]
-    const int64_t cb = blockIdx.x % col_blocks;
-    const int64_t rb = (blockIdx.x / col_blocks) % row_blocks;
-    const int64_t split = blockIdx.x / (col_blocks * row_blocks);
-    const int64_t n = cb * kScatterCols + threadIdx.x;
-    const int32_t c0 = (int32_t)(rb * kScatterRows);
-    const bool live = n < N;
-    for (int c = 0; c < kScatterRows; ++c) acc[c * kScatterCols + threadIdx.x] = 0.0f;
-    const int64_t k0 = split * rows_per_split;
-    const int64_t k1 = (k0 + rows_per_split < R) ? k0 + rows_per_split : R;
-    constexpr int kAhead = 8;  // B values in flight per lane
-    for (int64_t kb = k0; kb < k1; kb += kAhead) {
-        float b[kAhead];
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u)
-            b[u] = (live && kb + u < k1) ? __builtin_nontemporal_load(B + (kb + u) * ldb + n) : 0.0f;
-#pragma unroll
-        for (int u = 0; u < kAhead; ++u) {
-            if (kb + u >= k1) break;
-            const int32_t j0 = row_ptr[kb + u], j1 = row_ptr[kb + u + 1];
-            for (int32_t j = j0; j < j1; ++j) {
-                const int32_t c = col_idx[j] - c0;
-                if (c < 0 || c >= kScatterRows) continue;
-                float *cell = acc + c * kScatterCols + threadIdx.x;
-                *cell = *cell + vals[j] * b[u];
-            }
+__global__ __launch_bounds__(kT) void transpose_fill_kernel(int64_t R, const int32_t *__restrict__ row_ptr,
+                                                            const int32_t *__restrict__ col_idx,
+                                                            const float *__restrict__ vals,
+                                                            int32_t *__restrict__ cursor, int32_t *__restrict__ out_col,
+                                                            float *__restrict__ out_val) {
+    // one workgroup per row of S; cursor[c] starts at the first slot of row c of the result
+    for (int64_t r = blockIdx.x; r < R; r += gridDim.x)
+        for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) {
+            const int32_t at = atomicAdd(&cursor[col_idx[j]], 1);
+            out_col[at] = (int32_t)r;
+            out_val[at] = vals[j];
+        }
+}
+
+__global__ __launch_bounds__(kT) void sort_rows_kernel(int64_t R, const int32_t *__restrict__ row_ptr,
+                                                       int32_t *__restrict__ col_idx, float *__restrict__ vals) {
+    // insertion sort of every row by column index, one thread per row
+    for (int64_t r = (int64_t)blockIdx.x * kT + threadIdx.x; r < R; r += (int64_t)gridDim.x * kT) {
+        const int32_t j0 = row_ptr[r], j1 = row_ptr[r + 1];
+        for (int32_t j = j0 + 1; j < j1; ++j) {
+            const int32_t c = col_idx[j];
+            const float v = vals[j];
+            int32_t i = j - 1;
+            while (i >= j0 && col_idx[i] > c) { col_idx[i + 1] = col_idx[i]; vals[i + 1] = vals[i]; --i; }
+            col_idx[i + 1] = c;
+            vals[i + 1] = v;
         }
     }
-    if (!live) return;
-    const int64_t rows_here = (Cc - c0 < kScatterRows) ? Cc - c0 : kScatterRows;
-    if (splits > 1) {
-        float *plane = partial + split * Cc * N;
-        for (int64_t c = 0; c < rows_here; ++c) plane[(c0 + c) * N + n] = acc[c * kScatterCols + threadIdx.x];
-    } else {
-        for (int64_t c = 0; c < rows_here; ++c) out[(c0 + c) * ldo + n] = acc[c * kScatterCols + threadIdx.x];
-    }
+}
+
+__global__ __launch_bounds__(kT) void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) dst[i] = src[i];
 }
 
 cn_status check_csr_args(const char *who, int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr,
@@ -305,47 +311,39 @@ cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_p
     return CN_OK;
 }
 
-cn_status cn_csr_gemm_tn_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
-                             const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, int splits,
-                             void *stream) {
-    cn_status s = check_csr_args("csr_gemm_tn_f32", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo);
-    if (s != CN_OK) return s;
-    if (Cc == 0 || N == 0) return CN_OK;
-    if (!out) { set_error("csr_gemm_tn_f32: NULL output"); return CN_ERR_NULL; }
+cn_status cn_csr_transpose(int64_t R, int64_t Cc, int64_t nnz, const int32_t *row_ptr, const int32_t *col_idx,
+                           const float *vals, int32_t *t_row_ptr, int32_t *t_col_idx, float *t_vals,
+                           int32_t *scratch, void *stream) {
+    if (R < 0 || Cc < 0 || nnz < 0 || R > 0x7fffffffLL || Cc > 0x7fffffffLL || nnz > 0x7fffffffLL) {
+        set_error("csr_transpose: bad dimensions");
+        return CN_ERR_SHAPE;
+    }
+    if (!row_ptr || !t_row_ptr || (Cc > 0 && !scratch) || (nnz > 0 && (!col_idx || !vals || !t_col_idx || !t_vals))) {
+        set_error("csr_transpose: NULL pointer");
+        return CN_ERR_NULL;
+    }
     Context *ctx;
-    s = current_context(&ctx);
+    cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
-    const int64_t col_blocks = (N + kScatterCols - 1) / kScatterCols;
-    const int64_t row_blocks = (Cc + kScatterRows - 1) / kScatterRows;
-    if (splits <= 0) {  // enough workgroups for one per compute unit, chunks at least 256 rows deep
-        int64_t want = ((int64_t)ctx->num_cu + col_blocks * row_blocks - 1) / (col_blocks * row_blocks);
-        int64_t most = R / 256;
-        if (want > most) want = most;
-        if (want > 64) want = 64;
-        splits = (int)(want < 1 ? 1 : want);
-    }
-    if (splits > 1 && (size_t)splits * (size_t)Cc * (size_t)N * sizeof(float) > ctx->workspace_bytes) {
-        size_t fit = ctx->workspace_bytes / ((size_t)Cc * (size_t)N * sizeof(float));
-        splits = (int)(fit < 1 ? 1 : fit);
-    }
-    int64_t rows_per_split = (R + splits - 1) / splits;
-    if (rows_per_split < 1) rows_per_split = 1;
-    splits = (int)((R + rows_per_split - 1) / rows_per_split);
-    if (splits < 1) splits = 1;
-    const size_t lds = (size_t)kScatterRows * kScatterCols * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_gemm_tn_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        configured = true;
-    }
-    const int64_t grid = col_blocks * row_blocks * splits;
-    if (grid > 0x7fffffffLL) { set_error("csr_gemm_tn_f32: too many workgroups"); return CN_ERR_SHAPE; }
-    hipLaunchKernelGGL(csr_gemm_tn_kernel, dim3((unsigned)grid), dim3(kT), lds, st, R, Cc, N, row_ptr, col_idx, vals, B, ldb,
-                       out, ldo, (float *)ctx->workspace, col_blocks, row_blocks, splits, rows_per_split);
+    const int wide = ctx->num_cu * 8;
+    int64_t *total_dev = reinterpret_cast<int64_t *>(ctx->sum_scratch);
+    hipLaunchKernelGGL(zero_counts_kernel, dim3(wide), dim3(kT), 0, st, t_row_ptr, Cc + 1);
     CN_HIP(hipGetLastError());
-    if (splits > 1) return add_chunk_planes(ctx, splits, Cc, N, out, ldo, nullptr, st);
+    if (nnz > 0) {
+        hipLaunchKernelGGL(histogram_kernel, dim3(wide), dim3(kT), 0, st, col_idx, nnz, t_row_ptr);
+        CN_HIP(hipGetLastError());
+    }
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kT), 0, st, t_row_ptr, Cc, t_row_ptr, total_dev);
+    CN_HIP(hipGetLastError());
+    if (nnz == 0) return CN_OK;
+    hipLaunchKernelGGL(copy_i32_kernel, dim3(wide), dim3(kT), 0, st, t_row_ptr, scratch, Cc);
+    CN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)(R < wide ? (R > 0 ? R : 1) : wide)), dim3(kT), 0, st, R, row_ptr,
+                       col_idx, vals, scratch, t_col_idx, t_vals);
+    CN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(sort_rows_kernel, dim3(wide), dim3(kT), 0, st, Cc, t_row_ptr, t_col_idx, t_vals);
+    CN_HIP(hipGetLastError());
     return CN_OK;
 }
 

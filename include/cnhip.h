@@ -169,18 +169,18 @@ cn_status cn_csr_from_dense_f32(const float *A_device, int64_t rows, int64_t col
 
 /* out[R x N] = S B with S an R x C CSR matrix and B a dense C x N matrix: every output row gathers the
  * rows of B named by its nonzeros, in ascending order, each term as a rounded product added to the
- * running sum.  dot_sparse, source/clusterNet.cpp:301-401 (cusparseScsrmm2, non-transposed A). */
+ * running sum (reproducible to the bit).  dot_sparse, source/clusterNet.cpp:301-401 (cusparseScsrmm2). */
 cn_status cn_csr_gemm_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
                           const int32_t *col_idx_device, const float *vals_device, const float *B_device,
                           int64_t ldb, float *out_device, int64_t ldo, void *stream);
 
-/* out[C x N] = S^T B with S an R x C CSR matrix and B a dense R x N matrix: B is read once, row k of B is
- * added, scaled, into the output rows named by row k of S.  Tdot_sparse (transposed A of
- * cusparseScsrmm2), source/clusterNet.cpp:304,307.  `splits` > 0 fixes the number of chunks the R rows
- * are cut into (partial outputs are added in ascending order; 1 = none), 0 lets the library choose. */
-cn_status cn_csr_gemm_tn_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
-                             const int32_t *col_idx_device, const float *vals_device, const float *B_device,
-                             int64_t ldb, float *out_device, int64_t ldo, int splits, void *stream);
+/* CSR of S^T from the CSR of the R x C matrix S with nnz nonzeros (t_row_ptr: C + 1 entries, t_col_idx
+ * and t_vals: nnz entries, column indices ascending within a row).  `scratch` is C int32 of device
+ * memory.  With it Tdot_sparse (the transposed operand of cusparseScsrmm2, source/clusterNet.cpp:304,307)
+ * is cn_csr_gemm_f32 on the transposed arrays. */
+cn_status cn_csr_transpose(int64_t R, int64_t C, int64_t nnz, const int32_t *row_ptr_device,
+                           const int32_t *col_idx_device, const float *vals_device, int32_t *t_row_ptr_device,
+                           int32_t *t_col_idx_device, float *t_vals_device, int32_t *scratch_device, void *stream);
 
 /* ---- small kernels used around the path by its callers (row-major, flat where no shape is given).
  * They are not on the measured hot path; each names the reference routine it stands in for. */

@@ -40,7 +40,6 @@ def _load():
     lib.cn_oracle_csr_from_dense.argtypes = [_f32p, _c.c_int64, _c.c_int64, _c.c_int, _i32p, _c.c_void_p, _c.c_void_p]
     lib.cn_oracle_csr_from_dense.restype = _c.c_int64
     lib.cn_oracle_csr_gemm.argtypes = [_c.c_int64, _c.c_int64, _i32p, _i32p, _f32p, _f32p, _f32p]
-    lib.cn_oracle_csr_gemm_tn.argtypes = [_c.c_int64, _c.c_int64, _c.c_int64, _i32p, _i32p, _f32p, _f32p, _f32p, _c.c_int]
     lib.cn_oracle_absmax.argtypes = [_f32p, _c.c_size_t]
     lib.cn_oracle_absmax.restype = _c.c_float
     g = [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _f32p, _c.c_int64, _f32p,
@@ -149,15 +148,6 @@ def csr_gemm(csr, B):
     B = _f32(B)
     out = np.empty((row_ptr.size - 1, B.shape[1]), np.float32)
     _lib.cn_oracle_csr_gemm(row_ptr.size - 1, B.shape[1], row_ptr, col_idx, vals, B, out)
-    return out
-
-
-def csr_gemm_tn(csr, cols, B, splits=1):
-    """S^T B for the R x cols matrix S = (row_ptr, col_idx, vals) and B with R rows."""
-    row_ptr, col_idx, vals = _csr_arrays(csr)
-    B = _f32(B)
-    out = np.empty((cols, B.shape[1]), np.float32)
-    _lib.cn_oracle_csr_gemm_tn(row_ptr.size - 1, cols, B.shape[1], row_ptr, col_idx, vals, B, out, int(splits))
     return out
 
 

@@ -20,7 +20,7 @@
  *                                0 and 1, zero gradient, and an fp64 evaluation of the same formula
  *                                (tests/test_oracle_codec.py)
  *   cn_oracle_csr_from_dense     dense_to_sparse, source/clusterNet.cpp:1004-1032 (cusparseSnnz +
- *   cn_oracle_csr_gemm(_tn)      cusparseSdense2csr) and dot_sparse / Tdot_sparse, :301-401
+ *   cn_oracle_csr_gemm           cusparseSdense2csr) and dot_sparse / Tdot_sparse, :301-401
  *                                (cusparseScsrmm2).  cuSPARSE is closed source; what it computes is the
  *                                textbook CSR layout and product, restated here with sums in ascending
  *                                index order.  Pinned by scipy.sparse (layout) and by the dense
@@ -211,29 +211,6 @@ void cn_oracle_csr_gemm(int64_t R, int64_t N, const int32_t *row_ptr, const int3
             }
             out[r * N + n] = acc;
         }
-}
-
-/* out[C x N] = S^T B, the rows of S taken in ascending order within each of `splits` equal chunks,
- * chunk sums added in ascending order (splits = 1: one running sum). */
-void cn_oracle_csr_gemm_tn(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
-                           const float *vals, const float *B, float *out, int splits) {
-    const int64_t per = (R + splits - 1) / (splits > 0 ? splits : 1);
-    float *part = (float *)malloc((size_t)(C * N ? C * N : 1) * sizeof(float));
-    for (int64_t i = 0; i < C * N; ++i) out[i] = 0.0f;
-    for (int64_t k0 = 0, chunk = 0; k0 < R || chunk == 0; k0 += per, ++chunk) {
-        const int64_t k1 = k0 + per < R ? k0 + per : R;
-        for (int64_t i = 0; i < C * N; ++i) part[i] = 0.0f;
-        for (int64_t k = k0; k < k1; ++k)
-            for (int32_t j = row_ptr[k]; j < row_ptr[k + 1]; ++j)
-                for (int64_t n = 0; n < N; ++n) {
-                    volatile float term = vals[j] * B[k * N + n];
-                    part[(int64_t)col_idx[j] * N + n] = part[(int64_t)col_idx[j] * N + n] + term;
-                }
-        if (chunk == 0) memcpy(out, part, (size_t)(C * N) * sizeof(float));
-        else for (int64_t i = 0; i < C * N; ++i) out[i] = out[i] + part[i];
-        if (per <= 0) break;
-    }
-    free(part);
 }
 
 /* max_i |x_i|, start value -1 as in the reference's reduction; NaN propagates. */

@@ -1,6 +1,6 @@
-"""Parity of the sparse (CSR) path with the CPU checker through the C-ABI: layout bit for bit, the
-gather product bit for bit (same summation order), the scatter product bit for bit when the chunking
-is given and within the GEMM tolerance of the fp64 dense product otherwise."""
+"""Parity of the sparse (CSR) path with the CPU checker through the C-ABI: layout, transposition and
+product bit for bit (the product sums in the checker's order), and the products of the training step
+within the GEMM tolerance of the fp64 dense product."""
 import numpy as np
 import pytest
 
@@ -81,31 +81,23 @@ def test_gather_product_is_bit_exact(dev, R, Cc, N, density):
     assert np.array_equal(_bits(got), _bits(want))
 
 
-@pytest.mark.parametrize("R,Cc,N,density", [(211, 37, 19, 0.05), (5000, 128, 1024, 0.02), (3000, 64, 300, 0.1),
-                                            (9, 5, 1, 0.5), (1000, 300, 520, 0.05), (40, 16, 7, 0.0)])
-def test_scatter_product(dev, R, Cc, N, density):
+@pytest.mark.parametrize("shape,density", [((1, 1), 1.0), ((7, 11), 0.3), ((128, 5000), 0.02), ((300, 257), 0.1),
+                                           ((5, 1000), 0.0), ((64, 64), 1.0), ((1000, 3), 0.5)])
+def test_csr_transpose_equals_csr_of_the_transpose(dev, shape, density):
     from clusternet_amd import _lib as L
-    rng = np.random.default_rng(R + N + 1)
-    S_dense = _sparse(rng, R, Cc, density)
-    B = rng.normal(0, 1, (R, N)).astype(np.float32)
-    S = L.csr_from_dense(_t(S_dense, dev))
-    csr = oracle.csr_from_dense(S_dense)
-    for splits in (1, 3):
-        got = L.csr_gemm_tn(S, _t(B, dev), splits=splits).cpu().numpy()
-        eff = -(-R // -(-R // splits))             # chunks actually formed
-        want = oracle.csr_gemm_tn(csr, Cc, B, eff)
-        assert np.array_equal(_bits(got), _bits(want)), splits
-    got = L.csr_gemm_tn(S, _t(B, dev)).cpu().numpy()      # library's own chunking
-    ref = S_dense.T.astype(np.float64) @ B.astype(np.float64)
-    scale = np.abs(S_dense.T.astype(np.float64)) @ np.abs(B.astype(np.float64))
-    tol = gemm_tolerance(R)
-    assert np.max(np.abs(got - ref)) <= tol * max(np.max(np.abs(ref)), 1e-30)
-    assert np.all(np.abs(got - ref) <= tol * np.maximum(scale, 1e-30))
+    rng = np.random.default_rng(shape[0] * 17 + shape[1])
+    A = _sparse(rng, *shape, density)
+    T = L.csr_transpose(L.csr_from_dense(_t(A, dev)))
+    row_ptr, col_idx, vals = oracle.csr_from_dense(A, transpose=True)
+    assert (T.rows, T.cols) == (shape[1], shape[0])
+    assert np.array_equal(T.row_ptr.cpu().numpy(), row_ptr)
+    assert np.array_equal(T.col_idx.cpu().numpy(), col_idx)
+    assert np.array_equal(_bits(T.vals.cpu().numpy()), _bits(vals))
 
 
-def test_batch_products_through_the_transposed_csr(dev):
-    """The two products of the training step on a 2 % dense batch: X W = S^T W and X^T E = S E with
-    S = CSR(X^T); against the dense kernels of this library and the fp64 product."""
+def test_batch_products(dev):
+    """The two products of the training step on a 2 % dense batch: X W = CSR(X) W and
+    X^T E = CSR(X^T) E; against the dense kernels of this library, the fp64 product and the checker."""
     import torch
     import clusternet_amd as cn
     from clusternet_amd import _lib as L
@@ -114,9 +106,11 @@ def test_batch_products_through_the_transposed_csr(dev):
     W = rng.uniform(-0.01, 0.01, (6000, 2048)).astype(np.float32)
     E = rng.normal(0, 0.01, (128, 2048)).astype(np.float32)
     Xt, Wt, Et = _t(X, dev), _t(W, dev), _t(E, dev)
-    S = L.csr_from_dense(Xt, transpose=True)
+    Sx = L.csr_from_dense(Xt)
+    S = L.csr_transpose(Sx)
     assert (S.rows, S.cols) == (6000, 128)
-    fwd = L.csr_gemm_tn(S, Wt).cpu().numpy()
+    fwd = L.csr_gemm(Sx, Wt).cpu().numpy()
+    assert np.array_equal(_bits(fwd), _bits(oracle.csr_gemm(oracle.csr_from_dense(X), W)))
     ref = X.astype(np.float64) @ W.astype(np.float64)
     assert np.max(np.abs(fwd - ref)) <= gemm_tolerance(6000) * np.max(np.abs(ref))
     assert np.max(np.abs(fwd - cn.dot(Xt, Wt).cpu().numpy())) <= 2 * gemm_tolerance(6000) * np.max(np.abs(ref))
@@ -133,7 +127,6 @@ def test_shape_errors(dev):
     assert S.nnz == 0
     with pytest.raises(L.CnError):
         L.csr_gemm(S, torch.zeros((4, 3), device=dev))
-    with pytest.raises(L.CnError):
-        L.csr_gemm_tn(S, torch.zeros((5, 3), device=dev))
     assert torch.equal(L.csr_gemm(S, torch.ones((5, 3), device=dev)), torch.zeros((4, 3), device=dev))
-    assert torch.equal(L.csr_gemm_tn(S, torch.ones((4, 3), device=dev)), torch.zeros((5, 3), device=dev))
+    T = L.csr_transpose(S)
+    assert (T.rows, T.cols, T.nnz) == (5, 4, 0) and int(T.row_ptr.abs().sum()) == 0
