@@ -50,6 +50,7 @@ def lib():
     L.cn_csr_from_dense_f32.argtypes = [vp, i64, i64, i64, C.c_int, vp, vp, vp, i64, C.POINTER(i64), vp]
     L.cn_csr_gemm_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp]
     L.cn_csr_transpose.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp]
+    L.cn_csr_to_dense_f32.argtypes = [i64, i64, vp, vp, vp, vp, i64, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
     L.cn_compress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
@@ -203,6 +204,16 @@ def csr_gemm(S, B, out=None):
     _need(out, torch.float32, "out")
     check(lib().cn_csr_gemm_f32(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
                                 B.data_ptr(), _ld(B), out.data_ptr(), _ld(out), _stream()))
+    return out
+
+
+def csr_to_dense(S, out=None):
+    import torch
+    if out is None:
+        out = torch.empty((S.rows, S.cols), dtype=torch.float32, device=S.row_ptr.device)
+    _need(out, torch.float32, "out")
+    check(lib().cn_csr_to_dense_f32(S.rows, S.cols, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                    out.data_ptr(), _ld(out), _stream()))
     return out
 
 

@@ -28,19 +28,32 @@ inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_
 // ---- dense -> CSR ----------------------------------------------------------------------------------
 // counts[i] = number of nonzeros of row i of op(A); op = identity or transpose.  A value is a nonzero
 // when it compares unequal to 0 (so -0.0 is dropped and NaN is kept).
-__global__ __launch_bounds__(kT) void count_rows_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
-                                                        int64_t lda, int32_t *__restrict__ counts) {
-    // one workgroup per row of A
+// A row is cut into segments of kSegment columns so that a short, wide matrix still fills the machine.
+constexpr int64_t kSegment = 4096;
+
+// counts[r * segments + g] = nonzeros of columns [g kSegment, (g + 1) kSegment) of row r; one workgroup
+// per (row, segment).
+__global__ __launch_bounds__(kT) void count_segments_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
+                                                            int64_t lda, int64_t segments, int32_t *__restrict__ counts) {
     __shared__ int partial[kT / 64];
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    for (int64_t unit = blockIdx.x; unit < rows * segments; unit += gridDim.x) {
+        const int64_t r = unit / segments, j0 = (unit % segments) * kSegment;
+        const int64_t j1 = (j0 + kSegment < cols) ? j0 + kSegment : cols;
         int c = 0;
-        for (int64_t j = threadIdx.x; j < cols; j += kT) c += (A[r * lda + j] != 0.0f) ? 1 : 0;
+        for (int64_t j = j0 + threadIdx.x; j < j1; j += kT) c += (A[r * lda + j] != 0.0f) ? 1 : 0;
         for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
         if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = c;
         __syncthreads();
-        if (threadIdx.x == 0) counts[r] = partial[0] + partial[1] + partial[2] + partial[3];
+        if (threadIdx.x == 0) counts[unit] = partial[0] + partial[1] + partial[2] + partial[3];
         __syncthreads();
     }
+}
+
+// row_ptr[r] = offset of the first segment of row r; row_ptr[rows] = offsets[rows * segments].
+__global__ __launch_bounds__(kT) void row_ptr_from_segments_kernel(const int32_t *__restrict__ offsets, int64_t rows,
+                                                                   int64_t segments, int32_t *__restrict__ row_ptr) {
+    for (int64_t r = (int64_t)blockIdx.x * kT + threadIdx.x; r <= rows; r += (int64_t)gridDim.x * kT)
+        row_ptr[r] = offsets[r * segments];
 }
 
 __global__ __launch_bounds__(kT) void count_cols_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
@@ -57,46 +70,97 @@ __global__ __launch_bounds__(kT) void zero_counts_kernel(int32_t *__restrict__ c
     for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) counts[i] = 0;
 }
 
-// row_ptr[0 .. n] = exclusive prefix sums of counts[0 .. n - 1] (in place: counts == row_ptr is allowed
-// because every thread reads its run before any thread writes); *total = row_ptr[n].  One workgroup.
+// row_ptr[0 .. n] = exclusive prefix sums of counts[0 .. n - 1]; counts == row_ptr is allowed (a tile is
+// read completely before it is written); *total = row_ptr[n].  One workgroup walks the array in tiles
+// of 256 with coalesced accesses; a tile is scanned by shuffles inside each wavefront and a four-entry
+// table across wavefronts.
 __global__ __launch_bounds__(kT) void scan_kernel(const int32_t *counts, int64_t n, int32_t *row_ptr,
                                                   int64_t *__restrict__ total) {
-    __shared__ int64_t sums[kT];
-    const int64_t per = (n + kT - 1) / kT;
-    const int64_t lo = (int64_t)threadIdx.x * per, hi = (lo + per < n) ? lo + per : n;
-    int64_t s = 0;
-    for (int64_t i = lo; i < hi; ++i) s += counts[i];
-    sums[threadIdx.x] = s;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int64_t run = 0;
-        for (int i = 0; i < kT; ++i) { const int64_t v = sums[i]; sums[i] = run; run += v; }
-        *total = run;
+    __shared__ int wave_sum[kT / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int64_t carry = 0;
+    for (int64_t i0 = 0; i0 < n; i0 += kT) {
+        const int64_t i = i0 + threadIdx.x;
+        const int c = (i < n) ? counts[i] : 0;
+        int inc = c;  // inclusive scan within the wavefront
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(inc, off, 64);
+            if (lane >= off) inc += up;
+        }
+        if (lane == 63) wave_sum[wave] = inc;
+        __syncthreads();
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += wave_sum[w];
+        const int tile_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+        if (i < n) row_ptr[i] = (int32_t)(carry + before + inc - c);
+        carry += tile_total;
+        __syncthreads();
     }
-    __syncthreads();
-    int64_t run = sums[threadIdx.x];
-    for (int64_t i = lo; i < hi; ++i) {
-        const int32_t c = counts[i];
-        row_ptr[i] = (int32_t)run;
-        run += c;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) row_ptr[n] = (int32_t)*total;
+    if (threadIdx.x == 0) { row_ptr[n] = (int32_t)carry; *total = carry; }
 }
 
-// CSR of A: one workgroup per row, columns compacted in ascending order.
-__global__ __launch_bounds__(kT) void fill_rows_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
-                                                       int64_t lda, const int32_t *__restrict__ row_ptr,
-                                                       int32_t *__restrict__ col_idx, float *__restrict__ vals) {
+// Prefix sums of a long array in three launches: sums of blocks of kScanBlock elements, their prefix
+// sums (scan_kernel), then every block scans itself from its offset.
+constexpr int64_t kScanBlock = 4096;
+
+__global__ __launch_bounds__(kT) void block_sums_kernel(const int32_t *__restrict__ counts, int64_t n,
+                                                        int32_t *__restrict__ sums) {
+    __shared__ int partial[kT / 64];
+    const int64_t i0 = (int64_t)blockIdx.x * kScanBlock;
+    const int64_t i1 = (i0 + kScanBlock < n) ? i0 + kScanBlock : n;
+    int c = 0;
+    for (int64_t i = i0 + threadIdx.x; i < i1; i += kT) c += counts[i];
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) sums[blockIdx.x] = partial[0] + partial[1] + partial[2] + partial[3];
+}
+
+__global__ __launch_bounds__(kT) void block_scan_kernel(const int32_t *counts, int64_t n,
+                                                        const int32_t *__restrict__ block_offsets, int32_t *row_ptr,
+                                                        const int64_t *__restrict__ total) {
+    __shared__ int wave_sum[kT / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t b0 = (int64_t)blockIdx.x * kScanBlock;
+    const int64_t b1 = (b0 + kScanBlock < n) ? b0 + kScanBlock : n;
+    int64_t carry = block_offsets[blockIdx.x];
+    for (int64_t i0 = b0; i0 < b1; i0 += kT) {
+        const int64_t i = i0 + threadIdx.x;
+        const int c = (i < b1) ? counts[i] : 0;
+        int inc = c;
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(inc, off, 64);
+            if (lane >= off) inc += up;
+        }
+        if (lane == 63) wave_sum[wave] = inc;
+        __syncthreads();
+        int before = 0;
+        for (int w = 0; w < wave; ++w) before += wave_sum[w];
+        const int tile_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+        if (i < b1) row_ptr[i] = (int32_t)(carry + before + inc - c);
+        carry += tile_total;
+        __syncthreads();
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) row_ptr[n] = (int32_t)*total;
+}
+
+// CSR of A: one workgroup per (row, segment), columns compacted in ascending order from the
+// segment's offset.
+__global__ __launch_bounds__(kT) void fill_segments_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
+                                                           int64_t lda, int64_t segments,
+                                                           const int32_t *__restrict__ offsets,
+                                                           int32_t *__restrict__ col_idx, float *__restrict__ vals) {
     __shared__ int wave_count[kT / 64];
     __shared__ int base;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-        if (threadIdx.x == 0) base = row_ptr[r];
+    for (int64_t unit = blockIdx.x; unit < rows * segments; unit += gridDim.x) {
+        const int64_t r = unit / segments, s0 = (unit % segments) * kSegment;
+        const int64_t s1 = (s0 + kSegment < cols) ? s0 + kSegment : cols;
+        if (threadIdx.x == 0) base = offsets[unit];
         __syncthreads();
-        for (int64_t j0 = 0; j0 < cols; j0 += kT) {
+        for (int64_t j0 = s0; j0 < s1; j0 += kT) {
             const int64_t j = j0 + threadIdx.x;
-            const float v = (j < cols) ? A[r * lda + j] : 0.0f;
+            const float v = (j < s1) ? A[r * lda + j] : 0.0f;
             const bool keep = v != 0.0f;
             const unsigned long long mask = __ballot(keep);
             const int before = __popcll(mask & ((1ull << lane) - 1ull));
@@ -127,8 +191,8 @@ __global__ __launch_bounds__(kT) void fill_cols_kernel(const float *__restrict__
 
 // ---- out = S B (gather) ---------------------------------------------------------------------------------
 // A workgroup owns a block of 1024 columns (4 per lane) and walks a range of output rows.  The
-// nonzeros of a row are taken eight at a time: indices and values first, then the eight B rows, then
-// the eight multiply-adds in order.
+// nonzeros of a row are taken eight at a time while eight are left: indices and values first, then the
+// eight B rows, then the eight multiply-adds in order.
 constexpr int kGather = 8;
 
 template <bool kVector>
@@ -144,21 +208,22 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
         if (kVector) {
             if (n >= N) continue;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            for (int32_t j = j0; j < j1; j += kGather) {
+            int32_t j = j0;
+            for (; j + kGather <= j1; j += kGather) {
                 int32_t c[kGather];
                 float v[kGather];
                 f32x4 b[kGather];
 #pragma unroll
-                for (int u = 0; u < kGather; ++u) {
-                    const int32_t at = (j + u < j1) ? j + u : j1 - 1;  // past the end: a valid, unused address
-                    c[u] = col_idx[at];
-                    v[u] = vals[at];
-                }
+                for (int u = 0; u < kGather; ++u) { c[u] = col_idx[j + u]; v[u] = vals[j + u]; }
 #pragma unroll
                 for (int u = 0; u < kGather; ++u) b[u] = *reinterpret_cast<const f32x4 *>(B + (int64_t)c[u] * ldb + n);
 #pragma unroll
-                for (int u = 0; u < kGather; ++u)
-                    if (j + u < j1) acc = acc + v[u] * b[u];
+                for (int u = 0; u < kGather; ++u) acc = acc + v[u] * b[u];
+            }
+            for (; j < j1; ++j) {
+                const float v = vals[j];
+                const f32x4 b = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + n);
+                acc = acc + v * b;
             }
             __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(out + r * ldo + n));
         } else {
@@ -214,8 +279,40 @@ __global__ __launch_bounds__(kT) void sort_rows_kernel(int64_t R, const int32_t 
     }
 }
 
+// out = dense form of S: zero fill, then one workgroup per row writes its nonzeros.
+__global__ __launch_bounds__(kT) void csr_to_dense_kernel(int64_t R, int64_t Cc, const int32_t *__restrict__ row_ptr,
+                                                          const int32_t *__restrict__ col_idx,
+                                                          const float *__restrict__ vals, float *__restrict__ out,
+                                                          int64_t ldo) {
+    for (int64_t r = blockIdx.x; r < R; r += gridDim.x) {
+        for (int64_t j = threadIdx.x; j < Cc; j += kT) out[r * ldo + j] = 0.0f;
+        __syncthreads();
+        for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) out[r * ldo + col_idx[j]] = vals[j];
+        __syncthreads();
+    }
+}
+
 __global__ __launch_bounds__(kT) void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
     for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) dst[i] = src[i];
+}
+
+// row_ptr[0 .. n] = exclusive prefix sums of counts[0 .. n - 1] (in place allowed), *total_dev = their sum.
+cn_status exclusive_scan(Context *ctx, const int32_t *counts, int64_t n, int32_t *row_ptr, int64_t *total_dev,
+                         hipStream_t st) {
+    const int64_t blocks = (n + kScanBlock - 1) / kScanBlock;
+    if (blocks <= 2 || blocks + 1 > kReduceSlots) {  // the scratch holds kReduceSlots words before its counter
+        hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kT), 0, st, counts, n, row_ptr, total_dev);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
+    int32_t *sums = reinterpret_cast<int32_t *>(ctx->reduce_scratch);
+    hipLaunchKernelGGL(block_sums_kernel, dim3((unsigned)blocks), dim3(kT), 0, st, counts, n, sums);
+    CN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kT), 0, st, sums, blocks, sums, total_dev);
+    CN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(block_scan_kernel, dim3((unsigned)blocks), dim3(kT), 0, st, counts, n, sums, row_ptr, total_dev);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
 }
 
 cn_status check_csr_args(const char *who, int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr,
@@ -250,22 +347,34 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
     const int64_t out_rows = transpose ? cols : rows;
     int64_t *total_dev = reinterpret_cast<int64_t *>(ctx->sum_scratch);  // 8 bytes of the reduction scratch
     const int wide = ctx->num_cu * 8;
-    if (rows > 0 && cols > 0) {
-        if (transpose) {
-            const int64_t blocks = (cols + kT - 1) / kT;
-            hipLaunchKernelGGL(count_cols_kernel, dim3((unsigned)(blocks < wide ? blocks : wide)), dim3(kT), 0, st, A, rows,
-                               cols, lda, row_ptr);
-        } else {
-            hipLaunchKernelGGL(count_rows_kernel, dim3((unsigned)(rows < wide ? rows : wide)), dim3(kT), 0, st, A, rows, cols,
-                               lda, row_ptr);
-        }
+    const int64_t segments = (cols + kSegment - 1) / kSegment;
+    const int64_t units = rows * segments;
+    int32_t *offsets = reinterpret_cast<int32_t *>(ctx->workspace);  // per (row, segment), transpose == 0 only
+    if (!transpose && (size_t)(units + 1) * sizeof(int32_t) > ctx->workspace_bytes) {
+        set_error("csr_from_dense_f32: matrix too large for the workspace");
+        return CN_ERR_WORKSPACE;
+    }
+    if (rows > 0 && cols > 0 && transpose) {
+        const int64_t blocks = (cols + kT - 1) / kT;
+        hipLaunchKernelGGL(count_cols_kernel, dim3((unsigned)(blocks < wide ? blocks : wide)), dim3(kT), 0, st, A, rows, cols,
+                           lda, row_ptr);
         CN_HIP(hipGetLastError());
-    } else if (out_rows > 0) {
-        hipLaunchKernelGGL(zero_counts_kernel, dim3(wide), dim3(kT), 0, st, row_ptr, out_rows);
+        { cn_status sc = exclusive_scan(ctx, row_ptr, out_rows, row_ptr, total_dev, st); if (sc != CN_OK) return sc; }
+    } else if (rows > 0 && cols > 0) {
+        hipLaunchKernelGGL(count_segments_kernel, dim3((unsigned)(units < wide ? units : wide)), dim3(kT), 0, st, A, rows, cols,
+                           lda, segments, offsets);
+        CN_HIP(hipGetLastError());
+        { cn_status sc = exclusive_scan(ctx, offsets, units, offsets, total_dev, st); if (sc != CN_OK) return sc; }
+        const int64_t blocks = (rows + kT) / kT;
+        hipLaunchKernelGGL(row_ptr_from_segments_kernel, dim3((unsigned)(blocks < wide ? blocks : wide)), dim3(kT), 0, st, offsets,
+                           rows, segments, row_ptr);
+        CN_HIP(hipGetLastError());
+    } else {
+        hipLaunchKernelGGL(zero_counts_kernel, dim3(wide), dim3(kT), 0, st, row_ptr, out_rows + 1);
+        CN_HIP(hipGetLastError());
+        hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kT), 0, st, row_ptr, (int64_t)0, row_ptr, total_dev);
         CN_HIP(hipGetLastError());
     }
-    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kT), 0, st, row_ptr, out_rows, row_ptr, total_dev);
-    CN_HIP(hipGetLastError());
     CN_HIP(hipMemcpyAsync(nnz_host, total_dev, sizeof(int64_t), hipMemcpyDeviceToHost, st));
     CN_HIP(hipStreamSynchronize(st));
     if (*nnz_host > 0x7fffffffLL) { set_error("csr_from_dense_f32: more than 2^31 nonzeros"); return CN_ERR_SHAPE; }
@@ -280,8 +389,8 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
         hipLaunchKernelGGL(fill_cols_kernel, dim3((unsigned)(blocks < wide ? blocks : wide)), dim3(kT), 0, st, A, rows, cols,
                            lda, row_ptr, col_idx, vals);
     } else {
-        hipLaunchKernelGGL(fill_rows_kernel, dim3((unsigned)(rows < wide ? rows : wide)), dim3(kT), 0, st, A, rows, cols, lda,
-                           row_ptr, col_idx, vals);
+        hipLaunchKernelGGL(fill_segments_kernel, dim3((unsigned)(units < wide ? units : wide)), dim3(kT), 0, st, A, rows, cols,
+                           lda, segments, offsets, col_idx, vals);
     }
     CN_HIP(hipGetLastError());
     return CN_OK;
@@ -311,6 +420,22 @@ cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_p
     return CN_OK;
 }
 
+cn_status cn_csr_to_dense_f32(int64_t R, int64_t Cc, const int32_t *row_ptr, const int32_t *col_idx, const float *vals,
+                              float *out, int64_t ldo, void *stream) {
+    if (R < 0 || Cc < 0 || ldo < Cc) { set_error("csr_to_dense_f32: bad dimensions"); return CN_ERR_SHAPE; }
+    if (R == 0 || Cc == 0) return CN_OK;
+    if (!row_ptr || !out) { set_error("csr_to_dense_f32: NULL pointer"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t wide = (int64_t)ctx->num_cu * 8;
+    hipLaunchKernelGGL(csr_to_dense_kernel, dim3((unsigned)(R < wide ? R : wide)), dim3(kT), 0, st, R, Cc, row_ptr, col_idx, vals,
+                       out, ldo);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
 cn_status cn_csr_transpose(int64_t R, int64_t Cc, int64_t nnz, const int32_t *row_ptr, const int32_t *col_idx,
                            const float *vals, int32_t *t_row_ptr, int32_t *t_col_idx, float *t_vals,
                            int32_t *scratch, void *stream) {
@@ -334,8 +459,7 @@ cn_status cn_csr_transpose(int64_t R, int64_t Cc, int64_t nnz, const int32_t *ro
         hipLaunchKernelGGL(histogram_kernel, dim3(wide), dim3(kT), 0, st, col_idx, nnz, t_row_ptr);
         CN_HIP(hipGetLastError());
     }
-    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kT), 0, st, t_row_ptr, Cc, t_row_ptr, total_dev);
-    CN_HIP(hipGetLastError());
+    { cn_status sc = exclusive_scan(ctx, t_row_ptr, Cc, t_row_ptr, total_dev, st); if (sc != CN_OK) return sc; }
     if (nnz == 0) return CN_OK;
     hipLaunchKernelGGL(copy_i32_kernel, dim3(wide), dim3(kT), 0, st, t_row_ptr, scratch, Cc);
     CN_HIP(hipGetLastError());

@@ -105,6 +105,113 @@ Matrix *ClusterNet::dot8bit_weights(Matrix *A, Matrix *B, float precisionB) {
     return out;
 }
 
+// ---- sparse operands -----------------------------------------------------------------------------
+static void require_sparse(Matrix *A) {
+    if (!A->isSparse) {
+        printf("Error: the first operand must be a sparse matrix (dense_to_sparse).\n");
+        throw "Matrix *size error:\n";
+    }
+}
+
+static Matrix *sparse_shell(int rows, int cols, long long nnz) {
+    Matrix *out = (Matrix *)calloc(1, sizeof(Matrix));
+    out->rows = rows;
+    out->cols = cols;
+    out->size = nnz;
+    out->bytes = (size_t)nnz * sizeof(float);
+    out->idx_bytes = (size_t)nnz * sizeof(int);
+    out->ptr_bytes = (size_t)(rows + 1) * sizeof(int);
+    out->isSparse = 1;
+    void *p = nullptr;
+    cn_throw_on_error(cn_malloc(&p, out->ptr_bytes));
+    out->ptr_rows = (int *)p;
+    cn_throw_on_error(cn_malloc(&p, out->idx_bytes ? out->idx_bytes : 4));
+    out->idx_cols = (int *)p;
+    cn_throw_on_error(cn_malloc(&p, out->bytes ? out->bytes : 4));
+    out->data = (float *)p;
+    return out;
+}
+
+static void free_sparse(Matrix *A) {
+    cn_free(A->data);
+    cn_free(A->idx_cols);
+    cn_free(A->ptr_rows);
+    free(A);
+}
+
+Matrix *ClusterNet::dense_to_sparse(Matrix *A) {
+    // first call sizes the arrays (capacity 0 reports the count), second call fills them
+    void *ptr = nullptr;
+    cn_throw_on_error(cn_malloc(&ptr, (size_t)(A->rows + 1) * sizeof(int)));
+    int64_t nnz = 0;
+    int status = cn_csr_from_dense_f32(A->data, A->rows, A->cols, A->cols, 0, (int *)ptr, nullptr, nullptr, 0, &nnz, nullptr);
+    cn_free(ptr);
+    if (status != CN_OK && status != CN_ERR_WORKSPACE) cn_throw_on_error(status);
+    Matrix *out = sparse_shell(A->rows, A->cols, nnz);
+    cn_throw_on_error(cn_csr_from_dense_f32(A->data, A->rows, A->cols, A->cols, 0, out->ptr_rows, out->idx_cols, out->data,
+                                            nnz, &nnz, nullptr));
+    return out;
+}
+
+Matrix *ClusterNet::sparse_to_dense(Matrix *A) {
+    require_sparse(A);
+    Matrix *out = empty(A->rows, A->cols);
+    cn_throw_on_error(cn_csr_to_dense_f32(A->rows, A->cols, A->ptr_rows, A->idx_cols, A->data, out->data, out->cols, nullptr));
+    return out;
+}
+
+void ClusterNet::dot_sparse(Matrix *A, Matrix *B, Matrix *out) {
+    require_sparse(A);
+    if (A->cols != B->rows || out->rows != A->rows || out->cols != B->cols) {
+        printf("Error: dot_sparse %ix%i times %ix%i into %ix%i.\n", A->rows, A->cols, B->rows, B->cols, out->rows, out->cols);
+        throw "Matrix *size error:\n";
+    }
+    cn_throw_on_error(cn_csr_gemm_f32(A->rows, A->cols, B->cols, A->ptr_rows, A->idx_cols, A->data, B->data, B->cols,
+                                      out->data, out->cols, nullptr));
+}
+
+void ClusterNet::Tdot_sparse(Matrix *A, Matrix *B, Matrix *out) {
+    require_sparse(A);
+    if (A->rows != B->rows || out->rows != A->cols || out->cols != B->cols) {
+        printf("Error: Tdot_sparse (%ix%i)^T times %ix%i into %ix%i.\n", A->rows, A->cols, B->rows, B->cols, out->rows, out->cols);
+        throw "Matrix *size error:\n";
+    }
+    Matrix *At = sparse_shell(A->cols, A->rows, A->size);
+    void *scratch = nullptr;
+    cn_throw_on_error(cn_malloc(&scratch, (size_t)(A->cols > 0 ? A->cols : 1) * sizeof(int)));
+    cn_throw_on_error(cn_csr_transpose(A->rows, A->cols, A->size, A->ptr_rows, A->idx_cols, A->data, At->ptr_rows, At->idx_cols,
+                                       At->data, (int *)scratch, nullptr));
+    cn_throw_on_error(cn_csr_gemm_f32(At->rows, At->cols, B->cols, At->ptr_rows, At->idx_cols, At->data, B->data, B->cols,
+                                      out->data, out->cols, nullptr));
+    cn_throw_on_error(cn_synchronize(nullptr));
+    cn_free(scratch);
+    free_sparse(At);
+}
+
+void ClusterNet::dotT_sparse(Matrix *A, Matrix *B, Matrix *out) {
+    require_sparse(A);
+    Matrix *Bt = T(B);
+    dot_sparse(A, Bt, out);
+    cn_throw_on_error(cn_synchronize(nullptr));
+    free_matrix(Bt);
+}
+
+Matrix *ClusterNet::dot_sparse(Matrix *A, Matrix *B) {
+    Matrix *out = empty(A->rows, B->cols);
+    dot_sparse(A, B, out);
+    return out;
+}
+Matrix *ClusterNet::Tdot_sparse(Matrix *A, Matrix *B) {
+    Matrix *out = empty(A->cols, B->cols);
+    Tdot_sparse(A, B, out);
+    return out;
+}
+Matrix *ClusterNet::dotT_sparse(Matrix *A, Matrix *B) {
+    Matrix *out = empty(A->rows, B->rows);
+    dotT_sparse(A, B, out);
+    return out;
+}
+
 static Matrix *upload(const std::vector<float> &host, int rows, int cols) {
     Matrix *out = empty(rows, cols);
     cn_throw_on_error(cn_memcpy_h2d(out->data, host.data(), out->bytes));

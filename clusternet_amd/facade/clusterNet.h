@@ -50,6 +50,17 @@ public:
     Matrix *dot8bit_weights(Matrix *A, Matrix *B, float precisionB);
     void dot8bit_weights(Matrix *A, Matrix *B, float precisionB, Matrix *out);
 
+    // Sparse operands (source/clusterNet.cpp:301-401,1004-1063): A is a sparse Matrix as made by
+    // dense_to_sparse (isSparse = 1; data = values, idx_cols, ptr_rows, size = number of nonzeros).
+    Matrix *dense_to_sparse(Matrix *A);
+    Matrix *sparse_to_dense(Matrix *A);
+    Matrix *dot_sparse(Matrix *A, Matrix *B);    // A B
+    Matrix *Tdot_sparse(Matrix *A, Matrix *B);   // A^T B
+    Matrix *dotT_sparse(Matrix *A, Matrix *B);   // A B^T
+    void dot_sparse(Matrix *A, Matrix *B, Matrix *out);
+    void Tdot_sparse(Matrix *A, Matrix *B, Matrix *out);
+    void dotT_sparse(Matrix *A, Matrix *B, Matrix *out);
+
     // Input generators of the test and benchmark harness (source/clusterNet.cpp:746-788,874-938).
     // Values come from a host-side generator seeded by the constructor, not from cuRAND.
     Matrix *rand(int rows, int cols);

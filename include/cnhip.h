@@ -174,6 +174,10 @@ cn_status cn_csr_gemm_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_pt
                           const int32_t *col_idx_device, const float *vals_device, const float *B_device,
                           int64_t ldb, float *out_device, int64_t ldo, void *stream);
 
+/* out[R x C] = dense form of S (zeros elsewhere).  sparse_to_dense, source/clusterNet.cpp:1034-1063. */
+cn_status cn_csr_to_dense_f32(int64_t R, int64_t C, const int32_t *row_ptr_device, const int32_t *col_idx_device,
+                              const float *vals_device, float *out_device, int64_t ldo, void *stream);
+
 /* CSR of S^T from the CSR of the R x C matrix S with nnz nonzeros (t_row_ptr: C + 1 entries, t_col_idx
  * and t_vals: nnz entries, column indices ascending within a row).  `scratch` is C int32 of device
  * memory.  With it Tdot_sparse (the transposed operand of cusparseScsrmm2, source/clusterNet.cpp:304,307)

@@ -41,6 +41,13 @@ static bool test_matrix(Matrix *A, int rows, int cols) {
            A->bytes == sizeof(float) * (size_t)rows * cols;
 }
 
+static float max_abs_diff(Matrix *a, Matrix *b) {
+    if (a->size != b->size) return INFINITY;
+    float worst = 0.0f;
+    for (long long i = 0; i < a->size; ++i) worst = fmaxf(worst, fabsf(a->data[i] - b->data[i]));
+    return worst;
+}
+
 static Matrix *host_matrix(int rows, int cols, const float *values) {
     Matrix *m = empty_cpu(rows, cols);
     memcpy(m->data, values, m->bytes);
@@ -220,6 +227,31 @@ static void run_codec_test(ClusterNet gpu) {
         RMSprop_with_weight_update_from_8bit(rms_b, codes, precision, w_b, 0.9f, 0.003f);
         CHECK(memcmp(to_host(rms_b)->data, rms_want.data(), rms->bytes) == 0, "RMSprop on codes: RMS");
         CHECK(memcmp(to_host(w_b)->data, w_want.data(), w->bytes) == 0, "RMSprop on codes: weights");
+    }
+
+    // sparse operands: layout and the three products against the dense ones (the reference's own
+    // criterion is agreement with the dense product, tests/clusterNet_test.cu:396-463)
+    {
+        Matrix *D = gpu.rand(64, 3000);
+        Matrix *mask = gpu.rand(64, 3000);
+        Matrix *dh = to_host(D), *mh = to_host(mask);
+        for (long long i = 0; i < dh->size; ++i) dh->data[i] = mh->data[i] < 0.03f ? dh->data[i] : 0.0f;
+        Matrix *Xs = to_gpu(dh);
+        Matrix *S = gpu.dense_to_sparse(Xs);
+        long long want_nnz = 0;
+        for (long long i = 0; i < dh->size; ++i) want_nnz += dh->data[i] != 0.0f;
+        CHECK(S->isSparse == 1 && S->size == want_nnz && S->rows == 64 && S->cols == 3000, "dense_to_sparse shape and count");
+        Matrix *back_dense = to_host(gpu.sparse_to_dense(S));
+        CHECK(memcmp(back_dense->data, dh->data, dh->bytes) == 0, "sparse_to_dense(dense_to_sparse(X)) == X");
+        Matrix *Wd = gpu.randn(3000, 96, 0.0f, 0.05f);
+        Matrix *Ed = gpu.randn(64, 80, 0.0f, 0.05f);
+        Matrix *Wt = gpu.randn(96, 3000, 0.0f, 0.05f);
+        CHECK(max_abs_diff(to_host(gpu.dot_sparse(S, Wd)), to_host(gpu.dot(Xs, Wd))) < 1e-4f, "dot_sparse == dot");
+        CHECK(max_abs_diff(to_host(gpu.Tdot_sparse(S, Ed)), to_host(gpu.Tdot(Xs, Ed))) < 1e-4f, "Tdot_sparse == Tdot");
+        CHECK(max_abs_diff(to_host(gpu.dotT_sparse(S, Wt)), to_host(gpu.dotT(Xs, Wt))) < 1e-4f, "dotT_sparse == dotT");
+        bool threw = false;
+        try { gpu.dot_sparse(Xs, Wd); } catch (const char *) { threw = true; }
+        CHECK(threw, "dot_sparse refuses a dense first operand");
     }
 
     // fused product on coded weights against dot on the decoded weights
