@@ -209,8 +209,19 @@ def bench_step(torch, cn, dev):
         for w, r, g in zip((W1, W2, W3), rms, state["grads"]):
             ms.coded_rmsprop_update(w, r, g, 0.9, 1e-3, fused=False, scratch=scratch[:g.numel()].view(g.shape))
 
+    def to_sparse():
+        state["Xs"] = ms.sparse_input(X)
+
+    def fwd_sparse():
+        state["p"], state["cache"] = ms.forward(state["Xs"], params, pool)
+
+    def bwd_absmax_sparse():
+        state["grads"] = ms.backward(state["Xs"], onehot, params, state["p"], state["cache"], pool, absmax_out=maxima)
+
     out = {}
-    for name, fn in (("forward", fwd), ("backward_with_absmax", bwd_absmax),
+    for name, fn in (("sparse_input", to_sparse), ("forward_sparse", fwd_sparse),
+                     ("backward_with_absmax_sparse", bwd_absmax_sparse),
+                     ("forward", fwd), ("backward_with_absmax", bwd_absmax),
                      ("compress_and_update_given_absmax", codec_update_given_max),
                      ("backward", bwd), ("codec_and_update", codec_update),
                      ("codec_and_update_unfused", codec_update_unfused), ("codec_and_rmsprop", codec_rmsprop),
@@ -226,6 +237,8 @@ def bench_step(torch, cn, dev):
     out["codec_and_rmsprop_GBps"] = elems * (4 + 5 + 17) / (out["codec_and_rmsprop_ms"] * 1e-3) / 1e9
     out["codec_and_rmsprop_unfused_GBps"] = elems * (4 + 5 + 5 + 20) / (out["codec_and_rmsprop_unfused_ms"] * 1e-3) / 1e9
     out["step_ms"] = out["forward_ms"] + out["backward_with_absmax_ms"] + out["compress_and_update_given_absmax_ms"]
+    out["step_sparse_ms"] = (out["sparse_input_ms"] + out["forward_sparse_ms"] + out["backward_with_absmax_sparse_ms"] +
+                             out["compress_and_update_given_absmax_ms"])
     out["step_unfused_ms"] = out["forward_ms"] + out["backward_ms"] + out["codec_and_update_unfused_ms"]
     out["note"] = ("bytes per gradient element: absmax 4 + compress 5, then fused decode+update 9 (unfused: decompress 5 + "
                    "update 12) or fused decode+RMSprop 17 (unfused 5 + 20); "

@@ -50,6 +50,7 @@ def lib():
     L.cn_csr_from_dense_f32.argtypes = [vp, i64, i64, i64, C.c_int, vp, vp, vp, i64, C.POINTER(i64), vp]
     L.cn_csr_gemm_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp]
     L.cn_csr_transpose.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp]
+    L.cn_csr_gemm_f32_absmax.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp, vp]
     L.cn_csr_to_dense_f32.argtypes = [i64, i64, vp, vp, vp, vp, i64, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
@@ -192,8 +193,9 @@ def csr_from_dense(A, transpose=False):
     return Csr(R, Cc, row_ptr, col_idx[:nnz.value], vals[:nnz.value])
 
 
-def csr_gemm(S, B, out=None):
-    """out = S B (S: Csr of shape R x C, B dense C x N)."""
+def csr_gemm(S, B, out=None, absmax_out=None):
+    """out = S B (S: Csr of shape R x C, B dense C x N); `absmax_out` (one-element device tensor)
+    also receives max|out|."""
     import torch
     _need(B, torch.float32, "B")
     if B.shape[0] != S.cols:
@@ -202,8 +204,13 @@ def csr_gemm(S, B, out=None):
     if out is None:
         out = torch.empty((S.rows, N), dtype=torch.float32, device=B.device)
     _need(out, torch.float32, "out")
-    check(lib().cn_csr_gemm_f32(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
-                                B.data_ptr(), _ld(B), out.data_ptr(), _ld(out), _stream()))
+    args = (S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(), B.data_ptr(), _ld(B),
+            out.data_ptr(), _ld(out))
+    if absmax_out is None:
+        check(lib().cn_csr_gemm_f32(*args, _stream()))
+    else:
+        _need(absmax_out, torch.float32, "absmax_out")
+        check(lib().cn_csr_gemm_f32_absmax(*args, absmax_out.data_ptr(), _stream()))
     return out
 
 

@@ -200,7 +200,8 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
                                                       const int32_t *__restrict__ col_idx,
                                                       const float *__restrict__ vals, const float *__restrict__ B,
                                                       int64_t ldb, float *__restrict__ out, int64_t ldo,
-                                                      int64_t col_blocks) {
+                                                      int64_t col_blocks, uint32_t *amax_out) {
+    uint32_t amax = 0;  // bit patterns of |x| order like |x|
     const int64_t cb = blockIdx.x % col_blocks, rg = blockIdx.x / col_blocks, row_groups = gridDim.x / col_blocks;
     const int64_t n = cb * 1024 + 4 * (int64_t)threadIdx.x;
     for (int64_t r = rg; r < R; r += row_groups) {
@@ -226,6 +227,11 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
                 acc = acc + v * b;
             }
             __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(out + r * ldo + n));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
+                amax = bits > amax ? bits : amax;
+            }
         } else {
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
             for (int32_t j = j0; j < j1; ++j) {
@@ -235,9 +241,25 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
                     if (n + e < N) acc[e] = acc[e] + v * b[e];
             }
             for (int e = 0; e < 4; ++e)
-                if (n + e < N) out[r * ldo + n + e] = acc[e];
+                if (n + e < N) {
+                    out[r * ldo + n + e] = acc[e];
+                    const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
+                    amax = bits > amax ? bits : amax;
+                }
         }
     }
+    if (amax_out) {  // uniform over the launch; every lane of every wave arrives here
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)amax, off, 64);
+            amax = o > amax ? o : amax;
+        }
+        if ((threadIdx.x & 63) == 0) atomicMax(amax_out, amax);
+    }
+}
+
+__global__ void preset_word_kernel(uint32_t *p, uint32_t value) {
+    if (threadIdx.x == 0) *p = value;
 }
 
 // ---- CSR(S) -> CSR(S^T) ------------------------------------------------------------------------------------
@@ -396,28 +418,46 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
     return CN_OK;
 }
 
-cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
-                          const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, void *stream) {
-    cn_status s = check_csr_args("csr_gemm_f32", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo);
+static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                          const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, float *absmax_out,
+                          void *stream) {
+    cn_status s = check_csr_args(who, R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo);
     if (s != CN_OK) return s;
-    if (R == 0 || N == 0) return CN_OK;
-    if (!out) { set_error("csr_gemm_f32: NULL output"); return CN_ERR_NULL; }
     Context *ctx;
     s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
+    uint32_t *amax = reinterpret_cast<uint32_t *>(absmax_out);
+    if (amax) {  // 0, or -1.0f for an empty result as the abs-max pass reports it
+        hipLaunchKernelGGL(preset_word_kernel, dim3(1), dim3(64), 0, st, amax, (R == 0 || N == 0) ? 0xbf800000u : 0u);
+        CN_HIP(hipGetLastError());
+    }
+    if (R == 0 || N == 0) return CN_OK;
+    if (!out) { set_error("%s: NULL output", who); return CN_ERR_NULL; }
     const int64_t col_blocks = (N + 1023) / 1024;
     int64_t row_groups = ((int64_t)ctx->num_cu * 8 + col_blocks - 1) / col_blocks;
     if (row_groups > R) row_groups = R;
     const bool vec = aligned(B, 16) && aligned(out, 16) && ldb % 4 == 0 && ldo % 4 == 0 && N % 4 == 0;
     if (vec)
         hipLaunchKernelGGL(csr_gemm_kernel<true>, dim3((unsigned)(col_blocks * row_groups)), dim3(kT), 0, st, R, N, row_ptr,
-                           col_idx, vals, B, ldb, out, ldo, col_blocks);
+                           col_idx, vals, B, ldb, out, ldo, col_blocks, amax);
     else
         hipLaunchKernelGGL(csr_gemm_kernel<false>, dim3((unsigned)(col_blocks * row_groups)), dim3(kT), 0, st, R, N, row_ptr,
-                           col_idx, vals, B, ldb, out, ldo, col_blocks);
+                           col_idx, vals, B, ldb, out, ldo, col_blocks, amax);
     CN_HIP(hipGetLastError());
     return CN_OK;
+}
+
+cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                          const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, void *stream) {
+    return csr_gemm("csr_gemm_f32", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo, nullptr, stream);
+}
+
+cn_status cn_csr_gemm_f32_absmax(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                                 const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo,
+                                 float *absmax_out, void *stream) {
+    if (!absmax_out) { set_error("csr_gemm_f32_absmax: NULL absmax_out"); return CN_ERR_NULL; }
+    return csr_gemm("csr_gemm_f32_absmax", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo, absmax_out, stream);
 }
 
 cn_status cn_csr_to_dense_f32(int64_t R, int64_t Cc, const int32_t *row_ptr, const int32_t *col_idx, const float *vals,

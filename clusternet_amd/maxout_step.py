@@ -10,13 +10,30 @@ into libcnhip.
     each gW -> absmax -> compression_8bit -> W -= rate * decode(codes)   (one fused pass, identical
     bit for bit to decompression_8bit followed by the update)
 Biases are inputs and are not updated.
+
+A sparse batch (the reference feeds its 2 % dense inputs as sparse matrices, source/Layer.cpp:250-255
+and 318-321) goes in as `sparse_input(X)`: the first layer's product and its weight gradient then run
+on the compressed rows of X and of X^T.
 """
 from . import _lib as L
 
 
+class SparseInput:
+    """X in compressed sparse rows together with X^T in the same form."""
+
+    def __init__(self, csr, csr_t):
+        self.csr, self.csr_t = csr, csr_t
+
+
+def sparse_input(X):
+    csr = L.csr_from_dense(X)
+    return SparseInput(csr, L.csr_transpose(csr))
+
+
 def forward(X, params, pool=2):
     W1, b1, W2, b2, W3, b3 = params
-    z1 = L.add_row_vector(L.dot(X, W1), b1)
+    xw = L.csr_gemm(X.csr, W1) if isinstance(X, SparseInput) else L.dot(X, W1)
+    z1 = L.add_row_vector(xw, b1)
     h1, a1 = L.maxout(z1, pool)
     z2 = L.add_row_vector(L.dot(h1, W2), b2)
     h2, a2 = L.maxout(z2, pool)
@@ -35,7 +52,10 @@ def backward(X, onehot, params, p, cache, pool=2, absmax_out=None):
     e2 = L.expand_to_maxout_grad(L.dotT(e3, W3), a2, pool)
     gW2 = L.Tdot(h1, e2, absmax_out=m2)
     e1 = L.expand_to_maxout_grad(L.dotT(e2, W2), a1, pool)
-    gW1 = L.Tdot(X, e1, absmax_out=m1)
+    if isinstance(X, SparseInput):
+        gW1 = L.csr_gemm(X.csr_t, e1, absmax_out=m1)
+    else:
+        gW1 = L.Tdot(X, e1, absmax_out=m1)
     return gW1, gW2, gW3
 
 

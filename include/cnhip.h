@@ -174,6 +174,14 @@ cn_status cn_csr_gemm_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_pt
                           const int32_t *col_idx_device, const float *vals_device, const float *B_device,
                           int64_t ldb, float *out_device, int64_t ldo, void *stream);
 
+/* cn_csr_gemm_f32 that also writes max |out[i][j]| to *absmax_out_device (equal bit for bit to
+ * cn_absmax_f32 over the result; -1.0f for an empty one): the sparse weight gradient X^T E followed by
+ * the max(abs(grad)) in front of compression_8bit (source/Layer.cpp:318-321,
+ * source/DeepNeuralNetwork.cpp:334-337) without a second pass over the gradient. */
+cn_status cn_csr_gemm_f32_absmax(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
+                                 const int32_t *col_idx_device, const float *vals_device, const float *B_device,
+                                 int64_t ldb, float *out_device, int64_t ldo, float *absmax_out_device, void *stream);
+
 /* out[R x C] = dense form of S (zeros elsewhere).  sparse_to_dense, source/clusterNet.cpp:1034-1063. */
 cn_status cn_csr_to_dense_f32(int64_t R, int64_t C, const int32_t *row_ptr_device, const int32_t *col_idx_device,
                               const float *vals_device, float *out_device, int64_t ldo, void *stream);

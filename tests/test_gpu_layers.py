@@ -105,6 +105,17 @@ def test_maxout_training_step_reduced_size(dev):
     want_codes = oracle.port_compress(g_host, prec_h)
     assert np.array_equal(codes.cpu().numpy(), want_codes)
     assert np.array_equal(g8.cpu().numpy().view(np.uint32), oracle.port_decompress(want_codes, prec_h).view(np.uint32))
+    # the same batch as a sparse input: the first layer's products run on compressed rows and agree
+    # with the dense ones to the product tolerance (different summation order, same terms)
+    Xs = ms.sparse_input(_t(X, dev))
+    assert Xs.csr.nnz == int((X != 0).sum()) and Xs.csr_t.rows == D
+    p_s, cache_s = ms.forward(Xs, dparams, pool)
+    np.testing.assert_allclose(p_s.cpu().numpy(), p.cpu().numpy(), rtol=2e-4, atol=1e-7)
+    maxima = [torch.empty(1, device=dev) for _ in range(3)]
+    grads_s = ms.backward(Xs, _t(onehot, dev), dparams, p, cache, pool, absmax_out=maxima)
+    err = float((grads_s[0] - grads[0]).abs().max() / grads[0].abs().max())
+    assert err < 1e-5, err
+    assert float(maxima[0].cpu()[0]) == float(grads_s[0].abs().max())
     # the full step runs and moves the weights by rate * decoded gradient
     before = dparams[4].clone()
     ms.step(_t(X, dev), _t(onehot, dev), dparams, 0.01, pool)
