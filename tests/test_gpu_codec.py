@@ -165,3 +165,25 @@ def test_large_tensor_by_tiling(dev):
     back = cn.decompression_8bit(codes, prec)
     bt = _t(oracle.decompress(want, prec), dev)
     assert torch.equal(back.view(reps, -1).view(torch.int32), bt.view(torch.int32).unsqueeze(0).expand(reps, -1))
+
+
+def test_stream_yardstick_moves_the_bytes_it_claims(dev):
+    """The arithmetic-free streams the bench compares the codec with: each does what its label says."""
+    import torch
+    from clusternet_amd import _lib as L
+    n = 4096 * 37
+    x = torch.randn(n, device=dev)
+    bits = x.view(torch.int32)
+    sink = torch.zeros(256 * 2 * L.num_compute_units(), dtype=torch.int32, device=dev)
+    L.stream_yardstick(0, x, sink, n, 2)
+    assert int(sink.view(torch.int32).to(torch.int64).__and__(0xffffffff).max()) == int(bits.to(torch.int64).__and__(0xffffffff).max())
+    top = torch.empty(n, dtype=torch.uint8, device=dev)
+    L.stream_yardstick(1, x, top, n, 4)
+    assert torch.equal(top, ((bits.to(torch.int64) & 0xffffffff) >> 24).to(torch.uint8))
+    back = torch.empty(n, device=dev)
+    L.stream_yardstick(2, top, back, n, 8)
+    assert torch.equal(back, top.float())
+    L.stream_yardstick(3, x, back, n, 16)
+    assert torch.equal(back, x)
+    with pytest.raises(L.CnError):
+        L.stream_yardstick(1, x, top, n - 1, 2)
