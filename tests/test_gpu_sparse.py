@@ -79,6 +79,30 @@ def test_gather_product_is_bit_exact(dev, R, Cc, N, density):
     got = L.csr_gemm(S, _t(B, dev)).cpu().numpy()
     want = oracle.csr_gemm(oracle.csr_from_dense(S_dense), B)
     assert np.array_equal(_bits(got), _bits(want))
+    # the variant that also reports max|out|: same product, and the maximum equals the abs-max pass
+    import torch
+    amax = torch.full((1,), 123.0, device=dev)
+    got2 = L.csr_gemm(S, _t(B, dev), absmax_out=amax).cpu().numpy()
+    assert np.array_equal(_bits(got2), _bits(want))
+    assert float(amax.cpu()[0]) == float(oracle.absmax(want))
+
+
+def test_gather_product_absmax_of_an_empty_result(dev):
+    import torch
+    from clusternet_amd import _lib as L
+    S = L.csr_from_dense(torch.zeros((0, 5), device=dev))
+    amax = torch.full((1,), 123.0, device=dev)
+    L.csr_gemm(S, torch.ones((5, 8), device=dev), absmax_out=amax)
+    assert float(amax.cpu()[0]) == -1.0
+
+
+def test_csr_to_dense_restores_the_matrix(dev):
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(12)
+    for shape, density in (((128, 5000), 0.02), ((7, 11), 0.3), ((5, 1000), 0.0), ((64, 300), 1.0)):
+        A = _sparse(rng, *shape, density)
+        S = L.csr_from_dense(_t(A, dev))
+        assert np.array_equal(_bits(L.csr_to_dense(S).cpu().numpy()), _bits(A))
 
 
 @pytest.mark.parametrize("shape,density", [((1, 1), 1.0), ((7, 11), 0.3), ((128, 5000), 0.02), ((300, 257), 0.1),
