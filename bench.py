@@ -233,8 +233,24 @@ def bench_step(torch, cn, dev):
     def bwd_absmax_sparse():
         state["grads"] = ms.backward(state["Xs"], onehot, params, state["p"], state["cache"], pool, absmax_out=maxima)
 
+    def bwd_deferred_sparse():  # the first layer's gradient is left to first_layer_update below
+        state["grads"] = ms.backward(state["Xs"], onehot, params, state["p"], state["cache"], pool, absmax_out=maxima,
+                                     defer_first=True)
+
+    codes1 = torch.empty((D, H), dtype=torch.uint8, device=dev)
+
+    def first_layer_update():  # max|X^T e1|, then codes + weight update from the recomputed gradient rows
+        ms.coded_sparse_update(W1, state["Xs"], state["grads"][0], 1e-3, prec=maxima[0], codes=codes1)
+
+    def other_layers_update():
+        for w, g, m in zip((W2, W3), state["grads"][1:], maxima[1:]):
+            ms.coded_update(w, g, 1e-3, fused=True, prec=m)
+
     out = {}
     for name, fn in (("sparse_input", to_sparse), ("forward_sparse", fwd_sparse),
+                     ("backward_deferred_sparse", bwd_deferred_sparse),
+                     ("first_layer_codes_and_update_sparse", first_layer_update),
+                     ("other_layers_compress_and_update", other_layers_update),
                      ("backward_with_absmax_sparse", bwd_absmax_sparse),
                      ("forward", fwd), ("backward_with_absmax", bwd_absmax),
                      ("compress_and_update_given_absmax", codec_update_given_max),
@@ -254,6 +270,8 @@ def bench_step(torch, cn, dev):
     out["step_ms"] = out["forward_ms"] + out["backward_with_absmax_ms"] + out["compress_and_update_given_absmax_ms"]
     out["step_sparse_ms"] = (out["sparse_input_ms"] + out["forward_sparse_ms"] + out["backward_with_absmax_sparse_ms"] +
                              out["compress_and_update_given_absmax_ms"])
+    out["step_sparse_fused_ms"] = (out["sparse_input_ms"] + out["forward_sparse_ms"] + out["backward_deferred_sparse_ms"] +
+                                   out["first_layer_codes_and_update_sparse_ms"] + out["other_layers_compress_and_update_ms"])
     out["step_unfused_ms"] = out["forward_ms"] + out["backward_ms"] + out["codec_and_update_unfused_ms"]
     out["note"] = ("bytes per gradient element: absmax 4 + compress 5, then fused decode+update 9 (unfused: decompress 5 + "
                    "update 12) or fused decode+RMSprop 17 (unfused 5 + 20); "

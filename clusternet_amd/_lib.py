@@ -52,6 +52,7 @@ def lib():
     L.cn_csr_transpose.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp]
     L.cn_csr_gemm_f32_absmax.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp, vp]
     L.cn_stream_yardstick.argtypes = [C.c_int, vp, vp, sz, C.c_int, vp]
+    L.cn_csr_gemm_coded_update.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, i64, f32, vp]
     L.cn_csr_to_dense_f32.argtypes = [i64, i64, vp, vp, vp, vp, i64, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
@@ -213,6 +214,42 @@ def csr_gemm(S, B, out=None, absmax_out=None):
         _need(absmax_out, torch.float32, "absmax_out")
         check(lib().cn_csr_gemm_f32_absmax(*args, absmax_out.data_ptr(), _stream()))
     return out
+
+
+def csr_gemm_absmax(S, B, absmax_out=None):
+    """max|S B| as a one-element device tensor; the product itself is not stored."""
+    import torch
+    _need(B, torch.float32, "B")
+    if B.shape[0] != S.cols:
+        raise CnError(2, "Matrix size error: S %dx%d, B %dx%d" % (S.rows, S.cols, B.shape[0], B.shape[1]))
+    if absmax_out is None:
+        absmax_out = torch.empty(1, dtype=torch.float32, device=B.device)
+    check(lib().cn_csr_gemm_f32_absmax(S.rows, S.cols, B.shape[1], S.row_ptr.data_ptr(), S.col_idx.data_ptr(),
+                                       S.vals.data_ptr(), B.data_ptr(), _ld(B), None, 0, absmax_out.data_ptr(), _stream()))
+    return absmax_out
+
+
+def csr_gemm_coded_update(S, B, precision, codes=None, w=None, alpha=1.0):
+    """codes of S B at the device scalar `precision`; with `w`, also w += alpha * decode(codes)."""
+    import torch
+    _need(B, torch.float32, "B")
+    _need(precision, torch.float32, "precision")
+    if B.shape[0] != S.cols:
+        raise CnError(2, "Matrix size error: S %dx%d, B %dx%d" % (S.rows, S.cols, B.shape[0], B.shape[1]))
+    N = B.shape[1]
+    if codes is None:
+        codes = torch.empty((S.rows, N), dtype=torch.uint8, device=B.device)
+    _need(codes, torch.uint8, "codes")
+    if not codes.is_contiguous() or codes.numel() != S.rows * N:
+        raise ValueError("codes must be a contiguous %d x %d uint8 tensor" % (S.rows, N))
+    if w is not None:
+        _need(w, torch.float32, "w")
+        if tuple(w.shape) != (S.rows, N):
+            raise CnError(2, "Matrix size error: w %s, S B %dx%d" % (tuple(w.shape), S.rows, N))
+    check(lib().cn_csr_gemm_coded_update(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                         B.data_ptr(), _ld(B), precision.data_ptr(), codes.data_ptr(),
+                                         None if w is None else w.data_ptr(), 0 if w is None else _ld(w), alpha, _stream()))
+    return codes
 
 
 def csr_to_dense(S, out=None):

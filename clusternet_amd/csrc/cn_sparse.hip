@@ -15,6 +15,7 @@
 // Sums run over the nonzeros in ascending order with a rounded product and a rounded addition per
 // term, so the results are reproducible to the bit.
 #include "cn_internal.h"
+#include "cn_encode_table.h"
 
 namespace cn {
 
@@ -226,7 +227,7 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
                 const f32x4 b = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + n);
                 acc = acc + v * b;
             }
-            __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(out + r * ldo + n));
+            if (out) __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(out + r * ldo + n));
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
             }
             for (int e = 0; e < 4; ++e)
                 if (n + e < N) {
-                    out[r * ldo + n + e] = acc[e];
+                    if (out) out[r * ldo + n + e] = acc[e];
                     const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
                     amax = bits > amax ? bits : amax;
                 }
@@ -258,8 +259,321 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
     }
 }
 
+// ---- rows with few nonzeros, software-pipelined ------------------------------------------------------
+// The weight gradient X^T E has 100000 rows of two or three nonzeros each; one row is a chain of four
+// dependent memory accesses (row pointers, nonzeros, rows of B, then the arithmetic), and a loop that walks
+// it row by row is bound by that latency.  Here a wavefront owns 256 columns (four per lane) of a block
+// of 16 consecutive rows and runs the block as straight-line code:
+//   * the row pointers of the block and its first 64 nonzeros sit in vector registers, one entry per
+//     lane, loaded a whole block ahead and handed to the scalar side with v_readlane;
+//   * the B rows of row u + 2 (four loads, a row with fewer nonzeros repeats one) and the weights of row
+//     u + 8 are requested while row u is summed, encoded and written, into register rings that the
+//     unrolled code indexes statically.
+// Every load is issued unconditionally in a fixed number per row, so each wait counts exactly the loads
+// issued after the one it needs.  Rows with more than four nonzeros, and rows of a block beyond its first
+// 64 nonzeros, take what is missing from memory as the plain kernel does.  The sums run in the same order
+// as there.
+//   kMode 1: max |S B| only            2: codes of S B            3: codes and w += alpha * decode(codes)
+constexpr int kRowThreads = 256;
+constexpr int kRowBlock = 16;  // rows per block
+#ifndef CN_ROW_AHEAD
+#define CN_ROW_AHEAD 1
+#endif
+constexpr int kBAhead = CN_ROW_AHEAD;  // B values are requested this many rows ahead
+constexpr int kBRing = 2 * kBAhead;
+constexpr int kWRing = 8;      // weights eight rows ahead
+#ifndef CN_ROW_FIXED
+#define CN_ROW_FIXED 4
+#endif
+constexpr int kFixed = CN_ROW_FIXED;  // B rows requested ahead per row
+
+struct RowBlockMeta {
+    int rp;    // lane l: row_ptr[first row + l], l <= 16
+    int c;     // lane l: column index of the block's nonzero l
+    float v;   // lane l: its value
+};
+
+template <int kMode>
+__global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
+    int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
+    const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks, uint32_t *amax_out,
+    const float *__restrict__ precision_ptr, uint8_t *__restrict__ codes, float *__restrict__ w, int64_t ldw, float alpha,
+    const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // decode table times alpha
+    const int t = threadIdx.x;
+    float precision = 0.0f;
+    bool exact_only = false;
+    if (kMode >= 2) {
+        precision = *precision_ptr;
+        exact_only = !build_table(sh, steps, step_count, precision, table);
+        if (t < 126) {
+            const float v = table[t] * precision;
+            dlut[t] = alpha * v;
+            dlut[t + 128] = alpha * (-v);
+        } else if (t == 126) {
+            dlut[126] = alpha * precision;
+            dlut[127] = alpha * precision;
+            dlut[254] = alpha * precision;
+            dlut[255] = alpha * (-precision);
+        }
+        __syncthreads();
+    }
+    const uint32_t first = xlut_first(precision);
+    auto encode = [&](float v) -> uint32_t {
+        if (exact_only) return encode_exact(v, precision, sh.slot);
+        const uint32_t bits = __float_as_uint(v);
+        return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
+    };
+
+    const int lane = t & 63;
+    const int32_t nnz = row_ptr[R];
+    const int32_t last = nnz > 0 ? nnz - 1 : 0;
+    const int64_t row_blocks = (R + kRowBlock - 1) / kRowBlock;
+    const int64_t units = row_blocks * col_blocks;
+    const int64_t unit_stride = (int64_t)gridDim.x * (kRowThreads / 64);
+    uint32_t amax = 0;
+
+    auto load_rp = [&](int64_t row0) -> int {
+        int64_t k = row0 + lane;
+        if (k > R) k = R;
+        return row_ptr[k];
+    };
+    auto load_nz = [&](int rp, int &c, float &v) {
+        int j = __builtin_amdgcn_readlane(rp, 0) + lane;
+        if (j > last) j = last;
+        c = nnz > 0 ? col_idx[j] : 0;
+        v = nnz > 0 ? vals[j] : 0.0f;
+    };
+
+    const int64_t unit_first = (int64_t)blockIdx.x * (kRowThreads / 64) + (t >> 6);
+    const uint32_t b_row_bytes = (uint32_t)(ldb * (int64_t)sizeof(float));  // B spans less than 4 GiB on this path
+    const char *Bbytes = reinterpret_cast<const char *>(B);
+    auto lane_column = [&](int64_t unit) -> int64_t {  // first of the lane's four columns; idle lanes use column 0
+        const int64_t n = (unit % col_blocks) * 256 + 4 * (int64_t)lane;
+        return n < N ? n : 0;
+    };
+    // B rows of row u of a unit (metadata m): one v_readlane, one add and the load per request
+    auto request_b = [&](const RowBlockMeta &m, int64_t unit, int u, f32x4 (&dst)[kFixed]) {
+        const int jb0 = __builtin_amdgcn_readlane(m.rp, 0);
+        const uint32_t row_off = (uint32_t)m.c * b_row_bytes;
+        const uint32_t lane_off = (uint32_t)(lane_column(unit) * (int64_t)sizeof(float));
+        const int q0 = __builtin_amdgcn_readlane(m.rp, u) - jb0, q1 = __builtin_amdgcn_readlane(m.rp, u + 1) - jb0;
+        int qlast = q1 - 1;  // a row with fewer nonzeros repeats its last one (an empty row any valid one)
+        if (qlast < q0) qlast = q0;
+        if (qlast > 63) qlast = 63;
+#pragma unroll
+        for (int s2 = 0; s2 < kFixed; ++s2) {
+            const int pick = q0 + s2 < qlast ? q0 + s2 : qlast;
+            const uint32_t off = (uint32_t)__builtin_amdgcn_readlane((int)row_off, pick) + lane_off;
+            dst[s2] = *reinterpret_cast<const f32x4 *>(Bbytes + off);
+        }
+    };
+    auto request_w = [&](int64_t unit, int u, f32x4 &dst) {
+        int64_t r = (unit / col_blocks) * kRowBlock + u;
+        if (r > R - 1) r = R - 1;
+        dst = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(w + r * ldw + lane_column(unit)));
+    };
+
+    f32x4 b[kBRing][kFixed];
+    f32x4 wr[kWRing];
+    RowBlockMeta next;  // of the unit after the current one: loaded while the current one is worked on
+    next.rp = load_rp((unit_first / col_blocks) * kRowBlock);
+    load_nz(next.rp, next.c, next.v);
+    if (unit_first < units) {  // the first unit's early requests; later units get theirs from the unit before
+        if (kMode == 3) {
+#pragma unroll
+            for (int u = 0; u < kWRing; ++u) request_w(unit_first, u, wr[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kBAhead; ++u) request_b(next, unit_first, u, b[u]);
+    }
+    for (int64_t unit = unit_first; unit < units; unit += unit_stride) {
+        const int64_t cb = unit % col_blocks, row0 = (unit / col_blocks) * kRowBlock;
+        const int64_t n = cb * 256 + 4 * (int64_t)lane;
+        const bool live = n < N;
+        const int64_t nc = live ? n : 0;
+        const RowBlockMeta m = next;
+        const int64_t unit_next = unit + unit_stride < units ? unit + unit_stride : unit;
+        next.rp = load_rp((unit_next / col_blocks) * kRowBlock);
+        const int jb0 = __builtin_amdgcn_readlane(m.rp, 0);
+#pragma unroll
+        for (int u = 0; u < kRowBlock; ++u) {
+            if (u + kBAhead < kRowBlock)
+                request_b(m, unit, u + kBAhead, b[(u + kBAhead) % kBRing]);
+            else
+                request_b(next, unit_next, u + kBAhead - kRowBlock, b[(u + kBAhead) % kBRing]);
+            const int64_t r = row0 + u;
+            const int j0 = __builtin_amdgcn_readlane(m.rp, u), j1 = __builtin_amdgcn_readlane(m.rp, u + 1);
+            const int count = j1 - j0, q0 = j0 - jb0;
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            int32_t j = j0;
+            if (q0 + (count < kFixed ? count : kFixed) <= 64) {  // the requested B values are the row's first ones
+#pragma unroll
+                for (int s2 = 0; s2 < kFixed; ++s2)
+                    if (s2 < count) {
+                        const float v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m.v), q0 + s2));
+                        acc = acc + v * b[u % kBRing][s2];
+                    }
+                j = j0 + (count < kFixed ? count : kFixed);
+            }
+            if (j < j1) {
+                for (; j + kGather <= j1; j += kGather) {
+                    int32_t c[kGather];
+                    float v[kGather];
+                    f32x4 bb[kGather];
+#pragma unroll
+                    for (int k = 0; k < kGather; ++k) { c[k] = col_idx[j + k]; v[k] = vals[j + k]; }
+#pragma unroll
+                    for (int k = 0; k < kGather; ++k) bb[k] = *reinterpret_cast<const f32x4 *>(B + (int64_t)c[k] * ldb + nc);
+#pragma unroll
+                    for (int k = 0; k < kGather; ++k) acc = acc + v[k] * bb[k];
+                }
+                for (; j < j1; ++j) {
+                    const float v = vals[j];
+                    const f32x4 bb = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + nc);
+                    acc = acc + v * bb;
+                }
+            }
+            if (r < R) {  // wave-uniform
+                if (kMode == 1) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
+                        amax = bits > amax ? bits : amax;
+                    }
+                } else {
+                    const uint32_t c0 = encode(acc.x), c1 = encode(acc.y), c2 = encode(acc.z), c3 = encode(acc.w);
+                    if (live)
+                        __builtin_nontemporal_store(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24),
+                                                    reinterpret_cast<uint32_t *>(codes + r * N + n));
+                    if (kMode == 3) {
+                        f32x4 wv = wr[u % kWRing];
+                        wv.x = wv.x + dlut[c0];
+                        wv.y = wv.y + dlut[c1];
+                        wv.z = wv.z + dlut[c2];
+                        wv.w = wv.w + dlut[c3];
+                        if (live) __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(w + r * ldw + n));
+                    }
+                }
+            }
+            if (kMode == 3) {
+                if (u + kWRing < kRowBlock)
+                    request_w(unit, u + kWRing, wr[u % kWRing]);
+                else
+                    request_w(unit_next, u + kWRing - kRowBlock, wr[u % kWRing]);
+            }
+            if (u == kRowBlock / 2) load_nz(next.rp, next.c, next.v);  // its row pointers were requested at the top
+        }
+    }
+    if (kMode == 1) {  // every lane of every wave arrives here
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)amax, off, 64);
+            amax = o > amax ? o : amax;
+        }
+        if (lane == 0) atomicMax(amax_out, amax);
+    }
+}
+
 __global__ void preset_word_kernel(uint32_t *p, uint32_t value) {
     if (threadIdx.x == 0) *p = value;
+}
+
+// ---- product -> codes -> update, without the product ever reaching memory -------------------------------
+// codes = compression_8bit(S B, *precision) and, if w is given, w += alpha * decompression_8bit(codes):
+// the weight gradient of the first layer, its 8-bit codes for the exchange and the update of the weights
+// in one pass that writes one byte per element and reads and writes the weights once.  Recomputing a row of
+// S B costs its few nonzeros; the precision (max |S B|) comes from a first pass that stores nothing.
+// Every value is computed, encoded and decoded exactly as by csr_gemm, compress and decompress_axpy.
+// Two rows per iteration and workgroup (512 threads) so that three workgroups with their 40 KB encoder
+// table fill the wavefront slots of a compute unit.
+constexpr int kCodedThreads = 512;
+
+template <bool kVector>
+__global__ __launch_bounds__(kCodedThreads) void csr_gemm_coded_kernel(
+    int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
+    const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks,
+    const float *__restrict__ precision_ptr, uint8_t *__restrict__ codes, float *__restrict__ w, int64_t ldw, float alpha,
+    const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // decode table times alpha
+    const float precision = *precision_ptr;
+    const bool exact_only = !build_table(sh, steps, step_count, precision, table);
+    const int t = threadIdx.x;
+    if (t < 126) {
+        const float v = table[t] * precision;
+        dlut[t] = alpha * v;
+        dlut[t + 128] = alpha * (-v);
+    } else if (t == 126) {
+        dlut[126] = alpha * precision;
+        dlut[127] = alpha * precision;
+        dlut[254] = alpha * precision;
+        dlut[255] = alpha * (-precision);
+    }
+    __syncthreads();
+    const uint32_t first = xlut_first(precision);
+    auto encode = [&](float v) -> uint32_t {
+        if (exact_only) return encode_exact(v, precision, sh.slot);
+        const uint32_t bits = __float_as_uint(v);
+        return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
+    };
+
+    const int64_t cb = blockIdx.x % col_blocks, rg = blockIdx.x / col_blocks, row_groups = gridDim.x / col_blocks;
+    const int slot = t >> 8;
+    const int64_t n = cb * 1024 + 4 * (int64_t)(t & 255);
+    for (int64_t r = rg * 2 + slot; r < R; r += row_groups * 2) {
+        const int32_t j0 = row_ptr[r], j1 = row_ptr[r + 1];
+        if (kVector) {
+            if (n >= N) continue;
+            f32x4 wv = {0.f, 0.f, 0.f, 0.f};
+            if (w) wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(w + r * ldw + n));
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            int32_t j = j0;
+            for (; j + kGather <= j1; j += kGather) {
+                int32_t c[kGather];
+                float v[kGather];
+                f32x4 b[kGather];
+#pragma unroll
+                for (int u = 0; u < kGather; ++u) { c[u] = col_idx[j + u]; v[u] = vals[j + u]; }
+#pragma unroll
+                for (int u = 0; u < kGather; ++u) b[u] = *reinterpret_cast<const f32x4 *>(B + (int64_t)c[u] * ldb + n);
+#pragma unroll
+                for (int u = 0; u < kGather; ++u) acc = acc + v[u] * b[u];
+            }
+            for (; j < j1; ++j) {
+                const float v = vals[j];
+                const f32x4 b = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + n);
+                acc = acc + v * b;
+            }
+            const uint32_t c0 = encode(acc.x), c1 = encode(acc.y), c2 = encode(acc.z), c3 = encode(acc.w);
+            __builtin_nontemporal_store(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24),
+                                        reinterpret_cast<uint32_t *>(codes + r * N + n));
+            if (w) {
+                wv.x = wv.x + dlut[c0];
+                wv.y = wv.y + dlut[c1];
+                wv.z = wv.z + dlut[c2];
+                wv.w = wv.w + dlut[c3];
+                __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(w + r * ldw + n));
+            }
+        } else {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int32_t j = j0; j < j1; ++j) {
+                const float v = vals[j];
+                const float *b = B + (int64_t)col_idx[j] * ldb + n;
+                for (int e = 0; e < 4; ++e)
+                    if (n + e < N) acc[e] = acc[e] + v * b[e];
+            }
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) {
+                    const uint32_t c = encode(acc[e]);
+                    codes[r * N + n + e] = (uint8_t)c;
+                    if (w) w[r * ldw + n + e] = w[r * ldw + n + e] + dlut[c];
+                }
+        }
+    }
 }
 
 // ---- CSR(S) -> CSR(S^T) ------------------------------------------------------------------------------------
@@ -341,7 +655,7 @@ cn_status check_csr_args(const char *who, int64_t R, int64_t Cc, int64_t N, cons
                          const int32_t *col_idx, const float *vals, const float *B, int64_t ldb, const float *out,
                          int64_t ldo) {
     if (R < 0 || Cc < 0 || N < 0) { set_error("%s: negative dimension", who); return CN_ERR_SHAPE; }
-    if (ldb < N || ldo < N) { set_error("%s: leading dimension too small", who); return CN_ERR_SHAPE; }
+    if (ldb < N || (out && ldo < N)) { set_error("%s: leading dimension too small", who); return CN_ERR_SHAPE; }
     if (R > 0x7fffffffLL || Cc > 0x7fffffffLL) { set_error("%s: more than 2^31 rows or columns", who); return CN_ERR_SHAPE; }
     if (!row_ptr) { set_error("%s: NULL row pointers", who); return CN_ERR_NULL; }
     (void)col_idx; (void)vals; (void)B; (void)out;
@@ -433,11 +747,22 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
         CN_HIP(hipGetLastError());
     }
     if (R == 0 || N == 0) return CN_OK;
-    if (!out) { set_error("%s: NULL output", who); return CN_ERR_NULL; }
+    if (!out && !amax) { set_error("%s: NULL output", who); return CN_ERR_NULL; }
+    if (!out && Cc > 0 && Cc * ldb < (1LL << 30) && aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0) {  // maximum only: the pipelined row kernel
+        const int64_t cblocks = (N + 255) / 256;
+        const int64_t units = ((R + kRowBlock - 1) / kRowBlock) * cblocks;
+        int64_t grid = (int64_t)ctx->num_cu * 5;
+        if (grid > (units + 3) / 4) grid = (units + 3) / 4;
+        hipLaunchKernelGGL(csr_rows_kernel<1>, dim3((unsigned)grid), dim3(kRowThreads), 0, st, R, N, row_ptr, col_idx, vals, B, ldb,
+                           cblocks, amax, (const float *)nullptr, (uint8_t *)nullptr, (float *)nullptr, (int64_t)0, 0.0f,
+                           (const XStep *)nullptr, 0, (const float *)nullptr);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
     const int64_t col_blocks = (N + 1023) / 1024;
     int64_t row_groups = ((int64_t)ctx->num_cu * 8 + col_blocks - 1) / col_blocks;
     if (row_groups > R) row_groups = R;
-    const bool vec = aligned(B, 16) && aligned(out, 16) && ldb % 4 == 0 && ldo % 4 == 0 && N % 4 == 0;
+    const bool vec = aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0 && (!out || (aligned(out, 16) && ldo % 4 == 0));
     if (vec)
         hipLaunchKernelGGL(csr_gemm_kernel<true>, dim3((unsigned)(col_blocks * row_groups)), dim3(kT), 0, st, R, N, row_ptr,
                            col_idx, vals, B, ldb, out, ldo, col_blocks, amax);
@@ -458,6 +783,56 @@ cn_status cn_csr_gemm_f32_absmax(int64_t R, int64_t Cc, int64_t N, const int32_t
                                  float *absmax_out, void *stream) {
     if (!absmax_out) { set_error("csr_gemm_f32_absmax: NULL absmax_out"); return CN_ERR_NULL; }
     return csr_gemm("csr_gemm_f32_absmax", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo, absmax_out, stream);
+}
+
+cn_status cn_csr_gemm_coded_update(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                                   const float *vals, const float *B, int64_t ldb, const float *precision_device,
+                                   uint8_t *codes, float *w, int64_t ldw, float alpha, void *stream) {
+    if (R < 0 || Cc < 0 || N < 0) { set_error("csr_gemm_coded_update: negative dimension"); return CN_ERR_SHAPE; }
+    if (ldb < N || (w && ldw < N)) { set_error("csr_gemm_coded_update: leading dimension too small"); return CN_ERR_SHAPE; }
+    if (R > 0x7fffffffLL || Cc > 0x7fffffffLL) { set_error("csr_gemm_coded_update: more than 2^31 rows or columns"); return CN_ERR_SHAPE; }
+    if (R == 0 || N == 0) return CN_OK;
+    if (!row_ptr || !precision_device || !codes) { set_error("csr_gemm_coded_update: NULL pointer"); return CN_ERR_NULL; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    const int lds = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
+    static bool configured = false;
+    if (!configured) {
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_gemm_coded_kernel<false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<2>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<3>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        configured = true;
+    }
+    const bool vec = Cc > 0 && Cc * ldb < (1LL << 30) && aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0 && aligned(codes, 4) &&
+                     (!w || (aligned(w, 16) && ldw % 4 == 0));
+    if (vec) {
+        const int64_t col_blocks = (N + 255) / 256;
+        const int64_t units = ((R + kRowBlock - 1) / kRowBlock) * col_blocks;
+        int64_t grid = (int64_t)ctx->num_cu * 3;  // the encoder table allows three workgroups per compute unit
+        if (grid > (units + 3) / 4) grid = (units + 3) / 4;
+        if (w)
+            hipLaunchKernelGGL(csr_rows_kernel<3>, dim3((unsigned)grid), dim3(kRowThreads), lds, st, R, N, row_ptr, col_idx, vals, B,
+                               ldb, col_blocks, (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, ctx->xsteps,
+                               ctx->xstep_count, ctx->table);
+        else
+            hipLaunchKernelGGL(csr_rows_kernel<2>, dim3((unsigned)grid), dim3(kRowThreads), lds, st, R, N, row_ptr, col_idx, vals, B,
+                               ldb, col_blocks, (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, ctx->xsteps,
+                               ctx->xstep_count, ctx->table);
+    } else {
+        const int64_t col_blocks = (N + 1023) / 1024;
+        int64_t row_groups = ((int64_t)ctx->num_cu * 3 + col_blocks - 1) / col_blocks;
+        if (row_groups > (R + 1) / 2) row_groups = (R + 1) / 2;
+        hipLaunchKernelGGL(csr_gemm_coded_kernel<false>, dim3((unsigned)(col_blocks * row_groups)), dim3(kCodedThreads), lds, st,
+                           R, N, row_ptr, col_idx, vals, B, ldb, col_blocks, precision_device, codes, w, ldw, alpha, ctx->xsteps,
+                           ctx->xstep_count, ctx->table);
+    }
+    CN_HIP(hipGetLastError());
+    return CN_OK;
 }
 
 cn_status cn_csr_to_dense_f32(int64_t R, int64_t Cc, const int32_t *row_ptr, const int32_t *col_idx, const float *vals,

@@ -41,9 +41,11 @@ def forward(X, params, pool=2):
     return p, (h1, a1, h2, a2)
 
 
-def backward(X, onehot, params, p, cache, pool=2, absmax_out=None):
+def backward(X, onehot, params, p, cache, pool=2, absmax_out=None, defer_first=False):
     """Weight gradients.  `absmax_out` = three one-element device tensors: the gradient products then
-    also deliver max|gW|, which saves the abs-max pass in front of compression_8bit."""
+    also deliver max|gW|, which saves the abs-max pass in front of compression_8bit.
+    `defer_first` (sparse input only): the first element of the result is the error signal e1 instead
+    of gW1 = X^T e1, for `coded_sparse_update`, which never stores that gradient."""
     W1, b1, W2, b2, W3, b3 = params
     h1, a1, h2, a2 = cache
     m1, m2, m3 = absmax_out if absmax_out is not None else (None, None, None)
@@ -52,7 +54,9 @@ def backward(X, onehot, params, p, cache, pool=2, absmax_out=None):
     e2 = L.expand_to_maxout_grad(L.dotT(e3, W3), a2, pool)
     gW2 = L.Tdot(h1, e2, absmax_out=m2)
     e1 = L.expand_to_maxout_grad(L.dotT(e2, W2), a1, pool)
-    if isinstance(X, SparseInput):
+    if isinstance(X, SparseInput) and defer_first:
+        gW1 = e1
+    elif isinstance(X, SparseInput):
         gW1 = L.csr_gemm(X.csr_t, e1, absmax_out=m1)
     else:
         gW1 = L.Tdot(X, e1, absmax_out=m1)
@@ -80,6 +84,16 @@ def coded_update(w, grad, rate, fused=True, scratch=None, prec=None):
     return codes, prec
 
 
+def coded_sparse_update(w, Xs, e1, rate, prec=None, codes=None):
+    """W -= rate * decode(encode(X^T e1)) for a sparse batch without the gradient ever reaching memory:
+    one pass for max|X^T e1|, one that recomputes each gradient row from its two or three nonzeros,
+    encodes it (the codes are what the exchange between GPUs sends) and updates the weights.  Bit for bit
+    the result of csr_gemm, absmax, compression_8bit and decompression_8bit_axpy."""
+    prec = L.csr_gemm_absmax(Xs.csr_t, e1, prec)
+    codes = L.csr_gemm_coded_update(Xs.csr_t, e1, prec, codes, w=w, alpha=-rate)
+    return codes, prec
+
+
 def coded_rmsprop_update(w, rms, grad, rms_multiplier, rate, fused=True, scratch=None):
     """RMSprop with weight update (source/basicOps.cu:1192-1197) on the 8-bit round trip of `grad`."""
     prec = L.absmax(grad)
@@ -95,9 +109,13 @@ def coded_rmsprop_update(w, rms, grad, rms_multiplier, rate, fused=True, scratch
 def step(X, onehot, params, rate, pool=2):
     import torch
     p, cache = forward(X, params, pool)
-    maxima = [torch.empty(1, dtype=torch.float32, device=X.device) for _ in range(3)]
-    grads = backward(X, onehot, params, p, cache, pool, absmax_out=maxima)
+    maxima = [torch.empty(1, dtype=torch.float32, device=p.device) for _ in range(3)]
+    sparse = isinstance(X, SparseInput)
+    grads = backward(X, onehot, params, p, cache, pool, absmax_out=maxima, defer_first=sparse)
     W = (params[0], params[2], params[4])
-    for w, g, m in zip(W, grads, maxima):
-        coded_update(w, g, rate, prec=m)
+    for i, (w, g, m) in enumerate(zip(W, grads, maxima)):
+        if sparse and i == 0:
+            coded_sparse_update(w, X, g, rate, prec=m)
+        else:
+            coded_update(w, g, rate, prec=m)
     return p

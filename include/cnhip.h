@@ -185,10 +185,23 @@ cn_status cn_csr_gemm_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_pt
 /* cn_csr_gemm_f32 that also writes max |out[i][j]| to *absmax_out_device (equal bit for bit to
  * cn_absmax_f32 over the result; -1.0f for an empty one): the sparse weight gradient X^T E followed by
  * the max(abs(grad)) in front of compression_8bit (source/Layer.cpp:318-321,
- * source/DeepNeuralNetwork.cpp:334-337) without a second pass over the gradient. */
+ * source/DeepNeuralNetwork.cpp:334-337) without a second pass over the gradient.  out_device may be
+ * NULL: then only the maximum is produced and the product is not stored. */
 cn_status cn_csr_gemm_f32_absmax(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
                                  const int32_t *col_idx_device, const float *vals_device, const float *B_device,
                                  int64_t ldb, float *out_device, int64_t ldo, float *absmax_out_device, void *stream);
+
+/* With G = S B (never stored): codes[R x N, contiguous] = the codes cn_compress_8bit_dp gives for G and
+ * *precision_device, and, when w_device is not NULL, w += alpha * (what cn_decompress_8bit gives for those
+ * codes) -- bit for bit the sequence cn_csr_gemm_f32, cn_compress_8bit_dp, cn_decompress_8bit_axpy_dp.
+ * It is the first-layer weight gradient of a sparse batch, its 8-bit codes for the exchange and the
+ * weight update (source/Layer.cpp:318-321, 365, 430-433; source/DeepNeuralNetwork.cpp:334-339) in one
+ * pass that reads and writes the weights once and writes one byte per gradient element; take
+ * *precision_device from cn_csr_gemm_f32_absmax with a NULL output. */
+cn_status cn_csr_gemm_coded_update(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
+                                   const int32_t *col_idx_device, const float *vals_device, const float *B_device,
+                                   int64_t ldb, const float *precision_device, uint8_t *codes_device,
+                                   float *w_device, int64_t ldw, float alpha, void *stream);
 
 /* out[R x C] = dense form of S (zeros elsewhere).  sparse_to_dense, source/clusterNet.cpp:1034-1063. */
 cn_status cn_csr_to_dense_f32(int64_t R, int64_t C, const int32_t *row_ptr_device, const int32_t *col_idx_device,

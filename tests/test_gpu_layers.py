@@ -116,10 +116,29 @@ def test_maxout_training_step_reduced_size(dev):
     err = float((grads_s[0] - grads[0]).abs().max() / grads[0].abs().max())
     assert err < 1e-5, err
     assert float(maxima[0].cpu()[0]) == float(grads_s[0].abs().max())
+    # the first layer's update straight from the error signal equals the one through the stored gradient
+    e1_first = ms.backward(Xs, _t(onehot, dev), dparams, p, cache, pool, defer_first=True)[0]
+    w_a, w_b = dparams[0].clone(), dparams[0].clone()
+    codes_a, prec_a = ms.coded_sparse_update(w_a, Xs, e1_first, 0.01)
+    codes_b, prec_b = ms.coded_update(w_b, grads_s[0].clone(), 0.01)
+    assert float(prec_a.cpu()[0]) == float(prec_b.cpu()[0])
+    assert torch.equal(codes_a.view(-1), codes_b.view(-1))
+    assert torch.equal(w_a.view(torch.int32), w_b.view(torch.int32))
     # the full step runs and moves the weights by rate * decoded gradient
     before = dparams[4].clone()
     ms.step(_t(X, dev), _t(onehot, dev), dparams, 0.01, pool)
     assert float((dparams[4] - before).abs().max()) > 0
+    # the sparse step is forward, backward and the three coded updates, nothing else
+    pa = tuple(t.clone() for t in dparams)
+    pb = tuple(t.clone() for t in dparams)
+    ms.step(Xs, _t(onehot, dev), pb, 0.01, pool)
+    p2, cache2 = ms.forward(Xs, pa, pool)
+    e1_2, g2, g3 = ms.backward(Xs, _t(onehot, dev), pa, p2, cache2, pool, defer_first=True)
+    ms.coded_sparse_update(pa[0], Xs, e1_2, 0.01)
+    ms.coded_update(pa[2], g2, 0.01)
+    ms.coded_update(pa[4], g3, 0.01)
+    for a, b2 in zip(pa, pb):
+        assert torch.equal(a.view(torch.int32), b2.view(torch.int32))
 
 
 def test_maxout_training_step_full_size_properties(dev):

@@ -96,6 +96,61 @@ def test_gather_product_absmax_of_an_empty_result(dev):
     assert float(amax.cpu()[0]) == -1.0
 
 
+@pytest.mark.parametrize("R,Cc,N,density", [(2000, 128, 1024, 0.02), (777, 64, 4100, 0.05), (37, 211, 19, 0.05),
+                                            (5, 9, 1, 0.5), (301, 16, 2052, 0.0), (4096, 128, 8192, 0.02)])
+@pytest.mark.parametrize("with_update", [False, True])
+def test_product_to_codes_and_update_equals_the_three_separate_calls(dev, R, Cc, N, density, with_update):
+    """max|S B| without storing, then codes (and the weight update) straight from the recomputed product:
+    bit for bit what csr_gemm, absmax, compression_8bit and decompression_8bit_axpy give, and what the
+    CPU checker gives for the same sequence."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(R * 7 + N)
+    S_dense = _sparse(rng, R, Cc, density)
+    B = rng.normal(0, 0.01, (Cc, N)).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    Bd = _t(B, dev)
+    G = L.csr_gemm(S, Bd)
+    prec = L.csr_gemm_absmax(S, Bd)
+    want_prec = L.absmax(G)
+    assert float(prec.cpu()[0]) == float(want_prec.cpu()[0])
+    want_codes = L.compression_8bit(G, want_prec)
+    w0 = rng.normal(0, 0.05, (R, N)).astype(np.float32)
+    w = _t(w0, dev) if with_update else None
+    codes = L.csr_gemm_coded_update(S, Bd, prec, w=w, alpha=-0.01)
+    assert torch.equal(codes, want_codes.view(R, N))
+    # against the CPU checker on the checker's own product
+    G_host = oracle.csr_gemm(oracle.csr_from_dense(S_dense), B)
+    p_host = oracle.absmax(G_host)
+    assert float(prec.cpu()[0]) == p_host
+    if p_host > 0:
+        assert np.array_equal(codes.cpu().numpy(), oracle.port_compress(G_host, p_host).reshape(R, N))
+    if with_update:
+        want_w = _t(w0, dev)
+        L.decompression_8bit_axpy(want_codes, want_prec, -0.01, want_w)
+        assert torch.equal(w.view(torch.int32), want_w.view(torch.int32))
+        if p_host > 0:
+            host_w = oracle.decompress_axpy(codes.cpu().numpy().reshape(-1), p_host, -0.01, w0.reshape(-1))
+            assert np.array_equal(_bits(w.cpu().numpy().reshape(-1)), _bits(host_w))
+
+
+def test_product_to_codes_takes_strided_operands(dev):
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(31)
+    S_dense = _sparse(rng, 300, 40, 0.1)
+    Bfull = rng.normal(0, 1, (40, 300)).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    Bd = _t(Bfull, dev)[:, 8:208]
+    wfull = torch.zeros((300, 256), device=dev)
+    prec = L.csr_gemm_absmax(S, Bd)
+    codes = L.csr_gemm_coded_update(S, Bd, prec, w=wfull[:, 16:216], alpha=1.0)
+    G = L.csr_gemm(S, Bd.contiguous())
+    assert torch.equal(codes, L.compression_8bit(G, prec).view(300, 200))
+    assert torch.equal(wfull[:, 16:216], L.decompression_8bit(codes.view(-1), prec).view(300, 200))
+    assert float(wfull[:, :16].abs().max()) == 0 and float(wfull[:, 216:].abs().max()) == 0
+
+
 def test_csr_to_dense_restores_the_matrix(dev):
     from clusternet_amd import _lib as L
     rng = np.random.default_rng(12)
