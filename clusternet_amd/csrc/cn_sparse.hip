@@ -266,9 +266,9 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
 // of 16 consecutive rows and runs the block as straight-line code:
 //   * the row pointers of the block and its first 64 nonzeros sit in vector registers, one entry per
 //     lane, loaded a whole block ahead and handed to the scalar side with v_readlane;
-//   * the B rows of row u + 2 (four loads, a row with fewer nonzeros repeats one) and the weights of row
-//     u + 8 are requested while row u is summed, encoded and written, into register rings that the
-//     unrolled code indexes statically.
+//   * the B rows of row u + 1 (four loads; what a shorter row does not need reads one fixed cache line)
+//     and the weights of row u + 8 are requested while row u is summed, encoded and written, into register
+//     rings that the unrolled code indexes statically; the requests run on into the next block.
 // Every load is issued unconditionally in a fixed number per row, so each wait counts exactly the loads
 // issued after the one it needs.  Rows with more than four nonzeros, and rows of a block beyond its first
 // 64 nonzeros, take what is missing from memory as the plain kernel does.  The sums run in the same order
@@ -276,16 +276,10 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
 //   kMode 1: max |S B| only            2: codes of S B            3: codes and w += alpha * decode(codes)
 constexpr int kRowThreads = 256;
 constexpr int kRowBlock = 16;  // rows per block
-#ifndef CN_ROW_AHEAD
-#define CN_ROW_AHEAD 1
-#endif
-constexpr int kBAhead = CN_ROW_AHEAD;  // B values are requested this many rows ahead
+constexpr int kBAhead = 1;     // B values are requested this many rows ahead
 constexpr int kBRing = 2 * kBAhead;
-constexpr int kWRing = 8;      // weights eight rows ahead
-#ifndef CN_ROW_FIXED
-#define CN_ROW_FIXED 4
-#endif
-constexpr int kFixed = CN_ROW_FIXED;  // B rows requested ahead per row
+constexpr int kWRing = 8;      // weights this many rows ahead
+constexpr int kFixed = 4;      // B rows requested ahead per row
 
 struct RowBlockMeta {
     int rp;    // lane l: row_ptr[first row + l], l <= 16
@@ -350,63 +344,89 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
     const int64_t unit_first = (int64_t)blockIdx.x * (kRowThreads / 64) + (t >> 6);
     const uint32_t b_row_bytes = (uint32_t)(ldb * (int64_t)sizeof(float));  // B spans less than 4 GiB on this path
     const char *Bbytes = reinterpret_cast<const char *>(B);
-    auto lane_column = [&](int64_t unit) -> int64_t {  // first of the lane's four columns; idle lanes use column 0
-        const int64_t n = (unit % col_blocks) * 256 + 4 * (int64_t)lane;
-        return n < N ? n : 0;
+    // Where a unit lives: computed once per unit, the rows then only add multiples of the leading dimensions.
+    struct UnitPos {
+        int64_t row0;
+        int rows;           // rows of the block inside the matrix (1 .. 16)
+        bool live;          // the lane's four columns exist
+        uint32_t lane_off;  // byte offset of the lane's columns inside a row of B (column 0 for idle lanes)
+        float *wp;          // weights of row0 at the lane's columns
+        uint8_t *cp;        // codes of row0 at the lane's columns
     };
-    // B rows of row u of a unit (metadata m): one v_readlane, one add and the load per request
-    auto request_b = [&](const RowBlockMeta &m, int64_t unit, int u, f32x4 (&dst)[kFixed]) {
-        const int jb0 = __builtin_amdgcn_readlane(m.rp, 0);
-        const uint32_t row_off = (uint32_t)m.c * b_row_bytes;
-        const uint32_t lane_off = (uint32_t)(lane_column(unit) * (int64_t)sizeof(float));
-        const int q0 = __builtin_amdgcn_readlane(m.rp, u) - jb0, q1 = __builtin_amdgcn_readlane(m.rp, u + 1) - jb0;
-        int qlast = q1 - 1;  // a row with fewer nonzeros repeats its last one (an empty row any valid one)
-        if (qlast < q0) qlast = q0;
-        if (qlast > 63) qlast = 63;
+    auto locate = [&](int64_t unit) -> UnitPos {
+        UnitPos p;
+        const uint32_t rb = (uint32_t)unit / (uint32_t)col_blocks, cb = (uint32_t)unit - rb * (uint32_t)col_blocks;
+        p.row0 = (int64_t)rb * kRowBlock;
+        const int64_t left = R - p.row0;
+        p.rows = left < kRowBlock ? (int)left : kRowBlock;
+        const int64_t n = (int64_t)cb * 256 + 4 * (int64_t)lane;
+        p.live = n < N;
+        const int64_t nc = p.live ? n : 0;
+        p.lane_off = (uint32_t)(nc * (int64_t)sizeof(float));
+        p.wp = kMode == 3 ? w + p.row0 * ldw + nc : nullptr;
+        p.cp = kMode >= 2 ? codes + p.row0 * N + nc : nullptr;
+        return p;
+    };
+    struct Ready {  // block metadata with what every request needs precomputed
+        int rp, jb0;
+        float v;
+        uint32_t row_off;  // lane l: byte offset of the B row of the block's nonzero l
+    };
+    auto prepare = [&](const RowBlockMeta &m) -> Ready {
+        Ready r;
+        r.rp = m.rp;
+        r.jb0 = __builtin_amdgcn_readlane(m.rp, 0);
+        r.v = m.v;
+        r.row_off = (uint32_t)m.c * b_row_bytes;
+        return r;
+    };
+    // B rows of row u of a block: one v_readlane, one add and the load per request
+    auto request_b = [&](const Ready &m, uint32_t lane_off, int u, f32x4 (&dst)[kFixed]) {
+        const int q0 = __builtin_amdgcn_readlane(m.rp, u) - m.jb0, q1 = __builtin_amdgcn_readlane(m.rp, u + 1) - m.jb0;
+        const int qend = q1 < 64 ? q1 : 64;
 #pragma unroll
         for (int s2 = 0; s2 < kFixed; ++s2) {
-            const int pick = q0 + s2 < qlast ? q0 + s2 : qlast;
-            const uint32_t off = (uint32_t)__builtin_amdgcn_readlane((int)row_off, pick) + lane_off;
+            // a request beyond the row's nonzeros (or the cached 64) is still issued, so that the number of
+            // loads per row is fixed, but all lanes then read the first 16 bytes of B: one cache line
+            const bool real = q0 + s2 < qend;
+            const uint32_t off = real ? (uint32_t)__builtin_amdgcn_readlane((int)m.row_off, (q0 + s2) & 63) + lane_off : 0u;
             dst[s2] = *reinterpret_cast<const f32x4 *>(Bbytes + off);
         }
     };
-    auto request_w = [&](int64_t unit, int u, f32x4 &dst) {
-        int64_t r = (unit / col_blocks) * kRowBlock + u;
-        if (r > R - 1) r = R - 1;
-        dst = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(w + r * ldw + lane_column(unit)));
+    auto request_w = [&](const UnitPos &p, int u, f32x4 &dst) {
+        const int uu = u < p.rows ? u : p.rows - 1;
+        dst = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.wp + (int64_t)uu * ldw));
     };
 
     f32x4 b[kBRing][kFixed];
     f32x4 wr[kWRing];
     RowBlockMeta next;  // of the unit after the current one: loaded while the current one is worked on
-    next.rp = load_rp((unit_first / col_blocks) * kRowBlock);
+    UnitPos pos_next = locate(unit_first < units ? unit_first : 0);
+    next.rp = load_rp(pos_next.row0);
     load_nz(next.rp, next.c, next.v);
     if (unit_first < units) {  // the first unit's early requests; later units get theirs from the unit before
         if (kMode == 3) {
 #pragma unroll
-            for (int u = 0; u < kWRing; ++u) request_w(unit_first, u, wr[u]);
+            for (int u = 0; u < kWRing; ++u) request_w(pos_next, u, wr[u]);
         }
+        const Ready first_ready = prepare(next);
 #pragma unroll
-        for (int u = 0; u < kBAhead; ++u) request_b(next, unit_first, u, b[u]);
+        for (int u = 0; u < kBAhead; ++u) request_b(first_ready, pos_next.lane_off, u, b[u]);
     }
     for (int64_t unit = unit_first; unit < units; unit += unit_stride) {
-        const int64_t cb = unit % col_blocks, row0 = (unit / col_blocks) * kRowBlock;
-        const int64_t n = cb * 256 + 4 * (int64_t)lane;
-        const bool live = n < N;
-        const int64_t nc = live ? n : 0;
-        const RowBlockMeta m = next;
-        const int64_t unit_next = unit + unit_stride < units ? unit + unit_stride : unit;
-        next.rp = load_rp((unit_next / col_blocks) * kRowBlock);
-        const int jb0 = __builtin_amdgcn_readlane(m.rp, 0);
+        const UnitPos pos = pos_next;
+        const Ready m = prepare(next);
+        pos_next = locate(unit + unit_stride < units ? unit + unit_stride : unit);
+        next.rp = load_rp(pos_next.row0);
+        Ready m_next = m;  // replaced once the next block's nonzeros are requested (row 8)
 #pragma unroll
         for (int u = 0; u < kRowBlock; ++u) {
             if (u + kBAhead < kRowBlock)
-                request_b(m, unit, u + kBAhead, b[(u + kBAhead) % kBRing]);
+                request_b(m, pos.lane_off, u + kBAhead, b[(u + kBAhead) % kBRing]);
             else
-                request_b(next, unit_next, u + kBAhead - kRowBlock, b[(u + kBAhead) % kBRing]);
-            const int64_t r = row0 + u;
+                request_b(m_next, pos_next.lane_off, u + kBAhead - kRowBlock, b[(u + kBAhead) % kBRing]);
             const int j0 = __builtin_amdgcn_readlane(m.rp, u), j1 = __builtin_amdgcn_readlane(m.rp, u + 1);
-            const int count = j1 - j0, q0 = j0 - jb0;
+            const int count = j1 - j0, q0 = j0 - m.jb0;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
             int32_t j = j0;
             if (q0 + (count < kFixed ? count : kFixed) <= 64) {  // the requested B values are the row's first ones
@@ -419,6 +439,7 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
                 j = j0 + (count < kFixed ? count : kFixed);
             }
             if (j < j1) {
+                const float *Bl = reinterpret_cast<const float *>(Bbytes + pos.lane_off);
                 for (; j + kGather <= j1; j += kGather) {
                     int32_t c[kGather];
                     float v[kGather];
@@ -426,17 +447,17 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
 #pragma unroll
                     for (int k = 0; k < kGather; ++k) { c[k] = col_idx[j + k]; v[k] = vals[j + k]; }
 #pragma unroll
-                    for (int k = 0; k < kGather; ++k) bb[k] = *reinterpret_cast<const f32x4 *>(B + (int64_t)c[k] * ldb + nc);
+                    for (int k = 0; k < kGather; ++k) bb[k] = *reinterpret_cast<const f32x4 *>(Bl + (int64_t)c[k] * ldb);
 #pragma unroll
                     for (int k = 0; k < kGather; ++k) acc = acc + v[k] * bb[k];
                 }
                 for (; j < j1; ++j) {
                     const float v = vals[j];
-                    const f32x4 bb = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + nc);
+                    const f32x4 bb = *reinterpret_cast<const f32x4 *>(Bl + (int64_t)col_idx[j] * ldb);
                     acc = acc + v * bb;
                 }
             }
-            if (r < R) {  // wave-uniform
+            if (u < pos.rows) {  // wave-uniform
                 if (kMode == 1) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -445,26 +466,29 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
                     }
                 } else {
                     const uint32_t c0 = encode(acc.x), c1 = encode(acc.y), c2 = encode(acc.z), c3 = encode(acc.w);
-                    if (live)
+                    if (pos.live)
                         __builtin_nontemporal_store(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24),
-                                                    reinterpret_cast<uint32_t *>(codes + r * N + n));
+                                                    reinterpret_cast<uint32_t *>(pos.cp + (int64_t)u * N));
                     if (kMode == 3) {
                         f32x4 wv = wr[u % kWRing];
                         wv.x = wv.x + dlut[c0];
                         wv.y = wv.y + dlut[c1];
                         wv.z = wv.z + dlut[c2];
                         wv.w = wv.w + dlut[c3];
-                        if (live) __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(w + r * ldw + n));
+                        if (pos.live) __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(pos.wp + (int64_t)u * ldw));
                     }
                 }
             }
             if (kMode == 3) {
                 if (u + kWRing < kRowBlock)
-                    request_w(unit, u + kWRing, wr[u % kWRing]);
+                    request_w(pos, u + kWRing, wr[u % kWRing]);
                 else
-                    request_w(unit_next, u + kWRing - kRowBlock, wr[u % kWRing]);
+                    request_w(pos_next, u + kWRing - kRowBlock, wr[u % kWRing]);
             }
-            if (u == kRowBlock / 2) load_nz(next.rp, next.c, next.v);  // its row pointers were requested at the top
+            if (u == kRowBlock / 2) {  // the next block's row pointers were requested at the top
+                load_nz(next.rp, next.c, next.v);
+            }
+            if (u == kRowBlock - kBAhead - 1) m_next = prepare(next);
         }
     }
     if (kMode == 1) {  // every lane of every wave arrives here
@@ -751,8 +775,9 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
     if (!out && Cc > 0 && Cc * ldb < (1LL << 30) && aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0) {  // maximum only: the pipelined row kernel
         const int64_t cblocks = (N + 255) / 256;
         const int64_t units = ((R + kRowBlock - 1) / kRowBlock) * cblocks;
+        const int64_t per_wg = kRowThreads / 64;
         int64_t grid = (int64_t)ctx->num_cu * 5;
-        if (grid > (units + 3) / 4) grid = (units + 3) / 4;
+        if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
         hipLaunchKernelGGL(csr_rows_kernel<1>, dim3((unsigned)grid), dim3(kRowThreads), 0, st, R, N, row_ptr, col_idx, vals, B, ldb,
                            cblocks, amax, (const float *)nullptr, (uint8_t *)nullptr, (float *)nullptr, (int64_t)0, 0.0f,
                            (const XStep *)nullptr, 0, (const float *)nullptr);
@@ -813,8 +838,9 @@ cn_status cn_csr_gemm_coded_update(int64_t R, int64_t Cc, int64_t N, const int32
     if (vec) {
         const int64_t col_blocks = (N + 255) / 256;
         const int64_t units = ((R + kRowBlock - 1) / kRowBlock) * col_blocks;
+        const int64_t per_wg = kRowThreads / 64;
         int64_t grid = (int64_t)ctx->num_cu * 3;  // the encoder table allows three workgroups per compute unit
-        if (grid > (units + 3) / 4) grid = (units + 3) / 4;
+        if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
         if (w)
             hipLaunchKernelGGL(csr_rows_kernel<3>, dim3((unsigned)grid), dim3(kRowThreads), lds, st, R, N, row_ptr, col_idx, vals, B,
                                ldb, col_blocks, (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, ctx->xsteps,
