@@ -87,6 +87,30 @@ def test_gather_product_is_bit_exact(dev, R, Cc, N, density):
     assert float(amax.cpu()[0]) == float(oracle.absmax(want))
 
 
+@pytest.mark.parametrize("R,Cc,N,density", [(128, 3000, 4096, 0.02), (100, 700, 2052, 0.1), (3, 50, 2048, 0.5),
+                                            (128, 64, 8192, 1.0)])
+def test_few_long_rows_take_the_strip_kernel_with_the_same_bits(dev, R, Cc, N, density):
+    """Few rows and many columns run one column strip per L2 at a time; same sums, same bits, also with
+    the maximum."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(R + N)
+    S_dense = _sparse(rng, R, Cc, density)
+    B = rng.normal(0, 1, (Cc, N)).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    amax = torch.zeros(1, device=dev)
+    got = L.csr_gemm(S, _t(B, dev), absmax_out=amax)
+    L.lib().cn_host_csr_strip_kernel(0)
+    try:
+        plain = L.csr_gemm(S, _t(B, dev))
+    finally:
+        L.lib().cn_host_csr_strip_kernel(1)
+    assert torch.equal(got.view(torch.int32), plain.view(torch.int32))
+    want = oracle.csr_gemm(oracle.csr_from_dense(S_dense), B)
+    assert np.array_equal(_bits(got.cpu().numpy()), _bits(want))
+    assert float(amax.cpu()[0]) == float(oracle.absmax(want))
+
+
 def test_gather_product_absmax_of_an_empty_result(dev):
     import torch
     from clusternet_amd import _lib as L
