@@ -236,11 +236,15 @@ def bench_step(torch, cn, dev):
     def bwd_deferred_sparse():  # the first layer's gradient is left to first_layer_update below
         state["grads"] = ms.backward(state["Xs"], onehot, params, state["p"], state["cache"], pool, absmax_out=maxima,
                                      defer_first=True)
+        state["e1"] = state["grads"][0]
 
     codes1 = torch.empty((D, H), dtype=torch.uint8, device=dev)
 
     def first_layer_update():  # max|X^T e1|, then codes + weight update from the recomputed gradient rows
         ms.coded_sparse_update(W1, state["Xs"], state["grads"][0], 1e-3, prec=maxima[0], codes=codes1)
+
+    def first_layer_rmsprop():
+        ms.coded_sparse_rmsprop_update(W1, rms[0], state["Xs"], state["e1"], 0.9, 1e-3, prec=maxima[0], codes=codes1)
 
     def other_layers_update():
         for w, g, m in zip((W2, W3), state["grads"][1:], maxima[1:]):
@@ -256,7 +260,8 @@ def bench_step(torch, cn, dev):
                      ("compress_and_update_given_absmax", codec_update_given_max),
                      ("backward", bwd), ("codec_and_update", codec_update),
                      ("codec_and_update_unfused", codec_update_unfused), ("codec_and_rmsprop", codec_rmsprop),
-                     ("codec_and_rmsprop_unfused", codec_rmsprop_unfused)):
+                     ("codec_and_rmsprop_unfused", codec_rmsprop_unfused),
+                     ("first_layer_codes_and_rmsprop_sparse", first_layer_rmsprop)):
         out[name + "_ms"] = time_region(torch, fn, 5, 2)
     flop_f = 2.0 * B * (D * H + (H // pool) * H + (H // pool) * C)
     flop_b = flop_f + 2.0 * B * ((H // pool) * H + (H // pool) * C)

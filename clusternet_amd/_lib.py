@@ -53,6 +53,7 @@ def lib():
     L.cn_csr_gemm_f32_absmax.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp, vp]
     L.cn_stream_yardstick.argtypes = [C.c_int, vp, vp, sz, C.c_int, vp]
     L.cn_csr_gemm_coded_update.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, i64, f32, vp]
+    L.cn_csr_gemm_coded_rmsprop.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, vp, i64, f32, f32, vp]
     L.cn_csr_to_dense_f32.argtypes = [i64, i64, vp, vp, vp, vp, i64, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
@@ -251,6 +252,28 @@ def csr_gemm_coded_update(S, B, precision, codes=None, w=None, alpha=1.0):
     check(lib().cn_csr_gemm_coded_update(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
                                          B.data_ptr(), _ld(B), precision.data_ptr(), codes.data_ptr(),
                                          None if w is None else w.data_ptr(), 0 if w is None else _ld(w), alpha, _stream()))
+    return codes
+
+
+def csr_gemm_coded_rmsprop(S, B, precision, rms, w, rms_multiplier, learning_rate, codes=None):
+    """codes of S B at the device scalar `precision`, then RMSprop with weight update on their decoded values."""
+    import torch
+    _need(B, torch.float32, "B")
+    _need(precision, torch.float32, "precision")
+    _need(rms, torch.float32, "rms")
+    _need(w, torch.float32, "w")
+    N = B.shape[1]
+    if B.shape[0] != S.cols or tuple(w.shape) != (S.rows, N) or tuple(rms.shape) != (S.rows, N) or _ld(rms) != _ld(w):
+        raise CnError(2, "Matrix size error: S %dx%d, B %s, w %s, rms %s" % (S.rows, S.cols, tuple(B.shape), tuple(w.shape),
+                                                                             tuple(rms.shape)))
+    if codes is None:
+        codes = torch.empty((S.rows, N), dtype=torch.uint8, device=B.device)
+    _need(codes, torch.uint8, "codes")
+    if not codes.is_contiguous() or codes.numel() != S.rows * N:
+        raise ValueError("codes must be a contiguous %d x %d uint8 tensor" % (S.rows, N))
+    check(lib().cn_csr_gemm_coded_rmsprop(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                          B.data_ptr(), _ld(B), precision.data_ptr(), codes.data_ptr(), rms.data_ptr(),
+                                          w.data_ptr(), _ld(w), rms_multiplier, learning_rate, _stream()))
     return codes
 
 

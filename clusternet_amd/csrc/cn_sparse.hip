@@ -274,11 +274,11 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
 // 64 nonzeros, take what is missing from memory as the plain kernel does.  The sums run in the same order
 // as there.
 //   kMode 1: max |S B| only            2: codes of S B            3: codes and w += alpha * decode(codes)
+//         4: codes and RMSprop with weight update on decode(codes)  (alpha = multiplier of the mean squares)
 constexpr int kRowThreads = 256;
 constexpr int kRowBlock = 16;  // rows per block
 constexpr int kBAhead = 1;     // B values are requested this many rows ahead
 constexpr int kBRing = 2 * kBAhead;
-constexpr int kWRing = 8;      // weights this many rows ahead
 constexpr int kFixed = 4;      // B rows requested ahead per row
 
 struct RowBlockMeta {
@@ -292,16 +292,18 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
     int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
     const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks, uint32_t *amax_out,
     const float *__restrict__ precision_ptr, uint8_t *__restrict__ codes, float *__restrict__ w, int64_t ldw, float alpha,
-    const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    float *__restrict__ rms, float rate, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
     float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // decode table times alpha
     const int t = threadIdx.x;
     float precision = 0.0f;
     bool exact_only = false;
+    const float rms_multiplier = alpha, one_minus = 1.0f - alpha;  // kMode 4 only
     if (kMode >= 2) {
         precision = *precision_ptr;
         exact_only = !build_table(sh, steps, step_count, precision, table);
+        if (kMode == 4) alpha = 1.0f;  // RMSprop takes the decoded gradient itself; `alpha` then carries the multiplier
         if (t < 126) {
             const float v = table[t] * precision;
             dlut[t] = alpha * v;
@@ -351,6 +353,7 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
         bool live;          // the lane's four columns exist
         uint32_t lane_off;  // byte offset of the lane's columns inside a row of B (column 0 for idle lanes)
         float *wp;          // weights of row0 at the lane's columns
+        float *rp2;         // running mean squares of row0 at the lane's columns (RMSprop)
         uint8_t *cp;        // codes of row0 at the lane's columns
     };
     auto locate = [&](int64_t unit) -> UnitPos {
@@ -363,7 +366,8 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
         p.live = n < N;
         const int64_t nc = p.live ? n : 0;
         p.lane_off = (uint32_t)(nc * (int64_t)sizeof(float));
-        p.wp = kMode == 3 ? w + p.row0 * ldw + nc : nullptr;
+        p.wp = kMode >= 3 ? w + p.row0 * ldw + nc : nullptr;
+        p.rp2 = kMode == 4 ? rms + p.row0 * ldw + nc : nullptr;
         p.cp = kMode >= 2 ? codes + p.row0 * N + nc : nullptr;
         return p;
     };
@@ -393,21 +397,23 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
             dst[s2] = *reinterpret_cast<const f32x4 *>(Bbytes + off);
         }
     };
-    auto request_w = [&](const UnitPos &p, int u, f32x4 &dst) {
+    auto request_w = [&](const UnitPos &p, int u, f32x4 &dst, f32x4 &dst2) {
         const int uu = u < p.rows ? u : p.rows - 1;
         dst = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.wp + (int64_t)uu * ldw));
+        if (kMode == 4) dst2 = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.rp2 + (int64_t)uu * ldw));
     };
 
     f32x4 b[kBRing][kFixed];
-    f32x4 wr[kWRing];
+    constexpr int kWRing = kMode == 4 ? 4 : 8;  // weights (and mean squares) this many rows ahead
+    f32x4 wr[kWRing], rr[kMode == 4 ? kWRing : 1];
     RowBlockMeta next;  // of the unit after the current one: loaded while the current one is worked on
     UnitPos pos_next = locate(unit_first < units ? unit_first : 0);
     next.rp = load_rp(pos_next.row0);
     load_nz(next.rp, next.c, next.v);
     if (unit_first < units) {  // the first unit's early requests; later units get theirs from the unit before
-        if (kMode == 3) {
+        if (kMode >= 3) {
 #pragma unroll
-            for (int u = 0; u < kWRing; ++u) request_w(pos_next, u, wr[u]);
+            for (int u = 0; u < kWRing; ++u) request_w(pos_next, u, wr[u], rr[kMode == 4 ? u : 0]);
         }
         const Ready first_ready = prepare(next);
 #pragma unroll
@@ -469,6 +475,21 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
                     if (pos.live)
                         __builtin_nontemporal_store(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24),
                                                     reinterpret_cast<uint32_t *>(pos.cp + (int64_t)u * N));
+                    if (kMode == 4) {  // kRMSprop_with_weight_update on the decoded gradient, operation by operation
+                        f32x4 wv = wr[u % kWRing], rv = rr[u % kWRing];
+                        const float g[4] = {dlut[c0], dlut[c1], dlut[c2], dlut[c3]};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float r2 = (rms_multiplier * rv[e]) + ((g[e] * g[e]) * one_minus);
+                            const float step = rate * (g[e] / (sqrtf(r2) + 1.0e-08f));
+                            rv[e] = r2;
+                            wv[e] = wv[e] - step;
+                        }
+                        if (pos.live) {
+                            __builtin_nontemporal_store(rv, reinterpret_cast<f32x4 *>(pos.rp2 + (int64_t)u * ldw));
+                            __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(pos.wp + (int64_t)u * ldw));
+                        }
+                    }
                     if (kMode == 3) {
                         f32x4 wv = wr[u % kWRing];
                         wv.x = wv.x + dlut[c0];
@@ -479,11 +500,11 @@ __global__ __launch_bounds__(kRowThreads) void csr_rows_kernel(
                     }
                 }
             }
-            if (kMode == 3) {
+            if (kMode >= 3) {
                 if (u + kWRing < kRowBlock)
-                    request_w(pos, u + kWRing, wr[u % kWRing]);
+                    request_w(pos, u + kWRing, wr[u % kWRing], rr[kMode == 4 ? u % kWRing : 0]);
                 else
-                    request_w(pos_next, u + kWRing - kRowBlock, wr[u % kWRing]);
+                    request_w(pos_next, u + kWRing - kRowBlock, wr[u % kWRing], rr[kMode == 4 ? u % kWRing : 0]);
             }
             if (u == kRowBlock / 2) {  // the next block's row pointers were requested at the top
                 load_nz(next.rp, next.c, next.v);
@@ -582,10 +603,12 @@ __global__ __launch_bounds__(kCodedThreads) void csr_gemm_coded_kernel(
     int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
     const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks,
     const float *__restrict__ precision_ptr, uint8_t *__restrict__ codes, float *__restrict__ w, int64_t ldw, float alpha,
-    const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    float *__restrict__ rms, float rate, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
     float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // decode table times alpha
+    const float rms_multiplier = alpha, one_minus = 1.0f - alpha;  // with rms: RMSprop on the decoded gradient
+    if (rms) alpha = 1.0f;
     const float precision = *precision_ptr;
     const bool exact_only = !build_table(sh, steps, step_count, precision, table);
     const int t = threadIdx.x;
@@ -656,7 +679,15 @@ __global__ __launch_bounds__(kCodedThreads) void csr_gemm_coded_kernel(
                 if (n + e < N) {
                     const uint32_t c = encode(acc[e]);
                     codes[r * N + n + e] = (uint8_t)c;
-                    if (w) w[r * ldw + n + e] = w[r * ldw + n + e] + dlut[c];
+                    if (rms) {
+                        const float g = dlut[c];
+                        const float r2 = (rms_multiplier * rms[r * ldw + n + e]) + ((g * g) * one_minus);
+                        const float step = rate * (g / (sqrtf(r2) + 1.0e-08f));
+                        rms[r * ldw + n + e] = r2;
+                        w[r * ldw + n + e] = w[r * ldw + n + e] - step;
+                    } else if (w) {
+                        w[r * ldw + n + e] = w[r * ldw + n + e] + dlut[c];
+                    }
                 }
         }
     }
@@ -844,7 +875,7 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
         if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
         hipLaunchKernelGGL(csr_rows_kernel<1>, dim3((unsigned)grid), dim3(kRowThreads), 0, st, R, N, row_ptr, col_idx, vals, B, ldb,
                            cblocks, amax, (const float *)nullptr, (uint8_t *)nullptr, (float *)nullptr, (int64_t)0, 0.0f,
-                           (const XStep *)nullptr, 0, (const float *)nullptr);
+                           (float *)nullptr, 0.0f, (const XStep *)nullptr, 0, (const float *)nullptr);
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
@@ -887,14 +918,15 @@ cn_status cn_csr_gemm_f32_absmax(int64_t R, int64_t Cc, int64_t N, const int32_t
     return csr_gemm("csr_gemm_f32_absmax", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo, absmax_out, stream);
 }
 
-cn_status cn_csr_gemm_coded_update(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
-                                   const float *vals, const float *B, int64_t ldb, const float *precision_device,
-                                   uint8_t *codes, float *w, int64_t ldw, float alpha, void *stream) {
-    if (R < 0 || Cc < 0 || N < 0) { set_error("csr_gemm_coded_update: negative dimension"); return CN_ERR_SHAPE; }
-    if (ldb < N || (w && ldw < N)) { set_error("csr_gemm_coded_update: leading dimension too small"); return CN_ERR_SHAPE; }
-    if (R > 0x7fffffffLL || Cc > 0x7fffffffLL) { set_error("csr_gemm_coded_update: more than 2^31 rows or columns"); return CN_ERR_SHAPE; }
+static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr,
+                                const int32_t *col_idx, const float *vals, const float *B, int64_t ldb,
+                                const float *precision_device, uint8_t *codes, float *w, int64_t ldw, float alpha, float *rms,
+                                float rate, void *stream) {
+    if (R < 0 || Cc < 0 || N < 0) { set_error("%s: negative dimension", who); return CN_ERR_SHAPE; }
+    if (ldb < N || (w && ldw < N)) { set_error("%s: leading dimension too small", who); return CN_ERR_SHAPE; }
+    if (R > 0x7fffffffLL || Cc > 0x7fffffffLL) { set_error("%s: more than 2^31 rows or columns", who); return CN_ERR_SHAPE; }
     if (R == 0 || N == 0) return CN_OK;
-    if (!row_ptr || !precision_device || !codes) { set_error("csr_gemm_coded_update: NULL pointer"); return CN_ERR_NULL; }
+    if (!row_ptr || !precision_device || !codes || (rms && !w)) { set_error("%s: NULL pointer", who); return CN_ERR_NULL; }
     Context *ctx;
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
@@ -908,34 +940,48 @@ cn_status cn_csr_gemm_coded_update(int64_t R, int64_t Cc, int64_t N, const int32
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<3>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<4>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         configured = true;
     }
     const bool vec = Cc > 0 && Cc * ldb < (1LL << 30) && aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0 && aligned(codes, 4) &&
-                     (!w || (aligned(w, 16) && ldw % 4 == 0));
+                     (!w || (aligned(w, 16) && ldw % 4 == 0)) && (!rms || aligned(rms, 16));
     if (vec) {
         const int64_t col_blocks = (N + 255) / 256;
         const int64_t units = ((R + kRowBlock - 1) / kRowBlock) * col_blocks;
         const int64_t per_wg = kRowThreads / 64;
         int64_t grid = (int64_t)ctx->num_cu * 3;  // the encoder table allows three workgroups per compute unit
         if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
-        if (w)
-            hipLaunchKernelGGL(csr_rows_kernel<3>, dim3((unsigned)grid), dim3(kRowThreads), lds, st, R, N, row_ptr, col_idx, vals, B,
-                               ldb, col_blocks, (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, ctx->xsteps,
-                               ctx->xstep_count, ctx->table);
-        else
-            hipLaunchKernelGGL(csr_rows_kernel<2>, dim3((unsigned)grid), dim3(kRowThreads), lds, st, R, N, row_ptr, col_idx, vals, B,
-                               ldb, col_blocks, (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, ctx->xsteps,
-                               ctx->xstep_count, ctx->table);
+        auto kernel = rms ? csr_rows_kernel<4> : (w ? csr_rows_kernel<3> : csr_rows_kernel<2>);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRowThreads), lds, st, R, N, row_ptr, col_idx, vals, B, ldb, col_blocks,
+                           (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, rms, rate, ctx->xsteps, ctx->xstep_count,
+                           ctx->table);
     } else {
         const int64_t col_blocks = (N + 1023) / 1024;
         int64_t row_groups = ((int64_t)ctx->num_cu * 3 + col_blocks - 1) / col_blocks;
         if (row_groups > (R + 1) / 2) row_groups = (R + 1) / 2;
         hipLaunchKernelGGL(csr_gemm_coded_kernel<false>, dim3((unsigned)(col_blocks * row_groups)), dim3(kCodedThreads), lds, st,
-                           R, N, row_ptr, col_idx, vals, B, ldb, col_blocks, precision_device, codes, w, ldw, alpha, ctx->xsteps,
-                           ctx->xstep_count, ctx->table);
+                           R, N, row_ptr, col_idx, vals, B, ldb, col_blocks, precision_device, codes, w, ldw, alpha, rms, rate,
+                           ctx->xsteps, ctx->xstep_count, ctx->table);
     }
     CN_HIP(hipGetLastError());
     return CN_OK;
+}
+
+cn_status cn_csr_gemm_coded_update(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                                   const float *vals, const float *B, int64_t ldb, const float *precision_device,
+                                   uint8_t *codes, float *w, int64_t ldw, float alpha, void *stream) {
+    return csr_gemm_coded("csr_gemm_coded_update", R, Cc, N, row_ptr, col_idx, vals, B, ldb, precision_device, codes, w, ldw,
+                          alpha, nullptr, 0.0f, stream);
+}
+
+cn_status cn_csr_gemm_coded_rmsprop(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                                    const float *vals, const float *B, int64_t ldb, const float *precision_device,
+                                    uint8_t *codes, float *rms, float *w, int64_t ld, float rms_multiplier,
+                                    float learning_rate, void *stream) {
+    if (!rms || !w) { set_error("csr_gemm_coded_rmsprop: NULL pointer"); return CN_ERR_NULL; }
+    return csr_gemm_coded("csr_gemm_coded_rmsprop", R, Cc, N, row_ptr, col_idx, vals, B, ldb, precision_device, codes, w, ld,
+                          rms_multiplier, rms, learning_rate, stream);
 }
 
 cn_status cn_csr_to_dense_f32(int64_t R, int64_t Cc, const int32_t *row_ptr, const int32_t *col_idx, const float *vals,

@@ -94,6 +94,14 @@ def coded_sparse_update(w, Xs, e1, rate, prec=None, codes=None):
     return codes, prec
 
 
+def coded_sparse_rmsprop_update(w, rms, Xs, e1, rms_multiplier, rate, prec=None, codes=None):
+    """RMSprop with weight update on the 8-bit round trip of X^T e1 for a sparse batch, the gradient never
+    stored: the RMSprop form of `coded_sparse_update`."""
+    prec = L.csr_gemm_absmax(Xs.csr_t, e1, prec)
+    codes = L.csr_gemm_coded_rmsprop(Xs.csr_t, e1, prec, rms, w, rms_multiplier, rate, codes)
+    return codes, prec
+
+
 def coded_rmsprop_update(w, rms, grad, rms_multiplier, rate, fused=True, scratch=None):
     """RMSprop with weight update (source/basicOps.cu:1192-1197) on the 8-bit round trip of `grad`."""
     prec = L.absmax(grad)

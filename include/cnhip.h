@@ -203,6 +203,16 @@ cn_status cn_csr_gemm_coded_update(int64_t R, int64_t C, int64_t N, const int32_
                                    int64_t ldb, const float *precision_device, uint8_t *codes_device,
                                    float *w_device, int64_t ldw, float alpha, void *stream);
 
+/* Same with RMSprop in place of the plain update: codes as above, then rms and w as cn_rmsprop_update_w8
+ * leaves them for those codes (rms and w share the leading dimension ld) -- bit for bit the sequence
+ * cn_csr_gemm_f32, cn_compress_8bit_dp, cn_rmsprop_update_w8_dp (source/basicOps.cu:1192-1197 on the
+ * round-tripped gradient), 17 bytes per element. */
+cn_status cn_csr_gemm_coded_rmsprop(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
+                                    const int32_t *col_idx_device, const float *vals_device, const float *B_device,
+                                    int64_t ldb, const float *precision_device, uint8_t *codes_device,
+                                    float *rms_device, float *w_device, int64_t ld, float rms_multiplier,
+                                    float learning_rate, void *stream);
+
 /* out[R x C] = dense form of S (zeros elsewhere).  sparse_to_dense, source/clusterNet.cpp:1034-1063. */
 cn_status cn_csr_to_dense_f32(int64_t R, int64_t C, const int32_t *row_ptr_device, const int32_t *col_idx_device,
                               const float *vals_device, float *out_device, int64_t ldo, void *stream);

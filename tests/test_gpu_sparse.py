@@ -158,6 +158,38 @@ def test_product_to_codes_and_update_equals_the_three_separate_calls(dev, R, Cc,
             assert np.array_equal(_bits(w.cpu().numpy().reshape(-1)), _bits(host_w))
 
 
+@pytest.mark.parametrize("R,Cc,N,density", [(2000, 128, 1024, 0.02), (777, 64, 4100, 0.05), (37, 211, 19, 0.05),
+                                            (301, 16, 2052, 0.0)])
+def test_product_to_codes_and_rmsprop_equals_the_separate_calls(dev, R, Cc, N, density):
+    """The RMSprop form: codes, running mean squares and weights bit for bit those of csr_gemm, absmax,
+    compression_8bit and rmsprop_update on the codes; and those of the CPU checker."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(R * 5 + N)
+    S_dense = _sparse(rng, R, Cc, density)
+    B = rng.normal(0, 0.01, (Cc, N)).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    Bd = _t(B, dev)
+    w0 = rng.normal(0, 0.05, (R, N)).astype(np.float32)
+    r0 = rng.uniform(1e-6, 1e-3, (R, N)).astype(np.float32)
+    G = L.csr_gemm(S, Bd)
+    prec = L.csr_gemm_absmax(S, Bd)
+    want_codes = L.compression_8bit(G, prec)
+    want_w, want_r = _t(w0, dev), _t(r0, dev)
+    L.rmsprop_update(want_r, want_codes, want_w, 0.9, 0.003, precision=prec)
+    w, r = _t(w0, dev), _t(r0, dev)
+    codes = L.csr_gemm_coded_rmsprop(S, Bd, prec, r, w, 0.9, 0.003)
+    assert torch.equal(codes, want_codes.view(R, N))
+    assert torch.equal(r.view(torch.int32), want_r.view(torch.int32))
+    assert torch.equal(w.view(torch.int32), want_w.view(torch.int32))
+    p_host = float(prec.cpu()[0])
+    if p_host > 0:
+        dec = oracle.port_decompress(codes.cpu().numpy().reshape(-1), p_host)
+        host_r, host_w = oracle.rmsprop_update(r0.reshape(-1), dec, w0.reshape(-1), 0.9, 0.003)
+        assert np.array_equal(_bits(r.cpu().numpy().reshape(-1)), _bits(host_r))
+        assert np.array_equal(_bits(w.cpu().numpy().reshape(-1)), _bits(host_w))
+
+
 def test_product_to_codes_takes_strided_operands(dev):
     import torch
     from clusternet_amd import _lib as L
