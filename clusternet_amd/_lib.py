@@ -186,15 +186,18 @@ def csr_from_dense(A, transpose=False):
     R, Cc = (cols, rows) if transpose else (rows, cols)
     row_ptr = torch.empty(R + 1, dtype=torch.int32, device=A.device)
     nnz = C.c_int64(0)
-    status = lib().cn_csr_from_dense_f32(A.data_ptr(), rows, cols, _ld(A), int(transpose), row_ptr.data_ptr(), None,
-                                         None, 0, C.byref(nnz), _stream())
-    if status not in (0, 5):
+    # room for one nonzero in sixteen; a denser matrix reports its count and is converted in a second call
+    capacity = max(1024, (rows * cols) // 16)
+    while True:
+        col_idx = torch.empty(max(capacity, 1), dtype=torch.int32, device=A.device)
+        vals = torch.empty(max(capacity, 1), dtype=torch.float32, device=A.device)
+        status = lib().cn_csr_from_dense_f32(A.data_ptr(), rows, cols, _ld(A), int(transpose), row_ptr.data_ptr(),
+                                             col_idx.data_ptr(), vals.data_ptr(), capacity, C.byref(nnz), _stream())
+        if status == 5 and nnz.value > capacity:
+            capacity = nnz.value
+            continue
         check(status)
-    col_idx = torch.empty(max(nnz.value, 1), dtype=torch.int32, device=A.device)
-    vals = torch.empty(max(nnz.value, 1), dtype=torch.float32, device=A.device)
-    if nnz.value:
-        check(lib().cn_csr_from_dense_f32(A.data_ptr(), rows, cols, _ld(A), int(transpose), row_ptr.data_ptr(),
-                                          col_idx.data_ptr(), vals.data_ptr(), nnz.value, C.byref(nnz), _stream()))
+        break
     return Csr(R, Cc, row_ptr, col_idx[:nnz.value], vals[:nnz.value])
 
 
