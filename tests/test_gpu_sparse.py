@@ -265,3 +265,34 @@ def test_shape_errors(dev):
     assert torch.equal(L.csr_gemm(S, torch.ones((5, 3), device=dev)), torch.zeros((4, 3), device=dev))
     T = L.csr_transpose(S)
     assert (T.rows, T.cols, T.nnz) == (5, 4, 0) and int(T.row_ptr.abs().sum()) == 0
+
+
+def test_coded_entries_report_bad_arguments_and_handle_empty_matrices(dev):
+    """Status codes of the fused entries through the C-ABI itself, and the all-zero matrix (every element
+    encodes as 'zero', whose decoded value is +precision as in decompression_8bit)."""
+    import ctypes
+    import torch
+    from clusternet_amd import _lib as L
+    lib = L.lib()
+    rng = np.random.default_rng(8)
+    S = L.csr_from_dense(_t(_sparse(rng, 40, 16, 0.2), dev))
+    B = torch.ones((16, 64), device=dev)
+    prec = L.csr_gemm_absmax(S, B)
+    codes = torch.empty((40, 64), dtype=torch.uint8, device=dev)
+    w = torch.zeros((40, 64), device=dev)
+    args = (40, 16, 64, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(), B.data_ptr(), 64)
+    assert lib.cn_csr_gemm_coded_update(*args, None, codes.data_ptr(), w.data_ptr(), 64, 1.0, None) == 1       # NULL precision
+    assert lib.cn_csr_gemm_coded_update(*args, prec.data_ptr(), None, w.data_ptr(), 64, 1.0, None) == 1        # NULL codes
+    assert lib.cn_csr_gemm_coded_update(*args, prec.data_ptr(), codes.data_ptr(), w.data_ptr(), 32, 1.0, None) == 2  # ldw < N
+    assert lib.cn_csr_gemm_coded_update(-1, 16, 64, *args[3:], prec.data_ptr(), codes.data_ptr(), None, 0, 1.0, None) == 2
+    assert lib.cn_csr_gemm_coded_rmsprop(*args, prec.data_ptr(), codes.data_ptr(), None, w.data_ptr(), 64, 0.9, 0.1, None) == 1
+    assert b"csr_gemm_coded_rmsprop" in ctypes.c_char_p(lib.cn_last_error()).value
+    assert lib.cn_csr_gemm_f32_absmax(*args, None, 0, None, None) == 1                                          # nothing to produce
+    # empty result: nothing is touched
+    assert lib.cn_csr_gemm_coded_update(0, 16, 64, *args[3:], prec.data_ptr(), codes.data_ptr(), None, 0, 1.0, None) == 0
+    # all-zero matrix with a positive precision: codes 254 throughout, weights move by alpha * precision
+    Z = L.csr_from_dense(torch.zeros((40, 16), device=dev))
+    one = torch.ones(1, device=dev)
+    got = L.csr_gemm_coded_update(Z, B, one, w=w, alpha=0.5)
+    assert int(got.min()) == 254 and int(got.max()) == 254
+    assert torch.equal(w, torch.full((40, 64), 0.5, device=dev))
