@@ -72,6 +72,8 @@ def lib():
     L.cn_host_force_gemm_tile_n.restype = None
     L.cn_host_csr_strip_kernel.argtypes = [C.c_int]
     L.cn_host_csr_strip_kernel.restype = None
+    L.cn_host_csr_lds_rows.argtypes = [C.c_int]
+    L.cn_host_csr_lds_rows.restype = None
     _lib = L
     return L
 

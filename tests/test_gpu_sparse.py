@@ -18,6 +18,16 @@ def dev():
     return torch.device("cuda:0")
 
 
+@pytest.fixture(autouse=True, params=["b_in_lds", "b_from_l2"])
+def short_row_kernel(request, dev):
+    """The max-only pass has two kernels (B strip in LDS when B has at most 128 rows, B from the L2
+    otherwise): every test runs with the first one allowed and with it switched off."""
+    from clusternet_amd import _lib as L
+    L.lib().cn_host_csr_lds_rows(1 if request.param == "b_in_lds" else 0)
+    yield
+    L.lib().cn_host_csr_lds_rows(1)
+
+
 def _t(a, dev):
     import torch
     return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
