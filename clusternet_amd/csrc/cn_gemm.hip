@@ -78,6 +78,7 @@ struct GemmArgs {
     float scale;         // fused: decode scale
     const float *table;  // fused: 126-entry codebook
     uint32_t *amax;      // optional: receives max |C| as the bit pattern of a non-negative float
+    int wide_store;      // the destination of the write-out (C, or the partial planes) allows 16-byte stores
 };
 
 // max over the wavefront of a non-negative float's bit pattern, then one atomic per wavefront.
@@ -493,21 +494,50 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
     else              { dst = g.C; ldd = g.ldc; }
     const bool want_amax = (g.amax != nullptr) && (g.splits == 1);  // with chunks the reduction does it
     uint32_t amax = 0;
+    if (g.wide_store && m0 + BM <= g.M && n0 + BN <= g.N) {
+        // Whole tile inside the matrix: every 32 x 32 block goes through a wavefront-private patch of LDS (the
+        // stages are no longer read: the last barrier of the loops is behind every wavefront) and leaves as
+        // 16-byte stores, four per lane and block instead of sixteen 4-byte ones.  Rows are padded to 36
+        // floats so that the two lane halves, four rows apart, fall into different banks.
+        constexpr int kPatchLd = 36;
+        float *patch = smem + wave * (32 * kPatchLd);
+        const int prow = lane >> 3, pcol = (lane & 7) * 4;
 #pragma unroll
-    for (int mi = 0; mi < FM; ++mi)
+        for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < FN; ++ni) {
-            const int64_t col = n0 + wave_n * (32 * FN) + ni * 32 + l32;
+            for (int ni = 0; ni < FN; ++ni) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t row = m0 + wave_m * (32 * FM) + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                if (row < g.M && col < g.N) {
-                    dst[row * ldd + col] = acc[mi][ni][r];
+                for (int r = 0; r < 16; ++r) {
+                    patch[(8 * (r >> 2) + 4 * half + (r & 3)) * kPatchLd + l32] = acc[mi][ni][r];
                     const uint32_t bits = __float_as_uint(acc[mi][ni][r]) & 0x7fffffffu;
                     amax = bits > amax ? bits : amax;
                 }
+                float *corner = dst + (m0 + wave_m * (32 * FM) + mi * 32) * ldd + n0 + wave_n * (32 * FN) + ni * 32 + pcol;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(patch + (prow + 8 * k) * kPatchLd + pcol);
+                    // the result itself is not read again soon; the partial planes are, by the chunk sum
+                    if (g.splits == 1) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(corner + (int64_t)(prow + 8 * k) * ldd));
+                    else               *reinterpret_cast<f32x4 *>(corner + (int64_t)(prow + 8 * k) * ldd) = v;
+                }
             }
-        }
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < FN; ++ni) {
+                const int64_t col = n0 + wave_n * (32 * FN) + ni * 32 + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t row = m0 + wave_m * (32 * FM) + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                    if (row < g.M && col < g.N) {
+                        dst[row * ldd + col] = acc[mi][ni][r];
+                        const uint32_t bits = __float_as_uint(acc[mi][ni][r]) & 0x7fffffffu;
+                        amax = bits > amax ? bits : amax;
+                    }
+                }
+            }
+    }
     if (want_amax) publish_absmax(amax, g.amax);
 }
 
@@ -594,6 +624,7 @@ static cn_status launch(const GemmArgs &args, int tile_n, hipStream_t st) {
 }
 
 static int g_force_tile_n = 0;
+static bool g_wide_store = true;
 
 static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_t K, const float *A,
                            int64_t lda, const void *B, int64_t ldb, float scale, float *C, int64_t ldc,
@@ -647,6 +678,8 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.vec_b = w8 ? (aligned(B, 4) && (ldb % 4 == 0)) : (aligned(B, 16) && (ldb % 4 == 0));
     a.scale = scale; a.table = ctx->table;
     a.amax = amax;
+    a.wide_store = g_wide_store && (plan.splits > 1 ? (N % 4 == 0 && (M * N) % 4 == 0)
+                                                     : (aligned(C, 16) && ldc % 4 == 0));
 
     if (w8)              s = launch<true, B_CODES>(a, plan.tile_n, st);
     else if (!ta && !tb) s = launch<true, B_IC>(a, plan.tile_n, st);
@@ -664,6 +697,9 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
 using namespace cn;
 
 extern "C" {
+
+// Test hook: 0 = write every tile with 4-byte stores.
+void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
 
 // Test and tuning hook: 0 = let the planner choose the tile width, 128 / 256 = force it.
 void cn_host_force_gemm_tile_n(int tile_n) { g_force_tile_n = (tile_n == 128 || tile_n == 256) ? tile_n : 0; }

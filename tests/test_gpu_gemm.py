@@ -162,6 +162,30 @@ def test_strided_operands_and_output_overwrite(dev):
     assert bool(torch.isnan(out_big[:, :5]).all()) and bool(torch.isnan(out_big[:, 93:]).all())
 
 
+@pytest.mark.parametrize("M,N,K,ta,tb", [(384, 512, 96, 0, 0), (640, 256, 128, 1, 0), (128, 1024, 4000, 0, 0),
+                                         (300, 520, 64, 0, 1), (256, 260, 40, 1, 1)])
+def test_wide_write_out_gives_the_same_bits(dev, M, N, K, ta, tb):
+    """Tiles that lie inside the matrix leave through LDS as 16-byte stores, the others (and everything
+    when the hook is off) as 4-byte stores: the same values either way, also in a padded output and with
+    the maximum."""
+    import torch
+    import clusternet_amd as cn
+    rng = np.random.default_rng(M + N + K)
+    A = _t(rng.normal(0, 1, (K, M) if ta else (M, K)).astype(np.float32), dev)
+    B = _t(rng.normal(0, 1, (N, K) if tb else (K, N)).astype(np.float32), dev)
+    big = torch.full((M, N + 12), float("nan"), device=dev)
+    amax = torch.zeros(1, device=dev)
+    wide = cn.gemm(A, B, bool(ta), bool(tb), out=big[:, 4:4 + N], absmax_out=amax).clone()
+    assert bool(torch.isnan(big[:, :4]).all()) and bool(torch.isnan(big[:, 4 + N:]).all())
+    cn.lib().cn_host_gemm_wide_store(0)
+    try:
+        narrow = cn.gemm(A, B, bool(ta), bool(tb))
+    finally:
+        cn.lib().cn_host_gemm_wide_store(1)
+    assert torch.equal(wide.view(torch.int32), narrow.view(torch.int32))
+    assert float(amax.cpu()[0]) == float(narrow.abs().max())
+
+
 def test_shape_errors_are_reported(dev):
     import torch
     import clusternet_amd as cn
