@@ -411,6 +411,8 @@ def _declare_layers(L):
     L.cn_sgd_update_f32.argtypes = [vp, vp, f32, sz, vp]
     L.cn_add_row_vector_f32.argtypes = [vp, vp, i64, i64, vp, vp]
     L.cn_maxout_f32.argtypes = [vp, i64, i64, C.c_int, vp, vp, vp]
+    L.cn_bias_maxout_f32.argtypes = [vp, i64, vp, i64, i64, C.c_int, vp, vp, vp]
+    L.cn_csr_gemm_bias_maxout_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, C.c_int, vp, vp, vp]
     L.cn_expand_to_maxout_grad_f32.argtypes = [vp, vp, i64, i64, C.c_int, vp, vp]
     L.cn_softmax_f32.argtypes = [vp, i64, i64, vp, vp]
     L.cn_timer_start.argtypes = [C.POINTER(vp), vp]
@@ -455,6 +457,37 @@ def maxout(A, pool):
     out = torch.empty((A.shape[0], A.shape[1] // pool), dtype=torch.float32, device=A.device)
     arg = torch.empty_like(out)
     check(L.cn_maxout_f32(A.data_ptr(), A.shape[0], A.shape[1], int(pool), out.data_ptr(), arg.data_ptr(), _stream()))
+    return out, arg
+
+
+def bias_maxout(A, v, pool):
+    """maxout(A + v) with v added to every row: (values, winners' columns), the sum never stored."""
+    import torch
+    L = _declare_layers(lib())
+    _need(A, torch.float32, "A")
+    _contig(v, "v")
+    if v.numel() != A.shape[1] or A.shape[1] % pool:
+        raise CnError(2, "Matrix size error: A %s, v %d, pool %d" % (tuple(A.shape), v.numel(), pool))
+    out = torch.empty((A.shape[0], A.shape[1] // pool), dtype=torch.float32, device=A.device)
+    arg = torch.empty_like(out)
+    check(L.cn_bias_maxout_f32(A.data_ptr(), _ld(A), v.data_ptr(), A.shape[0], A.shape[1], int(pool), out.data_ptr(),
+                               arg.data_ptr(), _stream()))
+    return out, arg
+
+
+def csr_gemm_bias_maxout(S, B, v, pool):
+    """maxout(S B + v): (values, winners' columns) of the first layer on a sparse batch."""
+    import torch
+    L = _declare_layers(lib())
+    _need(B, torch.float32, "B")
+    _contig(v, "v")
+    N = B.shape[1]
+    if B.shape[0] != S.cols or v.numel() != N or N % pool:
+        raise CnError(2, "Matrix size error: S %dx%d, B %s, v %d, pool %d" % (S.rows, S.cols, tuple(B.shape), v.numel(), pool))
+    out = torch.empty((S.rows, N // pool), dtype=torch.float32, device=B.device)
+    arg = torch.empty_like(out)
+    check(L.cn_csr_gemm_bias_maxout_f32(S.rows, S.cols, N, S.row_ptr.data_ptr(), S.col_idx.data_ptr(), S.vals.data_ptr(),
+                                        B.data_ptr(), _ld(B), v.data_ptr(), int(pool), out.data_ptr(), arg.data_ptr(), _stream()))
     return out, arg
 
 

@@ -91,6 +91,26 @@ __global__ __launch_bounds__(kT) void maxout_kernel(const float *__restrict__ A,
     }
 }
 
+// maxout_kernel on A + v (v added to every row) in one pass: the sums are formed, compared and dropped.
+__global__ __launch_bounds__(kT) void bias_maxout_kernel(const float *__restrict__ A, int64_t lda,
+                                                         const float *__restrict__ v, int64_t rows, int64_t cols, int pool,
+                                                         float *__restrict__ out, float *__restrict__ argmax) {
+    const int64_t oc = cols / pool, n = rows * oc;
+    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) {
+        const int64_t r = i / oc, o = i % oc;
+        const float *src = A + r * lda + o * pool;
+        const float *bias = v + o * pool;
+        float best = src[0] + bias[0];
+        int arg = 0;
+        for (int p = 1; p < pool; ++p) {
+            const float z = src[p] + bias[p];
+            if (best < z) { best = z; arg = p; }
+        }
+        out[i] = best;
+        argmax[i] = (float)(o * pool + arg);
+    }
+}
+
 // out (rows x pooled*pool): the pooled error lands on the winner's column, zero elsewhere.
 __global__ __launch_bounds__(kT) void expand_maxout_grad_kernel(const float *__restrict__ err,
                                                                 const float *__restrict__ argmax, int64_t rows,
@@ -238,6 +258,19 @@ cn_status cn_maxout_f32(const float *A, int64_t rows, int64_t cols, int pool, fl
     CN_REQUIRE(A && out && argmax, CN_ERR_NULL, "maxout_f32: NULL pointer");
     CN_ENTER();
     hipLaunchKernelGGL(maxout_kernel, dim3(grid_for(ctx, rows * (cols / pool))), dim3(kT), 0, st, A, rows, cols, pool, out, argmax);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+cn_status cn_bias_maxout_f32(const float *A, int64_t lda, const float *v, int64_t rows, int64_t cols, int pool, float *out,
+                             float *argmax, void *stream) {
+    CN_REQUIRE(rows >= 0 && cols >= 0 && pool >= 1 && lda >= cols, CN_ERR_SHAPE, "bias_maxout_f32: bad dimension");
+    CN_REQUIRE(cols % pool == 0, CN_ERR_SHAPE, "bias_maxout_f32: columns are not a multiple of the pool size");
+    if (rows == 0 || cols == 0) return CN_OK;
+    CN_REQUIRE(A && v && out && argmax, CN_ERR_NULL, "bias_maxout_f32: NULL pointer");
+    CN_ENTER();
+    hipLaunchKernelGGL(bias_maxout_kernel, dim3(grid_for(ctx, rows * (cols / pool))), dim3(kT), 0, st, A, lda, v, rows, cols, pool,
+                       out, argmax);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

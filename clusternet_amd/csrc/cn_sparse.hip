@@ -626,11 +626,17 @@ constexpr int kStripColumns = 256;
 constexpr int kStripGather = 16;
 typedef f32x4 f32xs;
 
+// kPool 0: out = S B (and optionally max |out|).  kPool 2 or 4: out = maxout(S B + bias) over kPool
+// consecutive columns, argmax = the winner's column as a float (first maximum wins): what add_row_vector
+// and maxout give, formed on the lane's four columns before anything is written.
+template <int kPool>
 __global__ __launch_bounds__(kT) void csr_gemm_strip_kernel(int64_t R, int64_t N, const int32_t *__restrict__ row_ptr,
                                                             const int32_t *__restrict__ col_idx,
                                                             const float *__restrict__ vals, const float *__restrict__ B,
                                                             int64_t ldb, float *__restrict__ out, int64_t ldo,
-                                                            int64_t strips, int64_t row_quads, uint32_t *amax_out) {
+                                                            int64_t strips, int64_t row_quads, uint32_t *amax_out,
+                                                            const float *__restrict__ bias, float *__restrict__ argmax,
+                                                            int64_t lda) {
     uint32_t amax = 0;
     const int64_t xcd = blockIdx.x % 8, local = blockIdx.x / 8;
     const int64_t strip = (local / row_quads) * 8 + xcd;
@@ -657,14 +663,35 @@ __global__ __launch_bounds__(kT) void csr_gemm_strip_kernel(int64_t R, int64_t N
             const f32xs b = *reinterpret_cast<const f32xs *>(Bn + (int64_t)col_idx[j] * ldb);
             acc = acc + v * b;
         }
-        if (out) __builtin_nontemporal_store(acc, reinterpret_cast<f32xs *>(out + r * ldo + n));
+        if constexpr (kPool == 0) {
+            if (out) __builtin_nontemporal_store(acc, reinterpret_cast<f32xs *>(out + r * ldo + n));
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
-            amax = bits > amax ? bits : amax;
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
+                amax = bits > amax ? bits : amax;
+            }
+        } else {
+            const f32x4 bv = *reinterpret_cast<const f32x4 *>(bias + n);
+            const float z[4] = {acc[0] + bv[0], acc[1] + bv[1], acc[2] + bv[2], acc[3] + bv[3]};
+            constexpr int kOut = 4 / kPool;
+            float best[kOut], arg[kOut];
+#pragma unroll
+            for (int o = 0; o < kOut; ++o) {
+                best[o] = z[o * kPool];
+                int a = 0;
+#pragma unroll
+                for (int p = 1; p < kPool; ++p)
+                    if (best[o] < z[o * kPool + p]) { best[o] = z[o * kPool + p]; a = p; }
+                arg[o] = (float)(n + o * kPool + a);
+            }
+#pragma unroll
+            for (int o = 0; o < kOut; ++o) {
+                out[r * ldo + n / kPool + o] = best[o];
+                argmax[r * lda + n / kPool + o] = arg[o];
+            }
         }
     }
-    if (amax_out) {
+    if (kPool == 0 && amax_out) {
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
             const uint32_t o = (uint32_t)__shfl_xor((int)amax, off, 64);
@@ -996,8 +1023,8 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
     if (vec && g_strip_kernel && row_quads <= ctx->num_cu / 8 && N >= 8 * kStripColumns) {
         const int64_t strips = (N + kStripColumns - 1) / kStripColumns;
         const int64_t grid = ((strips + 7) / 8) * row_quads * 8;
-        hipLaunchKernelGGL(csr_gemm_strip_kernel, dim3((unsigned)grid), dim3(kT), 0, st, R, N, row_ptr, col_idx, vals, B, ldb, out, ldo,
-                           strips, row_quads, amax);
+        hipLaunchKernelGGL(csr_gemm_strip_kernel<0>, dim3((unsigned)grid), dim3(kT), 0, st, R, N, row_ptr, col_idx, vals, B, ldb, out,
+                           ldo, strips, row_quads, amax, (const float *)nullptr, (float *)nullptr, (int64_t)0);
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
@@ -1017,6 +1044,45 @@ void cn_host_csr_lds_rows(int enabled) { g_lds_rows = enabled != 0; }
 cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
                           const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, void *stream) {
     return csr_gemm("csr_gemm_f32", R, Cc, N, row_ptr, col_idx, vals, B, ldb, out, ldo, nullptr, stream);
+}
+
+cn_status cn_csr_gemm_bias_maxout_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
+                                      const float *vals, const float *B, int64_t ldb, const float *bias, int pool, float *out,
+                                      float *argmax, void *stream) {
+    if (pool < 1 || N % (pool > 0 ? pool : 1) != 0) { set_error("csr_gemm_bias_maxout_f32: columns are not a multiple of the pool size"); return CN_ERR_SHAPE; }
+    cn_status s = check_csr_args("csr_gemm_bias_maxout_f32", R, Cc, N, row_ptr, col_idx, vals, B, ldb, nullptr, 0);
+    if (s != CN_OK) return s;
+    if (R == 0 || N == 0) return CN_OK;
+    if (!bias || !out || !argmax) { set_error("csr_gemm_bias_maxout_f32: NULL pointer"); return CN_ERR_NULL; }
+    Context *ctx;
+    s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t pooled = N / pool;
+    const int64_t row_quads = (R + 3) / 4;
+    const bool in_kernel = (pool == 2 || pool == 4) && g_strip_kernel && row_quads <= ctx->num_cu / 8 && N >= 8 * kStripColumns &&
+                           aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0 && aligned(bias, 16);
+    if (in_kernel) {
+        const int64_t strips = (N + kStripColumns - 1) / kStripColumns;
+        const int64_t grid = ((strips + 7) / 8) * row_quads * 8;
+        if (pool == 2)
+            hipLaunchKernelGGL(csr_gemm_strip_kernel<2>, dim3((unsigned)grid), dim3(kT), 0, st, R, N, row_ptr, col_idx, vals, B, ldb, out,
+                               pooled, strips, row_quads, (uint32_t *)nullptr, bias, argmax, pooled);
+        else
+            hipLaunchKernelGGL(csr_gemm_strip_kernel<4>, dim3((unsigned)grid), dim3(kT), 0, st, R, N, row_ptr, col_idx, vals, B, ldb, out,
+                               pooled, strips, row_quads, (uint32_t *)nullptr, bias, argmax, pooled);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
+    // any other shape: the product into the workspace, then bias and maxout in one pass over it
+    if ((size_t)R * (size_t)N * sizeof(float) > ctx->workspace_bytes) {
+        set_error("csr_gemm_bias_maxout_f32: product does not fit the workspace");
+        return CN_ERR_WORKSPACE;
+    }
+    float *z = reinterpret_cast<float *>(ctx->workspace);
+    s = csr_gemm("csr_gemm_bias_maxout_f32", R, Cc, N, row_ptr, col_idx, vals, B, ldb, z, N, nullptr, stream);
+    if (s != CN_OK) return s;
+    return cn_bias_maxout_f32(z, N, bias, R, N, pool, out, argmax, stream);
 }
 
 cn_status cn_csr_gemm_f32_absmax(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,

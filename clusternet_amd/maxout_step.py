@@ -32,11 +32,12 @@ def sparse_input(X):
 
 def forward(X, params, pool=2):
     W1, b1, W2, b2, W3, b3 = params
-    xw = L.csr_gemm(X.csr, W1) if isinstance(X, SparseInput) else L.dot(X, W1)
-    z1 = L.add_row_vector(xw, b1)
-    h1, a1 = L.maxout(z1, pool)
-    z2 = L.add_row_vector(L.dot(h1, W2), b2)
-    h2, a2 = L.maxout(z2, pool)
+    # bias and maxout are taken in one pass behind each product (inside it for the sparse first layer)
+    if isinstance(X, SparseInput):
+        h1, a1 = L.csr_gemm_bias_maxout(X.csr, W1, b1, pool)
+    else:
+        h1, a1 = L.bias_maxout(L.dot(X, W1), b1, pool)
+    h2, a2 = L.bias_maxout(L.dot(h1, W2), b2, pool)
     p = L.softmax(L.add_row_vector(L.dot(h2, W3), b3))
     return p, (h1, a1, h2, a2)
 

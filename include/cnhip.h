@@ -182,6 +182,15 @@ cn_status cn_csr_gemm_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_pt
                           const int32_t *col_idx_device, const float *vals_device, const float *B_device,
                           int64_t ldb, float *out_device, int64_t ldo, void *stream);
 
+/* out, argmax [R x N/pool, contiguous] = maxout(S B + bias): cn_csr_gemm_f32, cn_add_row_vector_f32 and
+ * cn_maxout_f32 in one call, the same values.  For a batch of few long rows (the first layer of the forward
+ * pass, source/Layer.cpp:250-258) and pool 2 or 4 the bias and the maximum are taken in the product's write-out
+ * and S B is never stored; other shapes go through the library's workspace. */
+cn_status cn_csr_gemm_bias_maxout_f32(int64_t R, int64_t C, int64_t N, const int32_t *row_ptr_device,
+                                      const int32_t *col_idx_device, const float *vals_device, const float *B_device,
+                                      int64_t ldb, const float *bias_device, int pool, float *out_device,
+                                      float *argmax_device, void *stream);
+
 /* cn_csr_gemm_f32 that also writes max |out[i][j]| to *absmax_out_device (equal bit for bit to
  * cn_absmax_f32 over the result; -1.0f for an empty one): the sparse weight gradient X^T E followed by
  * the max(abs(grad)) in front of compression_8bit (source/Layer.cpp:318-321,
@@ -249,6 +258,11 @@ cn_status cn_sgd_update_f32(float *w_device, const float *grad_device, float rat
 /* out[r][c] = A[r][c] + v[c].  addMatrixVector, source/basicOps.cu:966-974. */
 cn_status cn_add_row_vector_f32(const float *A_device, const float *v_device, int64_t rows,
                                 int64_t cols, float *out_device, void *stream);
+/* out, argmax = maxout(A + v) as cn_add_row_vector_f32 followed by cn_maxout_f32 give them, in one pass and
+ * without the sum in memory (A with leading dimension lda; out and argmax rows x cols/pool, contiguous).
+ * The bias-and-maxout step behind every dot of the forward pass, source/Layer.cpp:256-258. */
+cn_status cn_bias_maxout_f32(const float *A_device, int64_t lda, const float *v_device, int64_t rows, int64_t cols,
+                             int pool, float *out_device, float *argmax_device, void *stream);
 /* Maxout over `pool` consecutive columns: out and argmax are rows x cols/pool; argmax holds the
  * winner's absolute column index as a float, first maximum wins.  maxout,
  * source/basicOps.cu:1272-1299 (defined by the expectations of tests/basicOps_test.cu:580-610). */

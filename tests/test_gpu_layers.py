@@ -53,6 +53,24 @@ def test_helpers_match_checker(dev):
     assert arg.cpu().numpy().tolist() == [[0.0, 3.0]]
 
 
+@pytest.mark.parametrize("rows,cols,pool", [(128, 8192, 2), (7, 12, 3), (33, 260, 4), (1, 2, 1), (5, 64, 64)])
+def test_bias_and_maxout_in_one_pass_equal_the_two_kernels(dev, rows, cols, pool):
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(rows + cols)
+    A = rng.normal(0, 1, (rows, cols + 3)).astype(np.float32)
+    A[:, 1::2] = A[:, 0:-1:2][:, :A[:, 1::2].shape[1]]            # many ties between pool neighbours
+    v = rng.normal(0, 0.1, cols).astype(np.float32)
+    v[1::2] = v[0::2][:v[1::2].size]
+    Ad = _t(A, dev)[:, :cols]                                        # leading dimension above the width
+    out, arg = L.bias_maxout(Ad, _t(v, dev), pool)
+    want_out, want_arg = L.maxout(L.add_row_vector(Ad.contiguous(), _t(v, dev)), pool)
+    assert torch.equal(out.view(torch.int32), want_out.view(torch.int32)) and torch.equal(arg, want_arg)
+    z = oracle.add_row_vector(np.ascontiguousarray(A[:, :cols]), v)
+    h, a = oracle.maxout(z, pool)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), h.view(np.uint32)) and np.array_equal(arg.cpu().numpy(), a)
+
+
 def _cpu_step(X, onehot, params, rate, pool):
     W1, b1, W2, b2, W3, b3 = params
     z1 = oracle.add_row_vector(oracle.gemm(X, W1), b1)

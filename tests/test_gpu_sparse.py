@@ -121,6 +121,26 @@ def test_few_long_rows_take_the_strip_kernel_with_the_same_bits(dev, R, Cc, N, d
     assert float(amax.cpu()[0]) == float(oracle.absmax(want))
 
 
+@pytest.mark.parametrize("R,Cc,N,density,pool", [(128, 3000, 4096, 0.02, 2), (100, 700, 2048, 0.1, 4), (128, 300, 8192, 0.05, 2),
+                                                 (37, 211, 18, 0.05, 3), (300, 64, 4100, 0.1, 2), (5, 9, 6, 0.5, 6)])
+def test_product_bias_maxout_in_one_call_equals_the_three_kernels(dev, R, Cc, N, density, pool):
+    """Few long rows take bias and maximum in the product's write-out, other shapes go through the
+    workspace: either way the values and winners of csr_gemm, add_row_vector and maxout."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(R + N + pool)
+    S_dense = _sparse(rng, R, Cc, density)
+    B = rng.normal(0, 1, (Cc, N)).astype(np.float32)
+    v = rng.normal(0, 0.1, N).astype(np.float32)
+    S = L.csr_from_dense(_t(S_dense, dev))
+    out, arg = L.csr_gemm_bias_maxout(S, _t(B, dev), _t(v, dev), pool)
+    want_out, want_arg = L.maxout(L.add_row_vector(L.csr_gemm(S, _t(B, dev)), _t(v, dev)), pool)
+    assert torch.equal(out.view(torch.int32), want_out.view(torch.int32)) and torch.equal(arg, want_arg)
+    z = oracle.add_row_vector(oracle.csr_gemm(oracle.csr_from_dense(S_dense), B), v)
+    h, a = oracle.maxout(z, pool)
+    assert np.array_equal(_bits(out.cpu().numpy()), _bits(h)) and np.array_equal(arg.cpu().numpy(), a)
+
+
 def test_gather_product_absmax_of_an_empty_result(dev):
     import torch
     from clusternet_amd import _lib as L
