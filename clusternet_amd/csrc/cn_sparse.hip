@@ -624,7 +624,6 @@ __global__ void preset_word_kernel(uint32_t *p, uint32_t value) {
 // Sums and results as in csr_gemm_kernel.
 constexpr int kStripColumns = 256;
 constexpr int kStripGather = 16;
-typedef f32x4 f32xs;
 
 // kPool 0: out = S B (and optionally max |out|).  kPool 2 or 4: out = maxout(S B + bias) over kPool
 // consecutive columns, argmax = the winner's column as a float (first maximum wins): what add_row_vector
@@ -645,26 +644,26 @@ __global__ __launch_bounds__(kT) void csr_gemm_strip_kernel(int64_t R, int64_t N
     if (strip < strips && r < R && n < N) {
         const int32_t j0 = row_ptr[r], j1 = row_ptr[r + 1];
         const float *Bn = B + n;
-        f32xs acc = 0.0f;
+        f32x4 acc = 0.0f;
         int32_t j = j0;
         for (; j + kStripGather <= j1; j += kStripGather) {
             int32_t c[kStripGather];
             float v[kStripGather];
-            f32xs b[kStripGather];
+            f32x4 b[kStripGather];
 #pragma unroll
             for (int u = 0; u < kStripGather; ++u) { c[u] = col_idx[j + u]; v[u] = vals[j + u]; }
 #pragma unroll
-            for (int u = 0; u < kStripGather; ++u) b[u] = *reinterpret_cast<const f32xs *>(Bn + (int64_t)c[u] * ldb);
+            for (int u = 0; u < kStripGather; ++u) b[u] = *reinterpret_cast<const f32x4 *>(Bn + (int64_t)c[u] * ldb);
 #pragma unroll
             for (int u = 0; u < kStripGather; ++u) acc = acc + v[u] * b[u];
         }
         for (; j < j1; ++j) {
             const float v = vals[j];
-            const f32xs b = *reinterpret_cast<const f32xs *>(Bn + (int64_t)col_idx[j] * ldb);
+            const f32x4 b = *reinterpret_cast<const f32x4 *>(Bn + (int64_t)col_idx[j] * ldb);
             acc = acc + v * b;
         }
         if constexpr (kPool == 0) {
-            if (out) __builtin_nontemporal_store(acc, reinterpret_cast<f32xs *>(out + r * ldo + n));
+            if (out) __builtin_nontemporal_store(acc, reinterpret_cast<f32x4 *>(out + r * ldo + n));
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const uint32_t bits = __float_as_uint(acc[e]) & 0x7fffffffu;
@@ -702,16 +701,16 @@ __global__ __launch_bounds__(kT) void csr_gemm_strip_kernel(int64_t R, int64_t N
 }
 
 // ---- product -> codes -> update, without the product ever reaching memory -------------------------------
-// codes = compression_8bit(S B, *precision) and, if w is given, w += alpha * decompression_8bit(codes):
-// the weight gradient of the first layer, its 8-bit codes for the exchange and the update of the weights
-// in one pass that writes one byte per element and reads and writes the weights once.  Recomputing a row of
-// S B costs its few nonzeros; the precision (max |S B|) comes from a first pass that stores nothing.
-// Every value is computed, encoded and decoded exactly as by csr_gemm, compress and decompress_axpy.
-// Two rows per iteration and workgroup (512 threads) so that three workgroups with their 40 KB encoder
-// table fill the wavefront slots of a compute unit.
+// codes = compression_8bit(S B, *precision) and, if w is given, w += alpha * decompression_8bit(codes) (or
+// RMSprop with weight update on the decoded values): the weight gradient of the first layer, its 8-bit
+// codes for the exchange and the update of the weights in one pass that writes one byte per element and
+// reads and writes the weights once.  Recomputing a row of S B costs its few nonzeros; the precision
+// (max |S B|) comes from a first pass that stores nothing.  Every value is computed, encoded and decoded
+// exactly as by csr_gemm, compress and decompress_axpy.
+// This kernel is the plain form for operands that do not allow 16-byte accesses: one element at a time, row
+// after row; csr_rows_kernel below is the one that is tuned.
 constexpr int kCodedThreads = 512;
 
-template <bool kVector>
 __global__ __launch_bounds__(kCodedThreads) void csr_gemm_coded_kernel(
     int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
     const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks,
@@ -748,39 +747,7 @@ __global__ __launch_bounds__(kCodedThreads) void csr_gemm_coded_kernel(
     const int64_t n = cb * 1024 + 4 * (int64_t)(t & 255);
     for (int64_t r = rg * 2 + slot; r < R; r += row_groups * 2) {
         const int32_t j0 = row_ptr[r], j1 = row_ptr[r + 1];
-        if (kVector) {
-            if (n >= N) continue;
-            f32x4 wv = {0.f, 0.f, 0.f, 0.f};
-            if (w) wv = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(w + r * ldw + n));
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-            int32_t j = j0;
-            for (; j + kGather <= j1; j += kGather) {
-                int32_t c[kGather];
-                float v[kGather];
-                f32x4 b[kGather];
-#pragma unroll
-                for (int u = 0; u < kGather; ++u) { c[u] = col_idx[j + u]; v[u] = vals[j + u]; }
-#pragma unroll
-                for (int u = 0; u < kGather; ++u) b[u] = *reinterpret_cast<const f32x4 *>(B + (int64_t)c[u] * ldb + n);
-#pragma unroll
-                for (int u = 0; u < kGather; ++u) acc = acc + v[u] * b[u];
-            }
-            for (; j < j1; ++j) {
-                const float v = vals[j];
-                const f32x4 b = *reinterpret_cast<const f32x4 *>(B + (int64_t)col_idx[j] * ldb + n);
-                acc = acc + v * b;
-            }
-            const uint32_t c0 = encode(acc.x), c1 = encode(acc.y), c2 = encode(acc.z), c3 = encode(acc.w);
-            __builtin_nontemporal_store(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24),
-                                        reinterpret_cast<uint32_t *>(codes + r * N + n));
-            if (w) {
-                wv.x = wv.x + dlut[c0];
-                wv.y = wv.y + dlut[c1];
-                wv.z = wv.z + dlut[c2];
-                wv.w = wv.w + dlut[c3];
-                __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(w + r * ldw + n));
-            }
-        } else {
+        {
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
             for (int32_t j = j0; j < j1; ++j) {
                 const float v = vals[j];
@@ -1108,7 +1075,7 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
     const int lds = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
     static bool configured = false;
     if (!configured) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_gemm_coded_kernel<false>),
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_gemm_coded_kernel),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<2>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -1134,7 +1101,7 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
         const int64_t col_blocks = (N + 1023) / 1024;
         int64_t row_groups = ((int64_t)ctx->num_cu * 3 + col_blocks - 1) / col_blocks;
         if (row_groups > (R + 1) / 2) row_groups = (R + 1) / 2;
-        hipLaunchKernelGGL(csr_gemm_coded_kernel<false>, dim3((unsigned)(col_blocks * row_groups)), dim3(kCodedThreads), lds, st,
+        hipLaunchKernelGGL(csr_gemm_coded_kernel, dim3((unsigned)(col_blocks * row_groups)), dim3(kCodedThreads), lds, st,
                            R, N, row_ptr, col_idx, vals, B, ldb, col_blocks, precision_device, codes, w, ldw, alpha, rms, rate,
                            ctx->xsteps, ctx->xstep_count, ctx->table);
     }
