@@ -6,12 +6,15 @@
 // CSR form (row_ptr[R + 1], col_idx[nnz] ascending within a row, vals[nnz]), 32-bit indices.
 //
 //   csr_gemm        out[R x N] = S B: every output row gathers the B rows of its nonzeros, four columns
-//                   per lane, accumulators in registers.  Rows are processed by workgroups that run
-//                   side by side and walk their nonzeros in ascending order, so a B row needed by
-//                   several output rows is fetched from HBM once and served from L2 afterwards
+//                   per lane, accumulators in registers.  Three kernels by shape: many rows (one
+//                   workgroup per row and 1024 columns), few long rows (one wavefront per row and
+//                   256-column strip, a strip per XCD; optionally with bias and maxout in the write-out),
+//                   and many short rows (blocks of 16 rows, loads requested rows ahead) for the passes
+//                   that never store the product: its maximum, its 8-bit codes, and the weight update
 //   csr_transpose   CSR(S) -> CSR(S^T), for the products with the transposed sparse operand
+//   csr_from_dense, csr_to_dense   the conversions
 //
-// With X the 128 x 100000 batch:  X W = CSR(X) W and X^T E = CSR(X^T) E, both through csr_gemm.
+// With X the 128 x 100000 batch:  X W = CSR(X) W and X^T E = CSR(X^T) E.
 // Sums run over the nonzeros in ascending order with a rounded product and a rounded addition per
 // term, so the results are reproducible to the bit.
 #include "cn_internal.h"
