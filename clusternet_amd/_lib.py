@@ -54,6 +54,8 @@ def lib():
     L.cn_stream_yardstick.argtypes = [C.c_int, vp, vp, sz, C.c_int, vp]
     L.cn_csr_gemm_coded_update.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, i64, f32, vp]
     L.cn_csr_gemm_coded_rmsprop.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, vp, i64, f32, f32, vp]
+    L.cn_compress_8bit_axpy.argtypes = [vp, f32, sz, vp, f32, vp, vp]
+    L.cn_compress_8bit_axpy_dp.argtypes = [vp, vp, sz, vp, f32, vp, vp]
     L.cn_csr_to_dense_f32.argtypes = [i64, i64, vp, vp, vp, vp, i64, vp]
     L.cn_absmax_f32.argtypes = [vp, sz, vp, vp]
     L.cn_compress_8bit.argtypes = [vp, f32, sz, vp, vp]
@@ -338,6 +340,28 @@ def compression_8bit(A, precision, out=None):
         check(lib().cn_compress_8bit_dp(A.data_ptr(), precision.data_ptr(), A.numel(), out.data_ptr(), _stream()))
     else:
         check(lib().cn_compress_8bit(A.data_ptr(), float(precision), A.numel(), out.data_ptr(), _stream()))
+    return out
+
+
+def compression_8bit_axpy(A, precision, alpha, y, out=None):
+    """codes of A / precision and y += alpha * decode(codes) in one pass; returns the codes."""
+    import torch
+    _need(A, torch.float32, "A")
+    _need(y, torch.float32, "y")
+    if not A.is_contiguous() or not y.is_contiguous() or y.numel() != A.numel():
+        raise ValueError("A and y must be contiguous and of one size")
+    if out is None:
+        out = torch.empty(A.shape, dtype=torch.uint8, device=A.device)
+    _need(out, torch.uint8, "out")
+    if not out.is_contiguous() or out.numel() != A.numel():
+        raise ValueError("out must be a contiguous uint8 tensor of A's size")
+    if isinstance(precision, torch.Tensor):
+        _need(precision, torch.float32, "precision")
+        check(lib().cn_compress_8bit_axpy_dp(A.data_ptr(), precision.data_ptr(), A.numel(), out.data_ptr(), alpha,
+                                             y.data_ptr(), _stream()))
+    else:
+        check(lib().cn_compress_8bit_axpy(A.data_ptr(), float(precision), A.numel(), out.data_ptr(), alpha, y.data_ptr(),
+                                          _stream()))
     return out
 
 

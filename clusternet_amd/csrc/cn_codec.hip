@@ -17,15 +17,32 @@ constexpr int kTileVec = kThreads * kVecPerThread;       // float4 per workgroup
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <bool kVector>
+// kUpdate: besides the codes, y += alpha * (decoded value of each code), as decompress_axpy would add it
+// afterwards: the gradient's codes for the exchange and the own weight update in one pass over both arrays.
+template <bool kVector, bool kUpdate>
 __global__ __launch_bounds__(kThreads) void compress_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr,
     size_t n, uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count,
-    const float *__restrict__ table) {
+    const float *__restrict__ table, float alpha, float *__restrict__ y) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // kUpdate: decode table times alpha
     const float precision = precision_ptr ? *precision_ptr : precision_value;
     const bool exact_only = !build_table(sh, steps, step_count, precision, table);
+    if (kUpdate) {
+        const int t = threadIdx.x;
+        if (t < 126) {
+            const float v = table[t] * precision;
+            dlut[t] = alpha * v;
+            dlut[t + 128] = alpha * (-v);
+        } else if (t == 126) {
+            dlut[126] = alpha * precision;
+            dlut[127] = alpha * precision;
+            dlut[254] = alpha * precision;
+            dlut[255] = alpha * (-precision);
+        }
+        __syncthreads();
+    }
     const uint32_t first = xlut_first(precision);
     auto encode = [&](float v) -> uint32_t {
         const uint32_t bits = __float_as_uint(v);
@@ -37,15 +54,17 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
         const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
         uint32_t *c4 = reinterpret_cast<uint32_t *>(codes);
         const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
-        auto load_tile = [&](size_t tile, f32x4 (&v)[kVecPerThread]) {
+        f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
+        auto load_tile = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kVecPerThread]) {
             const size_t base = tile * kTileVec + threadIdx.x;
 #pragma unroll
             for (int j = 0; j < kVecPerThread; ++j) {
                 size_t i = base + (size_t)j * kThreads;
                 v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
+                if (kUpdate) w[j] = (i < nvec) ? __builtin_nontemporal_load(&y4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
         };
-        auto encode_tile = [&](size_t tile, const f32x4 (&v)[kVecPerThread]) {
+        auto encode_tile = [&](size_t tile, const f32x4 (&v)[kVecPerThread], f32x4 (&w)[kVecPerThread]) {
             const size_t base = tile * kTileVec + threadIdx.x;
             uint32_t packed[kVecPerThread];
             if (!exact_only) {
@@ -63,33 +82,54 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
             for (int j = 0; j < kVecPerThread; ++j) {
                 size_t i = base + (size_t)j * kThreads;
                 if (i < nvec) __builtin_nontemporal_store(packed[j], &c4[i]);
+                if (kUpdate) {
+                    f32x4 o;
+                    o.x = w[j].x + dlut[packed[j] & 0xffu];
+                    o.y = w[j].y + dlut[(packed[j] >> 8) & 0xffu];
+                    o.z = w[j].z + dlut[(packed[j] >> 16) & 0xffu];
+                    o.w = w[j].w + dlut[packed[j] >> 24];
+                    if (i < nvec) __builtin_nontemporal_store(o, &y4[i]);
+                }
             }
         };
         // Two register sets: the loads of the next tile are in flight while this one is encoded,
         // so the memory pipe stays busy even with only two wavefronts per SIMD.
-        f32x4 va[kVecPerThread], vb[kVecPerThread];
+        f32x4 va[kVecPerThread], vb[kVecPerThread], wa[kUpdate ? kVecPerThread : 1], wb[kUpdate ? kVecPerThread : 1];
+        auto load = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kUpdate ? kVecPerThread : 1]) {
+            load_tile(tile, v, reinterpret_cast<f32x4 (&)[kVecPerThread]>(w));
+        };
+        auto finish = [&](size_t tile, const f32x4 (&v)[kVecPerThread], f32x4 (&w)[kUpdate ? kVecPerThread : 1]) {
+            encode_tile(tile, v, reinterpret_cast<f32x4 (&)[kVecPerThread]>(w));
+        };
         size_t t0 = blockIdx.x;
         if (t0 < tiles) {
-            load_tile(t0, va);
+            load(t0, va, wa);
             for (;;) {
                 const size_t t1 = t0 + gridDim.x;
-                if (t1 < tiles) load_tile(t1, vb);
-                encode_tile(t0, va);
+                if (t1 < tiles) load(t1, vb, wb);
+                finish(t0, va, wa);
                 if (t1 >= tiles) break;
                 t0 = t1 + gridDim.x;
-                if (t0 < tiles) load_tile(t0, va);
-                encode_tile(t1, vb);
+                if (t0 < tiles) load(t0, va, wa);
+                finish(t1, vb, wb);
                 if (t0 >= tiles) break;
             }
         }
         // ragged tail (n % 4 elements)
         if (blockIdx.x == 0) {
             size_t i = nvec * 4 + threadIdx.x;
-            if (i < n) codes[i] = (uint8_t)(exact_only ? encode_exact(x[i], precision, sh.slot) : encode(x[i]));
+            if (i < n) {
+                const uint32_t c = exact_only ? encode_exact(x[i], precision, sh.slot) : encode(x[i]);
+                codes[i] = (uint8_t)c;
+                if (kUpdate) y[i] = y[i] + dlut[c];
+            }
         }
     } else {
-        for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
-            codes[i] = (uint8_t)(exact_only ? encode_exact(x[i], precision, sh.slot) : encode(x[i]));
+        for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads) {
+            const uint32_t c = exact_only ? encode_exact(x[i], precision, sh.slot) : encode(x[i]);
+            codes[i] = (uint8_t)c;
+            if (kUpdate) y[i] = y[i] + dlut[c];
+        }
     }
 }
 
@@ -263,10 +303,10 @@ static int stream_grid(const Context *ctx, size_t n, int per_cu) {
     return (int)(g < 1 ? 1 : g);
 }
 
-static cn_status compress_impl(const float *x, float precision, const float *precision_dev, size_t n,
-                               uint8_t *codes, void *stream) {
+static cn_status compress_impl(const char *who, const float *x, float precision, const float *precision_dev, size_t n,
+                               uint8_t *codes, float alpha, float *y, void *stream) {
     if (n == 0) return CN_OK;
-    if (!x || !codes) { set_error("compress_8bit: NULL pointer"); return CN_ERR_NULL; }
+    if (!x || !codes) { set_error("%s: NULL pointer", who); return CN_ERR_NULL; }
     Context *ctx;
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
@@ -274,20 +314,25 @@ static cn_status compress_impl(const float *x, float precision, const float *pre
     // two workgroups per CU: mixed read/write streams run fastest on this part with few wavefronts
     // in flight, and the kernel keeps its own next tile in flight to stay busy at that occupancy
     int grid = stream_grid(ctx, n, 2);
+    const int lds = (int)sizeof(EncodeShared) + (y ? 256 * (int)sizeof(float) : 0);
     static bool configured = false;
     if (!configured) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
+        const int most = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<true, false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<false, false>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<true, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<false, true>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
         configured = true;
     }
-    if (aligned(x, 16) && aligned(codes, 4))
-        hipLaunchKernelGGL(compress_kernel<true>, dim3(grid), dim3(kThreads), sizeof(EncodeShared), st, x, precision,
-                           precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
-    else
-        hipLaunchKernelGGL(compress_kernel<false>, dim3(grid), dim3(kThreads), sizeof(EncodeShared), st, x, precision,
-                           precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
+    const bool vec = aligned(x, 16) && aligned(codes, 4) && (!y || aligned(y, 16));
+    auto kernel = y ? (vec ? compress_kernel<true, true> : compress_kernel<false, true>)
+                    : (vec ? compress_kernel<true, false> : compress_kernel<false, false>);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, st, x, precision, precision_dev, n, codes, ctx->xsteps,
+                       ctx->xstep_count, ctx->table, alpha, y);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -318,13 +363,25 @@ using namespace cn;
 extern "C" {
 
 cn_status cn_compress_8bit(const float *x, float precision, size_t n, uint8_t *codes, void *stream) {
-    return compress_impl(x, precision, nullptr, n, codes, stream);
+    return compress_impl("compress_8bit", x, precision, nullptr, n, codes, 0.0f, nullptr, stream);
 }
 
 cn_status cn_compress_8bit_dp(const float *x, const float *precision_device, size_t n, uint8_t *codes,
                               void *stream) {
     if (n != 0 && !precision_device) { set_error("compress_8bit_dp: NULL precision"); return CN_ERR_NULL; }
-    return compress_impl(x, 0.0f, precision_device, n, codes, stream);
+    return compress_impl("compress_8bit_dp", x, 0.0f, precision_device, n, codes, 0.0f, nullptr, stream);
+}
+
+cn_status cn_compress_8bit_axpy(const float *x, float precision, size_t n, uint8_t *codes, float alpha, float *y,
+                                void *stream) {
+    if (n != 0 && !y) { set_error("compress_8bit_axpy: NULL pointer"); return CN_ERR_NULL; }
+    return compress_impl("compress_8bit_axpy", x, precision, nullptr, n, codes, alpha, y, stream);
+}
+
+cn_status cn_compress_8bit_axpy_dp(const float *x, const float *precision_device, size_t n, uint8_t *codes, float alpha,
+                                   float *y, void *stream) {
+    if (n != 0 && (!precision_device || !y)) { set_error("compress_8bit_axpy_dp: NULL pointer"); return CN_ERR_NULL; }
+    return compress_impl("compress_8bit_axpy_dp", x, 0.0f, precision_device, n, codes, alpha, y, stream);
 }
 
 cn_status cn_decompress_8bit(const uint8_t *codes, float precision, size_t n, float *out, void *stream) {

@@ -77,11 +77,10 @@ def coded_update(w, grad, rate, fused=True, scratch=None, prec=None):
     `prec` = max|grad| on the device if the caller already has it."""
     if prec is None:
         prec = L.absmax(grad)
-    codes = L.compression_8bit(grad, prec)
     if fused:
-        L.decompression_8bit_axpy(codes, prec, -rate, w)
-    else:
-        L.sgd_update(w, L.decompression_8bit(codes, prec, out=grad if scratch is None else scratch), rate)
+        return L.compression_8bit_axpy(grad, prec, -rate, w), prec
+    codes = L.compression_8bit(grad, prec)
+    L.sgd_update(w, L.decompression_8bit(codes, prec, out=grad if scratch is None else scratch), rate)
     return codes, prec
 
 

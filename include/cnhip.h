@@ -121,6 +121,14 @@ cn_status cn_compress_8bit(const float *x_device, float precision, size_t n,
 cn_status cn_compress_8bit_dp(const float *x_device, const float *precision_device, size_t n,
                               uint8_t *codes_device, void *stream);
 
+/* cn_compress_8bit followed by cn_decompress_8bit_axpy on its codes, in one pass: codes[i] as above and
+ * y[i] += alpha * (decoded value of codes[i]).  A gradient's codes for the exchange and the own weight
+ * update (source/Layer.cpp:365, 430-433) at 13 bytes per element instead of 5 + 9; same bits. */
+cn_status cn_compress_8bit_axpy(const float *x_device, float precision, size_t n, uint8_t *codes_device,
+                                float alpha, float *y_device, void *stream);
+cn_status cn_compress_8bit_axpy_dp(const float *x_device, const float *precision_device, size_t n,
+                                   uint8_t *codes_device, float alpha, float *y_device, void *stream);
+
 /* out[i] = lut[codes[i]] with lut[c] = table[c] * precision, lut[c + 128] = -lut[c] (c < 126),
  * lut[126] = lut[127] = lut[254] = +precision, lut[255] = -precision: bit-exact with
  * kDecompression_8bit (source/clusterKernels.cu:1135-1160; launcher source/basicOps.cu:1172-1176).

@@ -65,6 +65,50 @@ def test_decompress_axpy_equals_the_unfused_kernels_and_takes_device_precision(d
     assert torch.equal(w2[1:].view(torch.int32), w_ref[1:].view(torch.int32)) and w2[0] == w[0]
 
 
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 1023, 4096, 4097, 1_000_003, 8_388_608 + 6])
+@pytest.mark.parametrize("prec", [0.0371, 1e-30, 0.0])
+def test_compress_axpy_is_compress_then_decompress_axpy(dev, n, prec):
+    """Codes and updated array of the one-pass kernel against the two kernels it replaces and, for the
+    sizes the checker finishes quickly, against the checker.  A precision of 1e-30 or 0 takes the
+    encoder's search instead of its table."""
+    import torch
+    import clusternet_amd as cn
+    rng = np.random.default_rng(n + 3)
+    x = rng.normal(0, 0.01, n).astype(np.float32)
+    if n > 8:
+        x[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-38, -0.0371, 0.0371]
+    y = rng.normal(0, 1, n).astype(np.float32)
+    alpha = -0.0125
+    xd, yd = _t(x, dev), _t(y, dev)
+    want_codes = cn.compression_8bit(xd, prec)
+    want_y = cn.decompression_8bit_axpy(want_codes, prec, alpha, yd.clone())
+    got_y = yd.clone()
+    got_codes = cn.compression_8bit_axpy(xd, prec, alpha, got_y)
+    assert torch.equal(got_codes, want_codes)
+    assert torch.equal(got_y.view(torch.int32), want_y.view(torch.int32))
+    if n <= 1_000_003:
+        host_codes = oracle.compress(x, prec)
+        assert np.array_equal(got_codes.cpu().numpy(), host_codes)
+        assert np.array_equal(_bits(got_y.cpu().numpy()), _bits(oracle.decompress_axpy(host_codes, prec, alpha, y)))
+    # the precision on the device, and views that are not 16-byte aligned
+    if n > 1:
+        p_dev = torch.tensor([prec], dtype=torch.float32, device=dev)
+        y2 = yd.clone()
+        c2 = torch.zeros(n, dtype=torch.uint8, device=dev)
+        cn.compression_8bit_axpy(xd[1:], p_dev, alpha, y2[1:], out=c2[1:])
+        assert torch.equal(c2[1:], want_codes[1:]) and int(c2[0]) == 0
+        assert torch.equal(y2[1:].view(torch.int32), want_y[1:].view(torch.int32))
+        assert _bits(y2[:1].cpu().numpy())[0] == _bits(y[:1])[0]
+
+
+def test_compress_axpy_rejects_null(dev):
+    from clusternet_amd import _lib
+    L = _lib.lib()
+    assert L.cn_compress_8bit_axpy(None, 1.0, 4, None, 1.0, None, None) == 1
+    assert L.cn_compress_8bit_axpy_dp(None, None, 4, None, 1.0, None, None) == 1
+    assert L.cn_compress_8bit_axpy(None, 1.0, 0, None, 1.0, None, None) == 0
+
+
 @pytest.mark.parametrize("n", [0, 1, 5, 4099, 1_000_003])
 def test_rmsprop_update_matches_checker(dev, n):
     import clusternet_amd as cn
