@@ -354,7 +354,7 @@ def main():
         line["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                             "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                             "traffic": TRAFFIC_BYTES_GEMM1,
-                            "kernel": "gemm_kernel<true, 0, 256> (13 K-chunks x 157 tiles of 128x256) followed by "
+                            "kernel": "gemm_kernel<true, 0, 256, 128> (13 K-chunks x 157 tiles of 128x256) followed by "
                                       "splitk_reduce_kernel, 128x40000x100000; both are inside the timed bracket",
                             "avg_ms": g["gemm1_ms"]}
         extra["gemm2_128x20000x40000"] = {"ms": g["gemm2_ms"], "TFLOPs": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12,

@@ -1,16 +1,21 @@
 // fp32 GEMM for gfx950 on the matrix cores: C = op(A) op(B), row-major, alpha 1, beta 0, and the
 // fused variant whose B operand is 8-bit codes.
 //
-// One kernel template, gemm_kernel<A_KC, B_KIND, TN>, 256 lanes = 4 wavefronts, two workgroups per
-// compute unit, in two geometries:
-//   TN = 128  output tile 128 x 128, wavefronts 2 x 2, each 64 x 64 = 2 x 2 blocks of
+// One kernel template, gemm_kernel<A_KC, B_KIND, TN, TM>, 256 lanes = 4 wavefronts, at least two workgroups
+// per compute unit, in three geometries (TM x TN output tiles):
+//   128 x 128 output tile 128 x 128, wavefronts 2 x 2, each 64 x 64 = 2 x 2 blocks of
 //             v_mfma_f32_32x32x2_f32 (64 accumulators per lane); K advances 32 per stage through two
 //             LDS stages (64 KiB)
-//   TN = 256  output tile 128 x 256, wavefronts 1 x 4, each 128 x 64 = 4 x 2 blocks (128 accumulators
+//   128 x 256 output tile 128 x 256, wavefronts 1 x 4, each 128 x 64 = 4 x 2 blocks (128 accumulators
 //             per lane); K advances 16 per stage through two LDS stages (48 KiB).  The A
 //             tile is fetched once per 256 output columns and every B fragment read from LDS feeds four
 //             MFMAs instead of two: less L2 -> LDS and LDS -> register traffic per flop, which matters
 //             because the part runs power-limited on realistic data
+//   32 x 128  for products with no more than 64 rows (a batch of 32 against 8-bit weights): wavefronts
+//             1 x 4, one 32 x 32 block each; K advances 32 per stage through three LDS stages (60 KiB), two of
+//             them in flight.  A 128-row tile would spend
+//             three quarters of its MFMAs on rows that do not exist; with this one such a product costs
+//             its pass over B
 // Common to both:
 //   * one barrier per stage; the global loads of the next stage are issued before the MFMAs of the
 //     current one; the barrier sits eight MFMAs before the end of a stage
@@ -50,7 +55,6 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0xffffffff, 0x00020000);
 }
 
-constexpr int BM = kTileM;
 constexpr int NT = 256;  // lanes per workgroup
 constexpr int NW = 4;    // wavefronts per workgroup
 constexpr int kNumXcd = 8;
@@ -60,10 +64,13 @@ enum BKind { B_IC = 0 /* fp32 [k][n] */, B_KC = 1 /* fp32 [n][k] */, B_CODES = 2
 
 // Geometry of a tile width: wavefront grid WM x WN, FM x FN 32 x 32 blocks per wavefront, K depth
 // of a stage, LDS stages.
-template <int TN> struct Geo;
-template <> struct Geo<128> { static constexpr int WM = 2, WN = 2, FM = 2, FN = 2, BK = 32, NST = 2; };
-template <> struct Geo<256> { static constexpr int WM = 1, WN = 4, FM = 4, FN = 2, BK = 16, NST = 2; };
-static_assert(gemm_tile_k(128) == Geo<128>::BK && gemm_tile_k(256) == Geo<256>::BK, "planner and kernel disagree");
+template <int TM, int TN> struct Geo;
+template <> struct Geo<128, 128> { static constexpr int WM = 2, WN = 2, FM = 2, FN = 2, BK = 32, NST = 2; };
+template <> struct Geo<128, 256> { static constexpr int WM = 1, WN = 4, FM = 4, FN = 2, BK = 16, NST = 2; };
+template <> struct Geo<32, 128> { static constexpr int WM = 1, WN = 4, FM = 1, FN = 1, BK = 32, NST = 3; };
+static_assert(gemm_tile_k(128) == Geo<128, 128>::BK && gemm_tile_k(256) == Geo<128, 256>::BK &&
+                  gemm_tile_k(128) == Geo<kTileMLow, 128>::BK && kTileM == 128 && kTileMLow == 32,
+              "planner and kernel disagree");
 
 struct GemmArgs {
     const float *A;
@@ -261,9 +268,10 @@ struct GuardedIC {
     }
 };
 
-template <bool A_KC, int B_KIND, int TN>
+template <bool A_KC, int B_KIND, int TN, int TM>
 __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
-    using G = Geo<TN>;
+    using G = Geo<TM, TN>;
+    constexpr int BM = TM;
     constexpr bool B_IS_KC = (B_KIND == B_KC);
     constexpr bool kCodes = (B_KIND == B_CODES);
     constexpr int BN = TN, BK = G::BK, NST = G::NST, FM = G::FM, FN = G::FN;
@@ -388,56 +396,59 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi][s], b[ni][s], acc[mi][ni], 0, 0, 0);
     };
     // MFMA steps of the last group that are issued behind the barrier: eight MFMAs.
-    constexpr int kTailFrom = 4 - 8 / (FM * FN);
+    constexpr int kTailFrom = FM * FN >= 2 ? 4 - 8 / (FM * FN) : 0;
 
     // Stages [it0, it_direct) use the direct loads (operands allow 16-byte / 4-byte accesses and the
     // stage lies inside K); the rest, if any, goes through predicated registers.
+    // A ragged tile of codes (columns beyond N) is read byte by byte under conditions: predicated path.
+    const bool whole_n = (n0 + BN <= g.N);
     int it_direct = it0;
-    if (g.vec_a && g.vec_b) {
+    if (g.vec_a && g.vec_b && (!kCodes || whole_n)) {
         const int full = (int)(g.K / BK);
         it_direct = it1 < full ? it1 : full;
         if (it_direct < it0) it_direct = it0;
     }
 
-    if (it0 < it_direct) {
+    auto issue_stage = [&](int it, int slot) {
+        da.issue(corner_a(it), limit_of(g.A, end_a, corner_a(it)), sA + slot * kAStage, wave);
+        if (!kCodes) db.issue(corner_b(it), limit_of(Bf, end_b, corner_b(it)), sB + slot * kBStage, wave);
+    };
+    f32x4 a0[FM], b0[FN], a1[FM], b1[FN];
+    // The MFMAs of one stage up to the last eight.  Fragment reads are left to the compiler's schedule
+    // (just ahead of their MFMAs; the other workgroup on the compute unit covers their latency); the
+    // register sets alternate.  The barrier that publishes the next stage sits eight MFMAs before the
+    // end of a stage so that it is waited for in their shadow.
+    auto stage_head = [&](const float *pa, const float *pb) {
+        if (kGroups == 4) {
+            load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
+            load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, 4);
+            load_frag(pa, pb, 2, a0, b0); mfma_steps(a0, b0, 0, 4);
+            load_frag(pa, pb, 3, a1, b1); mfma_steps(a1, b1, 0, kTailFrom);
+        } else {
+            load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
+            load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, kTailFrom);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (NST == 2 && it0 < it_direct) {
         uint32_t rc[4];
-        const bool whole_n = (n0 + BN <= g.N);
-        static_assert(NST == 2, "the loop below double-buffers");
-        auto issue_stage = [&](int it, int slot) {
-            da.issue(corner_a(it), limit_of(g.A, end_a, corner_a(it)), sA + slot * kAStage, wave);
-            if (!kCodes) db.issue(corner_b(it), limit_of(Bf, end_b, corner_b(it)), sB + slot * kBStage, wave);
-        };
         issue_stage(it0, 0);
         if (kCodes) {
-            gb_ic.load_codes(make_rsrc(corner_c(it0)), BK, whole_n, rc);
+            gb_ic.load_codes(make_rsrc(corner_c(it0)), BK, true, rc);
             gb_ic.store_codes(sB, sLut, rc, BK);
         }
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
         __syncthreads();
-        f32x4 a0[FM], b0[FN], a1[FM], b1[FN];
         int slot = 0;
         for (int it = it0; it < it_direct; ++it) {
             const bool more = (it + 1 < it_direct);
             const int slot_next = slot ^ 1;
-            const float *pa = sA + slot * kAStage, *pb = sB + slot * kBStage;
             if (more) {  // lands in the other stage while this one is consumed
                 issue_stage(it + 1, slot_next);
-                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(it + 1)), BK, whole_n, rc);
+                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(it + 1)), BK, true, rc);
             }
-            // Fragment reads are left to the compiler's schedule (just ahead of their MFMAs; the other
-            // workgroup on the compute unit covers their latency); the register sets alternate.  The
-            // barrier that publishes the next stage sits eight MFMAs before the end of this one so
-            // that it is waited for in their shadow.
-            if (kGroups == 4) {
-                load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
-                load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, 4);
-                load_frag(pa, pb, 2, a0, b0); mfma_steps(a0, b0, 0, 4);
-                load_frag(pa, pb, 3, a1, b1); mfma_steps(a1, b1, 0, kTailFrom);
-            } else {
-                load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);
-                load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, kTailFrom);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+            stage_head(sA + slot * kAStage, sB + slot * kBStage);
             if (kCodes && more) gb_ic.store_codes(sB + slot_next * kBStage, sLut, rc, BK);
             __builtin_amdgcn_s_waitcnt(0x0f70);  // stage it + 1 has landed
             __syncthreads();
@@ -445,6 +456,58 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
             __builtin_amdgcn_sched_barrier(0);
             slot = slot_next;
         }
+    }
+
+    if (NST == 3 && it0 < it_direct) {
+        // Three LDS stages, two in flight: a tile of few rows has little to compute per stage, so what
+        // bounds it is how much of B is on its way.  Codes are held in two register sets, the one of
+        // stage it + 1 being expanded into LDS while the one of stage it + 2 is still arriving.
+        // Every step issues the same kStageLoads load instructions, past the last stage with a range of
+        // zero bytes (such loads return zeros and touch no memory): straight-line code, so that the waits
+        // can count.  "At most kStageLoads outstanding" then means that everything but the newest stage
+        // has arrived.
+        constexpr int kStageLoads = DirectLoader<A_KC, BM, BK>::J + (kCodes ? GuardedIC<TN, BK>::R : DirectLoader<B_IS_KC, TN, BK>::J);
+        static_assert(kStageLoads < 16, "wait-count immediate");
+        auto issue_ahead = [&](int it, int slot, uint32_t (&rc)[4]) {
+            const bool live = it < it_direct;
+            da.issue(corner_a(it), live ? limit_of(g.A, end_a, corner_a(it)) : 0u, sA + slot * kAStage, wave);
+            if (kCodes) {
+                const rsrc_t codes_of_stage = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(corner_c(it)), 0,
+                                                                                live ? 0xffffffff : 0, 0x00020000);
+                gb_ic.load_codes(codes_of_stage, BK, true, rc);
+            } else {
+                db.issue(corner_b(it), live ? limit_of(Bf, end_b, corner_b(it)) : 0u, sB + slot * kBStage, wave);
+            }
+        };
+        uint32_t rc_even[4], rc_odd[4];
+        issue_ahead(it0, 0, rc_even);
+        issue_ahead(it0 + 1, 1, rc_odd);
+        if (kCodes) gb_ic.store_codes(sB, sLut, rc_even, BK);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | kStageLoads);
+        __syncthreads();
+        int slot = 0;
+        // rc_next receives the codes of stage it + 2, rc_ready holds those of stage it + 1
+        auto step = [&](int it, uint32_t (&rc_ready)[4], uint32_t (&rc_next)[4]) {
+            const int slot1 = slot == 2 ? 0 : slot + 1, slot2 = slot1 == 2 ? 0 : slot1 + 1;
+            issue_ahead(it + 2, slot2, rc_next);  // into the stage that was consumed last
+            stage_head(sA + slot * kAStage, sB + slot * kBStage);
+            if (kCodes) gb_ic.store_codes(sB + slot1 * kBStage, sLut, rc_ready, BK);
+            __builtin_amdgcn_s_waitcnt(0x0f70 | kStageLoads);  // stage it + 1 has landed
+            __syncthreads();
+            mfma_steps(a1, b1, kTailFrom, 4);
+            __builtin_amdgcn_sched_barrier(0);
+            slot = slot1;
+        };
+        // whole pairs of steps in the loop, so that the register sets are in the same state every time
+        // round; an odd stage at the end on its own
+        int it = it0;
+        for (int pairs = (it_direct - it0) >> 1; pairs > 0; --pairs, it += 2) {
+            step(it, rc_odd, rc_even);
+            step(it + 1, rc_even, rc_odd);
+        }
+        if ((it_direct - it0) & 1) step(it, rc_odd, rc_even);
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // the zero-range loads behind the last stage
+        __syncthreads();
     }
 
     if (it_direct < it1) {
@@ -554,7 +617,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
             const int64_t m = i / nq, q = i % nq;
             const float *src = partial + m * N + 4 * q;
             f32x4 s = *reinterpret_cast<const f32x4 *>(src);
-            for (int c = 1; c < splits; ++c) s += *reinterpret_cast<const f32x4 *>(src + c * plane);
+            int c = 1;
+            // eight planes requested before the first is added: the order of the additions stays, the
+            // memory latencies overlap
+            for (; c + 8 <= splits; c += 8) {
+                f32x4 t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) t[u] = *reinterpret_cast<const f32x4 *>(src + (c + u) * plane);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s += t[u];
+            }
+            for (; c < splits; ++c) s += *reinterpret_cast<const f32x4 *>(src + c * plane);
             *reinterpret_cast<f32x4 *>(C + m * ldc + 4 * q) = s;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -603,24 +676,27 @@ cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float
     return CN_OK;
 }
 
-template <bool A_KC, int B_KIND, int TN>
+template <bool A_KC, int B_KIND, int TN, int TM>
 static cn_status launch_tile(const GemmArgs &args, hipStream_t st) {
-    using G = Geo<TN>;
-    const size_t lds = (size_t)(G::NST * (BM + TN) * G::BK + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
+    using G = Geo<TM, TN>;
+    // the stages, the decode table of the fused variant, and at least the four write-out patches
+    size_t lds = (size_t)(G::NST * (TM + TN) * G::BK + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
+    if (lds < NW * 32 * 36 * sizeof(float)) lds = NW * 32 * 36 * sizeof(float);
     static bool configured = false;
     if (!configured) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN>),
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN, TM>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         configured = true;
     }
-    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN>), dim3(args.units), dim3(NT), lds, st, args);
+    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN, TM>), dim3(args.units), dim3(NT), lds, st, args);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
 
 template <bool A_KC, int B_KIND>
-static cn_status launch(const GemmArgs &args, int tile_n, hipStream_t st) {
-    return tile_n == 256 ? launch_tile<A_KC, B_KIND, 256>(args, st) : launch_tile<A_KC, B_KIND, 128>(args, st);
+static cn_status launch(const GemmArgs &args, const GemmPlan &plan, hipStream_t st) {
+    if (plan.tile_m == kTileMLow) return launch_tile<A_KC, B_KIND, 128, kTileMLow>(args, st);
+    return plan.tile_n == 256 ? launch_tile<A_KC, B_KIND, 256, kTileM>(args, st) : launch_tile<A_KC, B_KIND, 128, kTileM>(args, st);
 }
 
 static int g_force_tile_n = 0;
@@ -681,11 +757,11 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.wide_store = g_wide_store && (plan.splits > 1 ? (N % 4 == 0 && (M * N) % 4 == 0)
                                                      : (aligned(C, 16) && ldc % 4 == 0));
 
-    if (w8)              s = launch<true, B_CODES>(a, plan.tile_n, st);
-    else if (!ta && !tb) s = launch<true, B_IC>(a, plan.tile_n, st);
-    else if (ta && !tb)  s = launch<false, B_IC>(a, plan.tile_n, st);
-    else if (!ta && tb)  s = launch<true, B_KC>(a, plan.tile_n, st);
-    else                 s = launch<false, B_KC>(a, plan.tile_n, st);
+    if (w8)              s = launch<true, B_CODES>(a, plan, st);
+    else if (!ta && !tb) s = launch<true, B_IC>(a, plan, st);
+    else if (ta && !tb)  s = launch<false, B_IC>(a, plan, st);
+    else if (!ta && tb)  s = launch<true, B_KC>(a, plan, st);
+    else                 s = launch<false, B_KC>(a, plan, st);
     if (s != CN_OK) return s;
 
     if (plan.splits > 1) return add_chunk_planes(ctx, plan.splits, M, N, C, ldc, amax, st);
@@ -701,8 +777,9 @@ extern "C" {
 // Test hook: 0 = write every tile with 4-byte stores.
 void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
 
-// Test and tuning hook: 0 = let the planner choose the tile width, 128 / 256 = force it.
-void cn_host_force_gemm_tile_n(int tile_n) { g_force_tile_n = (tile_n == 128 || tile_n == 256) ? tile_n : 0; }
+// Test and tuning hook: 0 = let the planner choose the tile, 128 / 256 = force that width of the 128-row
+// tile, 32 = force the 32 x 128 tile.
+void cn_host_force_gemm_tile_n(int tile_n) { g_force_tile_n = (tile_n == 128 || tile_n == 256 || tile_n == kTileMLow) ? tile_n : 0; }
 
 cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                       const float *B, int64_t ldb, float *C, int64_t ldc, void *stream) {

@@ -1,7 +1,9 @@
 // Host-side work decomposition for the fp32 GEMM kernels (pure function, no HIP calls).
 //
 // The output is cut into tiles of 128 rows and 128 or 256 columns, two workgroups per compute unit
-// either way.  The batches this library serves are skinny (M = 128), so tiles alone cannot fill 256
+// either way, or, when it has no more than 64 rows, into tiles of 32 rows and 128 columns: a 128-row tile
+// would spend most of its matrix-core work on rows that do not exist, while a 32-row tile leaves such a
+// product to what it is bound by, the one pass over B.  The batches this library serves are skinny (M = 128), so tiles alone cannot fill 256
 // compute units; K is therefore cut into `splits` chunks, every (chunk, tile) pair becomes one
 // workgroup, and a second kernel adds the chunk results in a fixed order (deterministic, no
 // atomics).  Chunks are ordered chunk-major so that workgroups running at the same time walk the
@@ -61,6 +63,7 @@ int64_t split_limit(int64_t k_iters, int min_iters, double out_bytes, size_t wor
 
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n) {
     GemmPlan p;
+    p.tile_m = kTileM;
     p.tiles_m = (M + kTileM - 1) / kTileM;
     const int64_t cus = num_cu > 0 ? num_cu : 1;
     const double out_bytes = (double)M * (double)N * 4.0;
@@ -68,6 +71,21 @@ GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace
     int64_t it128 = (K + gemm_tile_k(128) - 1) / gemm_tile_k(128), it256 = (K + gemm_tile_k(256) - 1) / gemm_tile_k(256);
     if (it128 < 1) it128 = 1;
     if (it256 < 1) it256 = 1;
+
+    if (force_tile_n == kTileMLow || (force_tile_n == 0 && M <= kLowTileMaxRows)) {
+        // A stage of the 32 x 128 tile moves 20 KB for a quarter of the unit's flops: it costs what its
+        // loads cost, about a third of the unit.
+        p.tile_m = kTileMLow;
+        p.tiles_m = (M + kTileMLow - 1) / kTileMLow;
+        const Choice c = best_split(p.tiles_m * tiles_n128, it128, cus, 0.35, split_limit(it128, 4, out_bytes, workspace_bytes), out_bytes);
+        p.tile_n = 128;
+        p.tiles_n = tiles_n128;
+        p.k_iters = it128;
+        p.splits = c.splits;
+        p.iters_per_split = c.ips;
+        p.units = p.tiles_m * p.tiles_n * p.splits;
+        return p;
+    }
 
     // a chunk is at least 128 k deep
     Choice narrow = best_split(p.tiles_m * tiles_n128, it128, cus, 1.0, split_limit(it128, 4, out_bytes, workspace_bytes), out_bytes);
@@ -92,7 +110,7 @@ GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace
 }  // namespace cn
 
 extern "C" void cn_host_plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes,
-                                  int force_tile_n, int64_t out[7]) {
+                                  int force_tile_n, int64_t out[8]) {
     cn::GemmPlan p = cn::plan_gemm(M, N, K, num_cu, workspace_bytes, force_tile_n);
     out[0] = p.tiles_m;
     out[1] = p.tiles_n;
@@ -101,4 +119,5 @@ extern "C" void cn_host_plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, s
     out[4] = p.iters_per_split;
     out[5] = p.units;
     out[6] = p.tile_n;
+    out[7] = p.tile_m;
 }

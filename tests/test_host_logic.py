@@ -132,19 +132,21 @@ def test_encoder_table_shape():
 
 def test_gemm_plan_covers_k_and_fits_workspace():
     L = cn.lib()
-    out = (C.c_int64 * 7)()
+    out = (C.c_int64 * 8)()
     rng = np.random.default_rng(0)
     shapes = [(128, 40000, 100000), (128, 20000, 40000), (128, 1024, 784), (784, 1024, 128),
               (128, 784, 1024), (100000, 8192, 128), (128, 4096, 4096), (2, 2, 3), (1, 1, 1),
               (128, 10, 4096), (5000, 5000, 31)]
     shapes += [tuple(int(v) for v in rng.integers(1, 3000, 3)) for _ in range(200)]
     for ws in (16 << 20, 1 << 30):
-        for force in (0, 128, 256):
+        for force in (0, 128, 256, 32):
             for (M, N, K) in shapes:
                 L.cn_host_plan_gemm(M, N, K, 256, ws, force, out)
-                tm, tn, kit, splits, ips, units, tile_n = list(out)
-                assert tile_n in (128, 256) and (force == 0 or tile_n == force)
-                assert tm == -(-M // 128) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
+                tm, tn, kit, splits, ips, units, tile_n, tile_m = list(out)
+                # the 32-row tile when asked for, and unasked for products of at most 64 rows
+                assert tile_m == (32 if force == 32 or (force == 0 and M <= 64) else 128)
+                assert tile_n in (128, 256) and (force in (0, 32) or tile_n == force) and (tile_m == 128 or tile_n == 128)
+                assert tm == -(-M // tile_m) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
                 assert splits >= 1 and units == tm * tn * splits
                 assert ips * splits >= kit and ips * (splits - 1) < kit  # every chunk non-empty
                 if splits > 1:
