@@ -255,10 +255,11 @@ struct GuardedIC {
     // Expand through the decode table.  Rows at or beyond K must contribute exactly zero whatever
     // code 0 decodes to; columns beyond N only reach outputs that are not stored.
     __device__ __forceinline__ void store_codes(float *__restrict__ lds, const float *__restrict__ lut,
-                                                const uint32_t (&reg)[4], int64_t kleft) const {
+                                                const uint32_t (&reg)[4], int64_t kleft, int r_begin = 0,
+                                                int r_end = R) const {
         const int cq = threadIdx.x % CQ, kr = threadIdx.x / CQ;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
+        for (int r = r_begin; r < r_end; ++r) {
             f32x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = lut[(reg[r] >> (8 * e)) & 0xffu];
@@ -431,31 +432,89 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
         __builtin_amdgcn_sched_barrier(0);
     };
 
-    if (NST == 2 && it0 < it_direct) {
-        uint32_t rc[4];
-        issue_stage(it0, 0);
-        if (kCodes) {
-            gb_ic.load_codes(make_rsrc(corner_c(it0)), BK, true, rc);
-            gb_ic.store_codes(sB, sLut, rc, BK);
+    // The same with a set of codes expanded into the LDS stage `pn` in four parts between the MFMA groups,
+    // where the table look-ups and LDS stores cost nothing: the matrix pipe is busy anyway.
+    auto stage_head_expanding = [&](const float *pa, const float *pb, float *pn, const uint32_t (&rc)[4]) {
+        static_assert(!kCodes || GuardedIC<TN, BK>::R == 4, "four parts");
+        if (kGroups == 4) {
+            load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);         gb_ic.store_codes(pn, sLut, rc, BK, 0, 1);
+            load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, 4);         gb_ic.store_codes(pn, sLut, rc, BK, 1, 2);
+            load_frag(pa, pb, 2, a0, b0); mfma_steps(a0, b0, 0, 4);         gb_ic.store_codes(pn, sLut, rc, BK, 2, 3);
+            load_frag(pa, pb, 3, a1, b1); mfma_steps(a1, b1, 0, kTailFrom); gb_ic.store_codes(pn, sLut, rc, BK, 3, 4);
+        } else {
+            load_frag(pa, pb, 0, a0, b0); mfma_steps(a0, b0, 0, 4);         gb_ic.store_codes(pn, sLut, rc, BK, 0, 2);
+            load_frag(pa, pb, 1, a1, b1); mfma_steps(a1, b1, 0, kTailFrom); gb_ic.store_codes(pn, sLut, rc, BK, 2, 4);
         }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    if (NST == 2 && !kCodes && it0 < it_direct) {
+        issue_stage(it0, 0);
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stage has landed in LDS
         __syncthreads();
         int slot = 0;
         for (int it = it0; it < it_direct; ++it) {
-            const bool more = (it + 1 < it_direct);
             const int slot_next = slot ^ 1;
-            if (more) {  // lands in the other stage while this one is consumed
-                issue_stage(it + 1, slot_next);
-                if (kCodes) gb_ic.load_codes(make_rsrc(corner_c(it + 1)), BK, true, rc);
-            }
+            if (it + 1 < it_direct) issue_stage(it + 1, slot_next);  // lands in the other stage while this one is consumed
             stage_head(sA + slot * kAStage, sB + slot * kBStage);
-            if (kCodes && more) gb_ic.store_codes(sB + slot_next * kBStage, sLut, rc, BK);
             __builtin_amdgcn_s_waitcnt(0x0f70);  // stage it + 1 has landed
             __syncthreads();
             mfma_steps(a1, b1, kTailFrom, 4);
             __builtin_amdgcn_sched_barrier(0);
             slot = slot_next;
         }
+    }
+
+    if (NST == 2 && kCodes && it0 < it_direct) {
+        // Codes are requested two stages ahead into two register sets that alternate, and the set of stage
+        // it + 1 is expanded into the other LDS stage between the MFMA groups of stage it.  The A tile of stage
+        // it + 1 is requested right behind the barrier that frees its LDS stage.  Code loads past the last
+        // stage get a range of zero bytes instead of being skipped (straight-line code, see the three-stage
+        // loop below); what they "decode" lands in a stage that is not read again.
+        constexpr int kCodeLoads = GuardedIC<TN, BK>::R;
+        auto codes_ahead = [&](int it, uint32_t (&rc)[4]) {
+            // the descriptor is the same for every lane: say so, or each load is wrapped in a loop over lanes
+            const uint64_t corner = reinterpret_cast<uint64_t>(corner_c(it));
+            const uint64_t uniform = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(corner >> 32)) << 32) |
+                                     (uint32_t)__builtin_amdgcn_readfirstlane((int)corner);
+            const int range = __builtin_amdgcn_readfirstlane(it < it_direct ? -1 : 0);
+            const rsrc_t codes_of_stage = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<uint8_t *>(uniform), 0, range, 0x00020000);
+            gb_ic.load_codes(codes_of_stage, BK, true, rc);
+        };
+        auto issue_a = [&](int it, int slot) {
+            da.issue(corner_a(it), limit_of(g.A, end_a, corner_a(it)), sA + slot * kAStage, wave);
+        };
+        uint32_t rc_even[4], rc_odd[4];
+        codes_ahead(it0, rc_even);
+        codes_ahead(it0 + 1, rc_odd);
+        issue_a(it0, 0);
+        gb_ic.store_codes(sB, sLut, rc_even, BK);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (it0 + 1 < it_direct) issue_a(it0 + 1, 1);
+        int slot = 0;
+        // rc_ready holds the codes of stage it + 1, rc_next receives those of stage it + 2
+        auto step = [&](int it, uint32_t (&rc_ready)[4], uint32_t (&rc_next)[4]) {
+            const int slot_next = slot ^ 1;
+            const float *pa = sA + slot * kAStage, *pb = sB + slot * kBStage;
+            float *pn = sB + slot_next * kBStage;
+            codes_ahead(it + 2, rc_next);
+            stage_head_expanding(pa, pb, pn, rc_ready);
+            // the A tile of stage it + 1 has landed: only the code loads of stage it + 2 are younger
+            __builtin_amdgcn_s_waitcnt(0x0f70 | kCodeLoads);
+            __syncthreads();
+            if (it + 2 < it_direct) issue_a(it + 2, slot);  // every wavefront is done reading this stage
+            mfma_steps(a1, b1, kTailFrom, 4);
+            __builtin_amdgcn_sched_barrier(0);
+            slot = slot_next;
+        };
+        int it = it0;
+        for (int pairs = (it_direct - it0) >> 1; pairs > 0; --pairs, it += 2) {
+            step(it, rc_odd, rc_even);
+            step(it + 1, rc_even, rc_odd);
+        }
+        if ((it_direct - it0) & 1) step(it, rc_odd, rc_even);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
     }
 
     if (NST == 3 && it0 < it_direct) {
@@ -490,8 +549,8 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
         auto step = [&](int it, uint32_t (&rc_ready)[4], uint32_t (&rc_next)[4]) {
             const int slot1 = slot == 2 ? 0 : slot + 1, slot2 = slot1 == 2 ? 0 : slot1 + 1;
             issue_ahead(it + 2, slot2, rc_next);  // into the stage that was consumed last
-            stage_head(sA + slot * kAStage, sB + slot * kBStage);
-            if (kCodes) gb_ic.store_codes(sB + slot1 * kBStage, sLut, rc_ready, BK);
+            if (kCodes) stage_head_expanding(sA + slot * kAStage, sB + slot * kBStage, sB + slot1 * kBStage, rc_ready);
+            else        stage_head(sA + slot * kAStage, sB + slot * kBStage);
             __builtin_amdgcn_s_waitcnt(0x0f70 | kStageLoads);  // stage it + 1 has landed
             __syncthreads();
             mfma_steps(a1, b1, kTailFrom, 4);
