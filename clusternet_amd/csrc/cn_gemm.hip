@@ -736,16 +736,15 @@ cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float
 }
 
 template <bool A_KC, int B_KIND, int TN, int TM>
-static cn_status launch_tile(const GemmArgs &args, hipStream_t st) {
+static cn_status launch_tile(const GemmArgs &args, int device, hipStream_t st) {
     using G = Geo<TM, TN>;
     // the stages, the decode table of the fused variant, and at least the four write-out patches
     size_t lds = (size_t)(G::NST * (TM + TN) * G::BK + (B_KIND == B_CODES ? 256 : 0)) * sizeof(float);
     if (lds < NW * 32 * 36 * sizeof(float)) lds = NW * 32 * 36 * sizeof(float);
-    static bool configured = false;
-    if (!configured) {
+    static OncePerDevice configured;
+    if (configured.first(device)) {
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN, TM>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        configured = true;
     }
     hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN, TM>), dim3(args.units), dim3(NT), lds, st, args);
     CN_HIP(hipGetLastError());
@@ -753,9 +752,10 @@ static cn_status launch_tile(const GemmArgs &args, hipStream_t st) {
 }
 
 template <bool A_KC, int B_KIND>
-static cn_status launch(const GemmArgs &args, const GemmPlan &plan, hipStream_t st) {
-    if (plan.tile_m == kTileMLow) return launch_tile<A_KC, B_KIND, 128, kTileMLow>(args, st);
-    return plan.tile_n == 256 ? launch_tile<A_KC, B_KIND, 256, kTileM>(args, st) : launch_tile<A_KC, B_KIND, 128, kTileM>(args, st);
+static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, hipStream_t st) {
+    if (plan.tile_m == kTileMLow) return launch_tile<A_KC, B_KIND, 128, kTileMLow>(args, device, st);
+    return plan.tile_n == 256 ? launch_tile<A_KC, B_KIND, 256, kTileM>(args, device, st)
+                              : launch_tile<A_KC, B_KIND, 128, kTileM>(args, device, st);
 }
 
 static int g_force_tile_n = 0;
@@ -816,11 +816,11 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.wide_store = g_wide_store && (plan.splits > 1 ? (N % 4 == 0 && (M * N) % 4 == 0)
                                                      : (aligned(C, 16) && ldc % 4 == 0));
 
-    if (w8)              s = launch<true, B_CODES>(a, plan, st);
-    else if (!ta && !tb) s = launch<true, B_IC>(a, plan, st);
-    else if (ta && !tb)  s = launch<false, B_IC>(a, plan, st);
-    else if (!ta && tb)  s = launch<true, B_KC>(a, plan, st);
-    else                 s = launch<false, B_KC>(a, plan, st);
+    if (w8)              s = launch<true, B_CODES>(a, plan, ctx->device, st);
+    else if (!ta && !tb) s = launch<true, B_IC>(a, plan, ctx->device, st);
+    else if (ta && !tb)  s = launch<false, B_IC>(a, plan, ctx->device, st);
+    else if (!ta && tb)  s = launch<true, B_KC>(a, plan, ctx->device, st);
+    else                 s = launch<false, B_KC>(a, plan, ctx->device, st);
     if (s != CN_OK) return s;
 
     if (plan.splits > 1) return add_chunk_planes(ctx, plan.splits, M, N, C, ldc, amax, st);

@@ -38,6 +38,17 @@ struct Context {
 constexpr int kMaxDevices = 16;
 constexpr int kReduceSlots = 4096;
 
+// A kernel's attributes (its dynamic LDS limit) are set per device: one flag per device for a call site.
+struct OncePerDevice {
+    bool done[kMaxDevices] = {};
+    bool first(int device) {
+        if (device < 0 || device >= kMaxDevices) return true;
+        const bool was = done[device];
+        done[device] = true;
+        return !was;
+    }
+};
+
 // Returns the context of the current device, initialising it on first use.
 cn_status current_context(Context **out);
 

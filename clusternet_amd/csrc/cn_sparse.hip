@@ -953,11 +953,10 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
     if (!out && !amax) { set_error("%s: NULL output", who); return CN_ERR_NULL; }
     if (!out && g_lds_rows && Cc > 0 && Cc <= kLdsMaxRows) {  // maximum only, B strip in LDS
         const int lds_rows = (int)(Cc * kLdsStrip * sizeof(float));
-        static bool lds_configured = false;
-        if (!lds_configured) {
+        static OncePerDevice lds_configured;
+        if (lds_configured.first(ctx->device)) {
             CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_max_lds_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMaxRows * kLdsStrip * (int)sizeof(float)));
-            lds_configured = true;
         }
         const int64_t strips = (N + kLdsStrip - 1) / kLdsStrip;
         if (strips > 0x7fffffLL) { set_error("%s: too many columns", who); return CN_ERR_SHAPE; }
@@ -1076,8 +1075,8 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
     const int lds = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
-    static bool configured = false;
-    if (!configured) {
+    static OncePerDevice configured;
+    if (configured.first(ctx->device)) {
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_gemm_coded_kernel),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<2>),
@@ -1086,7 +1085,6 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<4>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-        configured = true;
     }
     const bool vec = Cc > 0 && Cc * ldb < (1LL << 30) && aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0 && aligned(codes, 4) &&
                      (!w || (aligned(w, 16) && ldw % 4 == 0)) && (!rms || aligned(rms, 16));
