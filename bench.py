@@ -127,14 +127,14 @@ def bench_codec(torch, cn, dev):
             "decompress_frac_hbm_peak": 5.0 * n / t_d / 1e6 / PEAK_HBM_GBPS,
         }
         if n % 4096 == 0 and n >= 100000 * 8192:
-            # the same bytes moved by kernels that do no arithmetic: best of four grid sizes each
+            # the same bytes moved by kernels that do no arithmetic: best of six grid sizes each
             from clusternet_amd import _lib as L
             sink = torch.empty(256 * 64 * L.num_compute_units(), dtype=torch.int32, device=dev)
             yard = {}
             for label, kind, src, dst, nbytes in (("read_4B", 0, x, sink, 4.0), ("fp32_to_byte_4B_1B", 1, x, codes, 5.0),
                                                   ("byte_to_fp32_1B_4B", 2, codes, back, 5.0), ("copy_4B_4B", 3, x, back, 8.0)):
                 best = min(time_region(torch, lambda: L.stream_yardstick(kind, src, dst, n, per_cu), 10, 2)
-                           for per_cu in (2, 4, 8, 16))
+                           for per_cu in (2, 3, 4, 6, 8, 16))
                 yard[label + "_GBps"] = nbytes * n / best / 1e6
             res[name]["arithmetic_free_streams"] = yard
             res[name]["compress_frac_of_stream"] = res[name]["compress_GBps"] / yard["fp32_to_byte_4B_1B_GBps"]
