@@ -699,7 +699,15 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
              i += (int64_t)gridDim.x * blockDim.x) {
             const int64_t m = i / N, n = i % N;
             float s = partial[i];
-            for (int c = 1; c < splits; ++c) s += partial[i + c * plane];
+            int c = 1;
+            for (; c + 8 <= splits; c += 8) {
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) t[u] = partial[i + (c + u) * plane];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s += t[u];
+            }
+            for (; c < splits; ++c) s += partial[i + c * plane];
             C[m * ldc + n] = s;
             const uint32_t bits = __float_as_uint(s) & 0x7fffffffu;
             amax = bits > amax ? bits : amax;
