@@ -225,9 +225,8 @@ __device__ __forceinline__ float max_unkey(uint32_t key) {
 template <bool kVector, bool kAbs>
 __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restrict__ x, size_t n,
                                                           float *__restrict__ out,
-                                                          uint32_t *__restrict__ scratch) {
+                                                          uint32_t *__restrict__ tickets) {
     __shared__ uint32_t smem[kThreads / 64];
-    __shared__ uint32_t s_last;
     const uint32_t start = kAbs ? 0u : max_key<false>(0xbf800000u);
     uint32_t m = start;
     if (kVector) {
@@ -261,25 +260,24 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
             m = max(m, max_key<kAbs>(__float_as_uint(x[i])));
     }
     m = block_max(m, smem);
-    // Publish the workgroup's maximum, then let the last workgroup to arrive fold all of them.
-    // scratch[0..gridDim.x) = partial maxima, scratch[kReduceSlots] = arrival counter (left at 0).
+    // The workgroup folds its maximum into one word and then counts itself in on another; the last to arrive
+    // reads the maximum, writes the result and puts both words back to 0.  Both are device-scope atomics that
+    // return a value, and the count is made to depend on what the fold returned, so the fold has been performed
+    // before the count is issued: ordering by data dependence instead of by fences, which cost far more here
+    // (a release fence per workgroup writes the L2 back; nothing in this kernel needs that).
     if (threadIdx.x == 0) {
-        __hip_atomic_store(&scratch[blockIdx.x], m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __threadfence();
-        uint32_t ticket = atomicAdd(&scratch[kReduceSlots], 1u);
-        s_last = (ticket == gridDim.x - 1) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (s_last) {
-        __threadfence();
-        uint32_t r = start;
-        for (uint32_t i = threadIdx.x; i < gridDim.x; i += blockDim.x)
-            r = max(r, __hip_atomic_load(&scratch[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        __syncthreads();
-        r = block_max(r, smem);
-        if (threadIdx.x == 0) {
-            out[0] = max_unkey<kAbs>(r);
-            __hip_atomic_store(&scratch[kReduceSlots], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t *running = tickets, *arrived = tickets + kTicketStride;
+        const uint32_t before = atomicMax(running, m);
+        uint32_t one = 1u;
+        asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
+        uint32_t ticket = atomicAdd(arrived, one);
+        if (ticket == gridDim.x - 1) {
+            uint32_t *from = running;
+            asm volatile("" : "+v"(from) : "v"(ticket));
+            const uint32_t of_all = __hip_atomic_load(from, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            out[0] = max_unkey<kAbs>(of_all);
+            __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
@@ -296,20 +294,6 @@ __global__ __launch_bounds__(kThreads) void fill_kernel(float *__restrict__ dst,
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 static int g_workgroups_per_cu = 0;  // tuning hook: nonzero overrides every kernel's own figure
-
-// Grid of the reductions (abs-max, max).  Every workgroup ends with a fence and two atomics on words that all
-// workgroups share, and those cost about 19 ns per workgroup, one after the other: 512 workgroups add 10 us
-// to a kernel that reads a 20 MB buffer in 5.  So a small input gets one workgroup per five tiles (at least
-// 64), a large one two per CU.
-static int reduce_grid(const Context *ctx, size_t n) {
-    const size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
-    size_t g = tiles / 5;
-    if (g < 64) g = tiles < 64 ? (tiles < 1 ? 1 : tiles) : 64;
-    const size_t cap = g_workgroups_per_cu > 0 ? (size_t)ctx->num_cu * g_workgroups_per_cu : (size_t)ctx->num_cu * 2;
-    if (g > cap) g = cap;
-    if (g > (size_t)kReduceSlots) g = kReduceSlots;
-    return (int)g;
-}
 
 static int stream_grid(const Context *ctx, size_t n, int per_cu) {
     size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
@@ -428,11 +412,11 @@ cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
         return CN_OK;
     }
     if (!x) { set_error("absmax_f32: NULL input"); return CN_ERR_NULL; }
-    int grid = reduce_grid(ctx, n);
+    int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16))
-        hipLaunchKernelGGL((absmax_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+        hipLaunchKernelGGL((absmax_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
     else
-        hipLaunchKernelGGL((absmax_kernel<false, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+        hipLaunchKernelGGL((absmax_kernel<false, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -449,11 +433,11 @@ cn_status cn_max_f32(const float *x, size_t n, float *out, void *stream) {
         return CN_OK;
     }
     if (!x) { set_error("max_f32: NULL input"); return CN_ERR_NULL; }
-    int grid = reduce_grid(ctx, n);
+    int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16))
-        hipLaunchKernelGGL((absmax_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+        hipLaunchKernelGGL((absmax_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
     else
-        hipLaunchKernelGGL((absmax_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->reduce_scratch);
+        hipLaunchKernelGGL((absmax_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

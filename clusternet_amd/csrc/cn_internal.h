@@ -32,11 +32,15 @@ struct Context {
     int xstep_count = 0;
     void *workspace = nullptr;       // split-K partial sums
     size_t workspace_bytes = 0;
-    uint32_t *reduce_scratch = nullptr;  // per-workgroup partial maxima + ticket counters
+    uint32_t *reduce_scratch = nullptr;  // per-workgroup partial results + ticket counters
+    uint32_t *tickets = nullptr;         // running maximum and arrival count of the max reductions (kTicketWords words)
     double *sum_scratch = nullptr;       // per-workgroup partial sums (1024 doubles)
 };
 constexpr int kMaxDevices = 16;
 constexpr int kReduceSlots = 4096;
+// Max reductions: the running maximum and the arrival count, each on a 128-byte line of its own, both left at 0.
+constexpr int kTicketStride = 32;
+constexpr int kTicketWords = 2 * kTicketStride;
 
 // A kernel's attributes (its dynamic LDS limit) are set per device: one flag per device for a call site.
 struct OncePerDevice {

@@ -81,6 +81,8 @@ static cn_status init_device(int device) {
 
     CN_HIP(hipMalloc((void **)&c.reduce_scratch, (kReduceSlots + 64) * sizeof(uint32_t)));
     CN_HIP(hipMemset(c.reduce_scratch, 0, (kReduceSlots + 64) * sizeof(uint32_t)));
+    CN_HIP(hipMalloc((void **)&c.tickets, kTicketWords * sizeof(uint32_t)));
+    CN_HIP(hipMemset(c.tickets, 0, kTicketWords * sizeof(uint32_t)));
     CN_HIP(hipMalloc((void **)&c.sum_scratch, 1024 * sizeof(double)));
     CN_HIP(hipDeviceSynchronize());
     CN_HIP(hipSetDevice(previous));
@@ -147,6 +149,7 @@ cn_status cn_shutdown(void) {
         CN_HIP(hipFree(c.xsteps));
         CN_HIP(hipFree(c.workspace));
         CN_HIP(hipFree(c.reduce_scratch));
+        CN_HIP(hipFree(c.tickets));
         CN_HIP(hipFree(c.sum_scratch));
         c = Context();
     }

@@ -7,6 +7,11 @@
  * Every function returns a cn_status; 0 is success.  The library never falls back to the CPU:
  * without a usable GPU, cn_init and every compute entry point return CN_ERR_NO_DEVICE.
  *
+ * One stream at a time per device, as in the reference (one host thread, the default stream,
+ * source/clusterNet.cpp:406-407): the products that split K, the reductions and the sparse conversions
+ * keep partial results in per-device scratch memory owned by the library, so calls that may run at the
+ * same time on one device (different streams without an ordering between them) race on it.
+ *
  * Storage convention: matrices are ROW-major with an explicit leading dimension (elements per
  * row).  The reference keeps device matrices column-major (source/basicOps.cu:14-33) and calls
  * cublasSgemm with lda = rows (source/clusterNet.cpp:459-461); a column-major M x K matrix is the
