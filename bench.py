@@ -65,6 +65,32 @@ def time_region(torch, fn, iters, warmup):
     return s.elapsed_time(e) / iters  # ms
 
 
+def time_replayed(torch, fn, calls, replays):
+    """ms per call with the host out of the way: `calls` calls captured into one HIP graph, the graph
+    replayed `replays` times between two events.  For kernels of a few microseconds, where the loop of
+    time_region measures how fast Python can launch.  None if the capture is refused."""
+    try:
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(calls):
+                fn()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        s, e = event_pair(torch)
+        s.record()
+        for _ in range(replays):
+            graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / (calls * replays)
+    except Exception:  # noqa: BLE001 - any refusal means "not measured this way"
+        torch.cuda.synchronize()
+        return None
+
+
 def bench_gemm(torch, cn, dev, steps, warmup):
     gen = torch.Generator(device=dev).manual_seed(1234)
     batch = torch.rand((M, K1), device=dev, generator=gen)
@@ -113,10 +139,11 @@ def bench_codec(torch, cn, dev):
         prec = float(prec_t.cpu()[0])
         codes = torch.empty(n, dtype=torch.uint8, device=dev)
         back = torch.empty(n, device=dev)
-        t_abs = time_region(torch, lambda: cn.absmax(x, prec_t), iters, 3)
-        t_c = time_region(torch, lambda: cn.compression_8bit(x, prec, codes), iters, 3)
-        t_d = time_region(torch, lambda: cn.decompression_8bit(codes, prec, back), iters, 3)
-        t_copy = time_region(torch, lambda: back.copy_(x), iters, 3)
+        warm = 3 if n >= 100000 * 8192 else 1000  # microsecond kernels: let the clocks come up first
+        t_abs = time_region(torch, lambda: cn.absmax(x, prec_t), iters, warm)
+        t_c = time_region(torch, lambda: cn.compression_8bit(x, prec, codes), iters, warm)
+        t_d = time_region(torch, lambda: cn.decompression_8bit(codes, prec, back), iters, warm)
+        t_copy = time_region(torch, lambda: back.copy_(x), iters, warm)
         res[name] = {
             "elements": n,
             "absmax_GBps": 4.0 * n / t_abs / 1e6, "absmax_us": t_abs * 1e3,
@@ -126,6 +153,12 @@ def bench_codec(torch, cn, dev):
             "compress_frac_hbm_peak": 5.0 * n / t_c / 1e6 / PEAK_HBM_GBPS,
             "decompress_frac_hbm_peak": 5.0 * n / t_d / 1e6 / PEAK_HBM_GBPS,
         }
+        if n < 100000 * 8192:
+            # small buffers: the kernels take a few microseconds, so also time them replayed from a graph
+            replayed = {"absmax_us": time_replayed(torch, lambda: cn.absmax(x, prec_t), 20, 50),
+                        "compress_us": time_replayed(torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50),
+                        "decompress_us": time_replayed(torch, lambda: cn.decompression_8bit(codes, prec_t, back), 20, 50)}
+            res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
         if n % 4096 == 0 and n >= 100000 * 8192:
             # the same bytes moved by kernels that do no arithmetic: best of six grid sizes each
             from clusternet_amd import _lib as L
