@@ -28,6 +28,30 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
     float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // kUpdate: decode table times alpha
     const float precision = precision_ptr ? *precision_ptr : precision_value;
+
+    // The workgroup's first tile is requested before the table is built, so that its memory latency runs
+    // beside those of the table's inputs: a small input is one or two tiles per workgroup.
+    const size_t nvec = n / 4;
+    const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
+    f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
+    const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
+    auto load_tile = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kVecPerThread]) {
+        const size_t base = tile * kTileVec + threadIdx.x;
+#pragma unroll
+        for (int j = 0; j < kVecPerThread; ++j) {
+            size_t i = base + (size_t)j * kThreads;
+            v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
+            if (kUpdate) w[j] = (i < nvec) ? __builtin_nontemporal_load(&y4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    // Two register sets: the loads of the next tile are in flight while this one is encoded,
+    // so the memory pipe stays busy even with only a few wavefronts per SIMD.
+    f32x4 va[kVecPerThread], vb[kVecPerThread], wa[kUpdate ? kVecPerThread : 1], wb[kUpdate ? kVecPerThread : 1];
+    auto load = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kUpdate ? kVecPerThread : 1]) {
+        load_tile(tile, v, reinterpret_cast<f32x4 (&)[kVecPerThread]>(w));
+    };
+    if (kVector && blockIdx.x < tiles) load(blockIdx.x, va, wa);
+
     const bool exact_only = !build_table(sh, steps, step_count, precision, table);
     if (kUpdate) {
         const int t = threadIdx.x;
@@ -50,20 +74,7 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
     };
 
     if (kVector) {
-        const size_t nvec = n / 4;
-        const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x);
         uint32_t *c4 = reinterpret_cast<uint32_t *>(codes);
-        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
-        f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
-        auto load_tile = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kVecPerThread]) {
-            const size_t base = tile * kTileVec + threadIdx.x;
-#pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
-                size_t i = base + (size_t)j * kThreads;
-                v[j] = (i < nvec) ? __builtin_nontemporal_load(&x4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
-                if (kUpdate) w[j] = (i < nvec) ? __builtin_nontemporal_load(&y4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
-            }
-        };
         auto encode_tile = [&](size_t tile, const f32x4 (&v)[kVecPerThread], f32x4 (&w)[kVecPerThread]) {
             const size_t base = tile * kTileVec + threadIdx.x;
             uint32_t packed[kVecPerThread];
@@ -92,18 +103,11 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
                 }
             }
         };
-        // Two register sets: the loads of the next tile are in flight while this one is encoded,
-        // so the memory pipe stays busy even with only two wavefronts per SIMD.
-        f32x4 va[kVecPerThread], vb[kVecPerThread], wa[kUpdate ? kVecPerThread : 1], wb[kUpdate ? kVecPerThread : 1];
-        auto load = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kUpdate ? kVecPerThread : 1]) {
-            load_tile(tile, v, reinterpret_cast<f32x4 (&)[kVecPerThread]>(w));
-        };
         auto finish = [&](size_t tile, const f32x4 (&v)[kVecPerThread], f32x4 (&w)[kUpdate ? kVecPerThread : 1]) {
             encode_tile(tile, v, reinterpret_cast<f32x4 (&)[kVecPerThread]>(w));
         };
         size_t t0 = blockIdx.x;
-        if (t0 < tiles) {
-            load(t0, va, wa);
+        if (t0 < tiles) {  // its loads are on their way since before the table
             for (;;) {
                 const size_t t1 = t0 + gridDim.x;
                 if (t1 < tiles) load(t1, vb, wb);

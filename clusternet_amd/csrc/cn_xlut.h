@@ -184,46 +184,36 @@ constexpr int kXMaxSteps = 160;
 
 CN_HD uint32_t magnitude_code(uint32_t c) { return c == 254u ? 254u : (c & 0x7fu); }
 
-// Step `s` under `precision`: its entry (boundary in |x| patterns, the four codes).  False when the
-// step cannot be pinned down (estimate out of range, or the neighbourhood is not below ... above).
-CN_HD bool xlut_locate_step(XStep s, float precision, const float *slot, XEntry *entry) {
-    const uint32_t kSign = 0x80000000u;
+// Step `s` under `precision`: its entry (boundary in |x| patterns, the four codes).  The literal procedure
+// looks at x only through the quotient x / precision: it takes the sign from it, and the magnitude code is a
+// step function of a = |x / precision| whose steps (found once, at precision 1, where a = |x| exactly) are
+// the S of the list.  IEEE division is monotone in |x| and symmetric in the signs, so under another precision
+// the step sits at the smallest |x| pattern with fl(|x| / |p|) >= S, within two patterns of fl(S |p|): ten
+// divisions around that estimate find it, and the four codes follow from the step's two magnitude codes and
+// the sign of the precision (254 carries no sign: the reference returns it before the sign is applied).
+// False when the step cannot be pinned down (estimate out of range, no change of sides among the ten).
+CN_HD bool xlut_locate_step(XStep s, float precision, const float * /*slot*/, XEntry *entry) {
     const float ap = precision < 0 ? -precision : precision;
     const uint32_t est = x_to_bits(x_from_bits(s.boundary) * ap);
     if (!(est >= 16u && est <= 0x7f800000u - 16u)) return false;  // also false for a NaN estimate
     const uint32_t below = s.codes & 0xffu, above = (s.codes >> 8) & 0xffu;
-    // ten independent evaluations around the estimate (independent so that they overlap), then the
-    // position of the step among them
-    uint32_t probe[10], code[10];
-    for (int j = 0; j < 10; ++j) probe[j] = est - 5 + (uint32_t)j;
-    encode_exact_many<10>(probe, precision, slot, code);
-    if (magnitude_code(code[0]) != below) return false;
-    int at = 0;  // first j whose code is `above`
-    bool clean = true;
-    for (int j = 1; j < 10; ++j) {
-        const uint32_t m = magnitude_code(code[j]);
-        if (at == 0) {
-            if (m == above) at = j; else if (m != below) clean = false;
-        } else if (m != above) {
-            clean = false;
-        }
-    }
-    if (at == 0 || !clean) return false;
-    const uint32_t found = est - 5 + (uint32_t)at;
-    uint32_t bp = code[0], tp = code[1];
+    bool upper[10];
+    for (int j = 0; j < 10; ++j) upper[j] = x_to_bits(x_from_bits(est - 5 + (uint32_t)j) / ap) >= s.boundary;
+    if (upper[0] || !upper[9]) return false;
+    int at = 9;  // first j on the upper side
+    for (int j = 8; j >= 1; --j) at = upper[j] ? j : at;
     for (int j = 1; j < 10; ++j)
-        if (j == at) { bp = code[j - 1]; tp = code[j]; }
-    const uint32_t mirrored[2] = {(found - 1) | kSign, found | kSign};
-    uint32_t mirror_code[2];
-    encode_exact_many<2>(mirrored, precision, slot, mirror_code);
-    const uint32_t bn = mirror_code[0], tn = mirror_code[1];
-    if (magnitude_code(bn) != below || magnitude_code(tn) != above) return false;
-    *entry = XEntry{found, pack_codes(bp, tp, bn, tn)};
+        if (upper[j] != (j >= at)) return false;  // cannot happen with a monotone quotient; checked all the same
+    const uint32_t found = est - 5 + (uint32_t)at;
+    // quotient >= 0: the magnitude code; quotient < 0: with the sign bit, except 254
+    const uint32_t below_minus = below == 254u ? 254u : (below | 0x80u), above_minus = above == 254u ? 254u : (above | 0x80u);
+    const bool flip = precision < 0;  // then x >= 0 has the negative quotient
+    *entry = flip ? XEntry{found, pack_codes(below_minus, above_minus, below, above)}
+                  : XEntry{found, pack_codes(below, above, below_minus, above_minus)};
     return true;
 }
 
-// Entry of a bucket without a step, given the entry of the nearest step below (`from_above` false)
-// ... or the codes above the last step (`from_above` true).
+// Entry of a bucket without a step: the codes below the step `step` (`above` false) or above it (`above` true).
 CN_HD XEntry xlut_flat_entry(XEntry step, bool above) {
     const uint32_t c = step.codes;
     const uint32_t pos = above ? ((c >> 8) & 0xffu) : (c & 0xffu);
@@ -266,13 +256,16 @@ inline bool xlut_build_from_steps(const XStep *steps, int count, float precision
     lut[kXEntries - 1] = xlut_entry(kXEntries - 1, precision, slot, &bad);
     unusable |= bad;
     if ((uint64_t)first + kXBuckets > 0xff00u) unusable = true;  // infinity / NaN inside the window
+    // a bucket without a step carries the codes above the nearest step below it; below the first step,
+    // the codes below that one
     int previous = 0;
-    XEntry e{};
+    XEntry e{}, before{};
     for (int k = 0; k < count && !unusable; ++k) {
+        before = e;
         if (!xlut_locate_step(steps[k], precision, slot, &e)) { unusable = true; break; }
         const int64_t index = (int64_t)(e.boundary >> kXShift) - (int64_t)first + 1;
         if (index <= previous || index > kXBuckets) { unusable = true; break; }
-        for (int i = previous + 1; i < index; ++i) lut[i] = xlut_flat_entry(e, false);
+        for (int i = previous + 1; i < index; ++i) lut[i] = k == 0 ? xlut_flat_entry(e, false) : xlut_flat_entry(before, true);
         lut[index] = e;
         previous = (int)index;
     }
