@@ -264,24 +264,38 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
             m = max(m, max_key<kAbs>(__float_as_uint(x[i])));
     }
     m = block_max(m, smem);
-    // The workgroup folds its maximum into one word and then counts itself in on another; the last to arrive
-    // reads the maximum, writes the result and puts both words back to 0.  Both are device-scope atomics that
-    // return a value, and the count is made to depend on what the fold returned, so the fold has been performed
-    // before the count is issued: ordering by data dependence instead of by fences, which cost far more here
-    // (a release fence per workgroup writes the L2 back; nothing in this kernel needs that).
+    // Two-level ticket.  The workgroup folds its maximum into the running maximum of its group of eight with a
+    // device-scope atomicMax and counts itself in with an atomicAdd; the last of a group to arrive carries the
+    // group's maximum to the second level in the same way, and the last group there writes the result.  Every
+    // word is put back to 0 by whoever arrived last at it.  Both atomics return a value and the count is made
+    // to depend on what the fold returned, so the fold has been performed before the count is issued:
+    // ordering by data dependence instead of by fences, which cost far more here (a release fence per
+    // workgroup writes the L2 back; nothing in this kernel needs that).  Atomics on one word are performed one
+    // after the other, about 12 ns each, hence the groups: their words lie on lines of their own.
     if (threadIdx.x == 0) {
-        uint32_t *running = tickets, *arrived = tickets + kTicketStride;
-        const uint32_t before = atomicMax(running, m);
-        uint32_t one = 1u;
-        asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
-        uint32_t ticket = atomicAdd(arrived, one);
-        if (ticket == gridDim.x - 1) {
-            uint32_t *from = running;
-            asm volatile("" : "+v"(from) : "v"(ticket));
-            const uint32_t of_all = __hip_atomic_load(from, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            out[0] = max_unkey<kAbs>(of_all);
-            __hip_atomic_store(running, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t groups = (gridDim.x + kTicketGroup - 1) / kTicketGroup;
+        const uint32_t group = blockIdx.x / kTicketGroup;
+        const uint32_t left = gridDim.x - group * kTicketGroup;
+        const uint32_t members = left < (uint32_t)kTicketGroup ? left : (uint32_t)kTicketGroup;
+        uint32_t *first = tickets + (1 + group) * kTicketStride, *second = tickets;
+        auto fold_and_count = [](uint32_t *line, uint32_t value) -> uint32_t {
+            const uint32_t before = atomicMax(line, value);
+            uint32_t one = 1u;
+            asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
+            return atomicAdd(line + 1, one);
+        };
+        auto take = [](uint32_t *line, uint32_t ticket) -> uint32_t {
+            asm volatile("" : "+v"(line) : "v"(ticket));  // the read is not issued before the ticket is known
+            const uint32_t v = __hip_atomic_load(line, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(line, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(line + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return v;
+        };
+        const uint32_t ticket = fold_and_count(first, m);
+        if (ticket == members - 1) {
+            const uint32_t of_group = take(first, ticket);
+            const uint32_t ticket2 = fold_and_count(second, of_group);
+            if (ticket2 == groups - 1) out[0] = max_unkey<kAbs>(take(second, ticket2));
         }
     }
 }

@@ -38,9 +38,11 @@ struct Context {
 };
 constexpr int kMaxDevices = 16;
 constexpr int kReduceSlots = 4096;
-// Max reductions: the running maximum and the arrival count, each on a 128-byte line of its own, both left at 0.
+// Max reductions: a running maximum and an arrival count per group of kTicketGroup workgroups and one pair for
+// the groups, every pair on a 128-byte line of its own, all left at 0.
+constexpr int kTicketGroup = 8;
 constexpr int kTicketStride = 32;
-constexpr int kTicketWords = 2 * kTicketStride;
+constexpr int kTicketWords = (1 + kReduceSlots / kTicketGroup) * kTicketStride;
 
 // A kernel's attributes (its dynamic LDS limit) are set per device: one flag per device for a call site.
 struct OncePerDevice {
