@@ -143,8 +143,11 @@ def test_gemm_plan_covers_k_and_fits_workspace():
             for (M, N, K) in shapes:
                 L.cn_host_plan_gemm(M, N, K, 256, ws, force, out)
                 tm, tn, kit, splits, ips, units, tile_n, tile_m = list(out)
-                # the 32-row tile when asked for, and unasked for products of at most 64 rows
-                assert tile_m == (32 if force == 32 or (force == 0 and M <= 64) else 128)
+                # the 32-row tile when asked for; unasked for products of at most 64 rows and for those too
+                # small to give every compute unit two 128-row tiles even at the deepest split
+                deepest = max(1, min(64, max(1, -(-K // 32)) // 4, ws // (M * N * 4)))
+                small = -(-M // 128) * -(-N // 128) * deepest < 512
+                assert tile_m == (32 if force == 32 or (force == 0 and (M <= 64 or small)) else 128)
                 assert tile_n in (128, 256) and (force in (0, 32) or tile_n == force) and (tile_m == 128 or tile_n == 128)
                 assert tm == -(-M // tile_m) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
                 assert splits >= 1 and units == tm * tn * splits
