@@ -295,7 +295,18 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
     // (tile corners, buffer descriptors) must stay wave-uniform.
     const uint32_t tiles32 = (uint32_t)g.tiles, tiles_n32 = (uint32_t)g.tiles_n;
     const uint32_t split_v = unit / tiles32, tile_v = unit - split_v * tiles32;
-    const uint32_t tm_v = tile_v / tiles_n32, tn_v = tile_v - tm_v * tiles_n32;
+    // Tiles of 128 rows go row of tiles by row of tiles (neighbours share their A panel; the B panels of a
+    // chunk are shared through the L2 and the Infinity Cache).  The 32-row tiles of a product are few in m and
+    // there to be cheap in B traffic, so there the tiles of one B panel are neighbours.
+    uint32_t tm_v, tn_v;
+    if (TM == kTileM) {
+        tm_v = tile_v / tiles_n32;
+        tn_v = tile_v - tm_v * tiles_n32;
+    } else {
+        const uint32_t tiles_m32 = tiles32 / tiles_n32;
+        tn_v = tile_v / tiles_m32;
+        tm_v = tile_v - tn_v * tiles_m32;
+    }
     const int64_t split = __builtin_amdgcn_readfirstlane((int)split_v);
     const int64_t tm = __builtin_amdgcn_readfirstlane((int)tm_v);
     const int64_t tn = __builtin_amdgcn_readfirstlane((int)tn_v);
