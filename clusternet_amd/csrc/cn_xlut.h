@@ -6,9 +6,11 @@
 // search are both monotone in |x|) with the sign of x / precision on top.  The table is indexed by
 // the leading 17 bits of |x| (exponent and 8 mantissa bits): every bucket stores the code below and
 // above the one step it can contain, for either sign of x, and the first bit pattern that takes
-// the upper code.  All entries come from evaluations of the literal procedure (encode_exact), so the
-// table reproduces the literal procedure for every input by construction: no approximate quotient,
-// no guard band, no restriction on the precision.  Buckets of the logarithmic range are 0.4 % wide
+// the upper code.  The steps come from evaluations of the literal procedure (encode_exact) at precision 1,
+// where the quotient is |x| itself, and are carried to another precision by the one operation through
+// which the procedure sees x, the IEEE division (xlut_locate_step); the two sentinel entries are literal
+// evaluations at the precision itself.  No approximate quotient, no guard band, no restriction on the
+// precision.  Buckets of the logarithmic range are 0.4 % wide
 // and the codebook's steps are at least 0.8 % apart, so a bucket holds at most one step; where that
 // fails (denormal inputs under a tiny precision), where a step cannot be pinned down or where the
 // fixed-size table does not cover the coded range, the build says so and the encoder evaluates the
@@ -174,8 +176,8 @@ CN_HD XEntry xlut_entry(int index, float precision, const float *slot, bool *unu
 // smallest quotient pattern S that takes the upper code, with the two magnitude codes - are the same
 // for every precision, because the code depends on x only through fl(|x| / |p|).  For another
 // precision the step sits at the smallest |x| with fl(|x| / |p|) >= S, within two patterns of
-// fl(S |p|): a workgroup finds all steps with nine literal evaluations each and fills the buckets
-// between them, which is cheap enough to do in every workgroup instead of sharing a table.
+// fl(S |p|): a workgroup finds all steps with ten divisions each and fills the buckets between them,
+// which is cheap enough to do in every workgroup instead of sharing a table.
 struct XStep {
     uint32_t boundary;  // S: smallest quotient pattern that takes `above`
     uint32_t codes;     // below | above << 8, magnitude codes (0 .. 127 or 254)
