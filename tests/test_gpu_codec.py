@@ -144,6 +144,34 @@ def test_compress_random_precisions(dev):
         assert np.array_equal(got, oracle.port_compress(x, float(prec))), prec
 
 
+def test_compress_many_precisions_of_every_kind(dev):
+    """Sixty precisions drawn over sixty decades, of either sign, exact powers of two and values next to the
+    smallest normal number: each builds its own encoder table on the device (the steps of the code function
+    are carried over from precision 1 through the division), and the codes of 2^18 inputs spread over the
+    coded range must be those of the literal procedure."""
+    import clusternet_amd as cn
+    rng = np.random.default_rng(2026)
+    n = 1 << 18
+    for it in range(60):
+        kind = it % 5
+        if kind == 0:
+            p = np.exp(rng.uniform(np.log(1e-30), np.log(1e30)))
+        elif kind == 1:
+            p = -np.exp(rng.uniform(np.log(1e-6), np.log(1e3)))
+        elif kind == 2:
+            p = 2.0 ** int(rng.integers(-100, 100))
+        elif kind == 3:
+            p = rng.uniform(0.001, 10)
+        else:
+            p = np.exp(rng.uniform(np.log(1e-38), np.log(1e-30)))
+        p = float(np.float32(p))
+        mag = np.exp(rng.uniform(np.log(1e-7), np.log(1.5), n)).astype(np.float32) * np.float32(abs(p))
+        x = (mag * rng.choice(np.array([-1.0, 1.0], np.float32), n)).astype(np.float32)
+        x[:6] = [0.0, -0.0, np.inf, -np.inf, np.nan, p]
+        got = cn.compression_8bit(_t(x, dev), p).cpu().numpy()
+        assert np.array_equal(got, oracle.compress(x, p)), p
+
+
 def test_large_tensor_by_tiling(dev):
     """A 1.07e9-element tensor (4.3 GB) built by repeating a block whose codes are verified on the
     CPU: every repetition must carry the same codes, and decoding must repeat likewise."""
