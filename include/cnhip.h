@@ -128,7 +128,8 @@ cn_status cn_compress_8bit_dp(const float *x_device, const float *precision_devi
 
 /* cn_compress_8bit followed by cn_decompress_8bit_axpy on its codes, in one pass: codes[i] as above and
  * y[i] += alpha * (decoded value of codes[i]).  A gradient's codes for the exchange and the own weight
- * update (source/Layer.cpp:365, 430-433) at 13 bytes per element instead of 5 + 9; same bits. */
+ * update (source/Layer.cpp:365, 430-433) at 13 bytes per element instead of 5 + 9; same bits.  x, codes and y
+ * must not overlap. */
 cn_status cn_compress_8bit_axpy(const float *x_device, float precision, size_t n, uint8_t *codes_device,
                                 float alpha, float *y_device, void *stream);
 cn_status cn_compress_8bit_axpy_dp(const float *x_device, const float *precision_device, size_t n,
