@@ -11,7 +11,9 @@
 //             tile is fetched once per 256 output columns and every B fragment read from LDS feeds four
 //             MFMAs instead of two: less L2 -> LDS and LDS -> register traffic per flop, which matters
 //             because the part runs power-limited on realistic data
-//   32 x 128  for products with no more than 64 rows (a batch of 32 against 8-bit weights): wavefronts
+//   32 x 128  for products with no more than 32 rows (a batch of 32 against 8-bit weights) and for products
+//             too small to fill the machine with larger tiles (64 x 128, two blocks per wavefront, for 33 to
+//             64 rows): wavefronts
 //             1 x 4, one 32 x 32 block each; K advances 32 per stage through three LDS stages (60 KiB), two of
 //             them in flight.  A 128-row tile would spend
 //             three quarters of its MFMAs on rows that do not exist; with this one such a product costs
@@ -68,8 +70,10 @@ template <int TM, int TN> struct Geo;
 template <> struct Geo<128, 128> { static constexpr int WM = 2, WN = 2, FM = 2, FN = 2, BK = 32, NST = 2; };
 template <> struct Geo<128, 256> { static constexpr int WM = 1, WN = 4, FM = 4, FN = 2, BK = 16, NST = 2; };
 template <> struct Geo<32, 128> { static constexpr int WM = 1, WN = 4, FM = 1, FN = 1, BK = 32, NST = 3; };
+template <> struct Geo<64, 128> { static constexpr int WM = 1, WN = 4, FM = 2, FN = 1, BK = 32, NST = 3; };
 static_assert(gemm_tile_k(128) == Geo<128, 128>::BK && gemm_tile_k(256) == Geo<128, 256>::BK &&
-                  gemm_tile_k(128) == Geo<kTileMLow, 128>::BK && kTileM == 128 && kTileMLow == 32,
+                  gemm_tile_k(128) == Geo<kTileMLow, 128>::BK && gemm_tile_k(128) == Geo<kTileMMid, 128>::BK &&
+                  kTileM == 128 && kTileMLow == 32 && kTileMMid == 64,
               "planner and kernel disagree");
 
 struct GemmArgs {
@@ -773,6 +777,7 @@ static cn_status launch_tile(const GemmArgs &args, int device, hipStream_t st) {
 template <bool A_KC, int B_KIND>
 static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, hipStream_t st) {
     if (plan.tile_m == kTileMLow) return launch_tile<A_KC, B_KIND, 128, kTileMLow>(args, device, st);
+    if (plan.tile_m == kTileMMid) return launch_tile<A_KC, B_KIND, 128, kTileMMid>(args, device, st);
     return plan.tile_n == 256 ? launch_tile<A_KC, B_KIND, 256, kTileM>(args, device, st)
                               : launch_tile<A_KC, B_KIND, 128, kTileM>(args, device, st);
 }
@@ -856,8 +861,10 @@ extern "C" {
 void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
 
 // Test and tuning hook: 0 = let the planner choose the tile, 128 / 256 = force that width of the 128-row
-// tile, 32 = force the 32 x 128 tile.
-void cn_host_force_gemm_tile_n(int tile_n) { g_force_tile_n = (tile_n == 128 || tile_n == 256 || tile_n == kTileMLow) ? tile_n : 0; }
+// tile, 32 / 64 = force the 32 x 128 / 64 x 128 tile.
+void cn_host_force_gemm_tile_n(int tile_n) {
+    g_force_tile_n = (tile_n == 128 || tile_n == 256 || tile_n == kTileMLow || tile_n == kTileMMid) ? tile_n : 0;
+}
 
 cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                       const float *B, int64_t ldb, float *C, int64_t ldc, void *stream) {

@@ -77,12 +77,13 @@ GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace
     // tile: four times as many, lighter workgroups (measured: 128 x 1024 x 784 in 9.7 us instead of 18.5 us,
     // 784 x 1024 x 128 in 5.6 us instead of 11.8 us).
     const bool small = p.tiles_m * tiles_n128 * split_limit(it128, 4, out_bytes, workspace_bytes) < cus * 2;
-    if (force_tile_n == kTileMLow || (force_tile_n == 0 && (M <= kLowTileMaxRows || small))) {
+    if (force_tile_n == kTileMLow || force_tile_n == kTileMMid || (force_tile_n == 0 && (M <= kLowTileMaxRows || small))) {
         // A stage of the 32 x 128 tile moves 20 KB for a quarter of the unit's flops: it costs what its
-        // loads cost, about a third of the unit.
-        p.tile_m = kTileMLow;
-        p.tiles_m = (M + kTileMLow - 1) / kTileMLow;
-        const Choice c = best_split(p.tiles_m * tiles_n128, it128, cus, 0.35, split_limit(it128, 4, out_bytes, workspace_bytes), out_bytes);
+        // loads cost, about a third of the unit; the 64 x 128 tile, for 33 .. 64 rows, half of the unit.
+        const bool mid = force_tile_n == kTileMMid || (force_tile_n == 0 && !small && M > kTileMLow);
+        p.tile_m = mid ? kTileMMid : kTileMLow;
+        p.tiles_m = (M + p.tile_m - 1) / p.tile_m;
+        const Choice c = best_split(p.tiles_m * tiles_n128, it128, cus, mid ? 0.55 : 0.35, split_limit(it128, 4, out_bytes, workspace_bytes), out_bytes);
         p.tile_n = 128;
         p.tiles_n = tiles_n128;
         p.k_iters = it128;

@@ -60,14 +60,14 @@ cn_status current_context(Context **out);
 
 // ---- GEMM planning (host, pure function; exported for tests) ---------------------------------
 struct GemmPlan {
-    int tile_m;          // output tile is tile_m x tile_n: 128 x 128, 128 x 256, or 32 x 128 for a handful of rows
+    int tile_m;          // output tile is tile_m x tile_n: 128 x 128, 128 x 256, or 32 x 128 / 64 x 128 for a handful of rows
     int tile_n;
     int64_t tiles_m, tiles_n, k_iters;
     int splits;          // number of K chunks (1 = write C directly)
     int64_t iters_per_split;
     int64_t units;       // tiles_m * tiles_n * splits = grid size
 };
-// force_tile_n: 0 = choose, 128 or 256 = use that tile width, 32 = use the 32 x 128 tile.
+// force_tile_n: 0 = choose, 128 or 256 = use that tile width, 32 / 64 = use the 32 x 128 / 64 x 128 tile.
 // C = sum of `splits` M x N planes held at the start of the workspace (ascending order); optional max |C|.
 cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float *C, int64_t ldc, uint32_t *amax,
                            hipStream_t st);
@@ -75,8 +75,9 @@ cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 
 constexpr int kTileM = 128;
-constexpr int kTileMLow = 32;      // rows of the tile for products with a handful of rows
-constexpr int kLowTileMaxRows = 64;  // largest M that takes it unasked
+constexpr int kTileMLow = 32;      // rows of the tile for products with a handful of rows or little work
+constexpr int kTileMMid = 64;      // rows of the tile for products of 33 .. 64 rows
+constexpr int kLowTileMaxRows = 64;  // largest M that takes one of the two unasked
 // K depth of one pipeline stage for a tile width (iters in a GemmPlan count these).
 constexpr int gemm_tile_k(int tile_n) { return tile_n == 256 ? 16 : 32; }
 

@@ -19,10 +19,10 @@ def dev():
     return torch.device("cuda:0")
 
 
-@pytest.fixture(autouse=True, params=[128, 256, 32, 0], ids=["tile128", "tile256", "tile32x128", "planned"])
+@pytest.fixture(autouse=True, params=[128, 256, 32, 64, 0], ids=["tile128", "tile256", "tile32x128", "tile64x128", "planned"])
 def tile_width(request, dev):
-    """Every case runs on all three kernel geometries (128 x 128, 128 x 256 and 32 x 128 output tiles)
-    and once more with the planner's own choice."""
+    """Every case runs on all four kernel geometries (128 x 128, 128 x 256, 32 x 128 and 64 x 128 output
+    tiles) and once more with the planner's own choice."""
     import clusternet_amd as cn
     cn.lib().cn_host_force_gemm_tile_n(request.param)
     yield request.param

@@ -139,7 +139,7 @@ def test_gemm_plan_covers_k_and_fits_workspace():
               (128, 10, 4096), (5000, 5000, 31)]
     shapes += [tuple(int(v) for v in rng.integers(1, 3000, 3)) for _ in range(200)]
     for ws in (16 << 20, 1 << 30):
-        for force in (0, 128, 256, 32):
+        for force in (0, 128, 256, 32, 64):
             for (M, N, K) in shapes:
                 L.cn_host_plan_gemm(M, N, K, 256, ws, force, out)
                 tm, tn, kit, splits, ips, units, tile_n, tile_m = list(out)
@@ -147,8 +147,13 @@ def test_gemm_plan_covers_k_and_fits_workspace():
                 # small to give every compute unit two 128-row tiles even at the deepest split
                 deepest = max(1, min(64, max(1, -(-K // 32)) // 4, ws // (M * N * 4)))
                 small = -(-M // 128) * -(-N // 128) * deepest < 512
-                assert tile_m == (32 if force == 32 or (force == 0 and (M <= 64 or small)) else 128)
-                assert tile_n in (128, 256) and (force in (0, 32) or tile_n == force) and (tile_m == 128 or tile_n == 128)
+                if force in (32, 64):
+                    assert tile_m == force
+                elif force == 0 and (M <= 64 or small):
+                    assert tile_m == (64 if (32 < M <= 64 and not small) else 32)
+                else:
+                    assert tile_m == 128
+                assert tile_n in (128, 256) and (force in (0, 32, 64) or tile_n == force) and (tile_m == 128 or tile_n == 128)
                 assert tm == -(-M // tile_m) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
                 assert splits >= 1 and units == tm * tn * splits
                 assert ips * splits >= kit and ips * (splits - 1) < kit  # every chunk non-empty
