@@ -178,6 +178,27 @@ def bench_codec(torch, cn, dev):
     return res
 
 
+def bench_cfg1(torch, cn, dev):
+    """The reference's own small case: one 784 -> 1024 layer on a batch of 128 (forward product, weight
+    gradient, input gradient; 0.2 GFLOP each).  Microsecond kernels, so timed replayed from a HIP graph where
+    the capture is allowed, else launched one by one."""
+    gen = torch.Generator(device=dev).manual_seed(11)
+    A = torch.rand((128, 784), device=dev, generator=gen)
+    W = make_uniform(torch, (784, 1024), (6.0 / (784 + 1024)) ** 0.5, dev, gen)
+    dC = torch.empty((128, 1024), device=dev).normal_(0.0, 0.01, generator=gen)
+    out = {}
+    for name, fn, shape in (("dot_128x1024x784", lambda c: cn.gemm(A, W, False, False, out=c), (128, 1024)),
+                            ("Tdot_784x1024x128", lambda c: cn.gemm(A, dC, True, False, out=c), (784, 1024)),
+                            ("dotT_128x784x1024", lambda c: cn.gemm(dC, W, False, True, out=c), (128, 784))):
+        C = torch.empty(shape, device=dev)
+        t = time_replayed(torch, lambda: fn(C), 20, 50)
+        how = "replayed from a graph"
+        if t is None:
+            t, how = time_region(torch, lambda: fn(C), 200, 1000), "launched one by one"
+        out[name] = {"us": t * 1e3, "TFLOPs": 2.0 * 128 * 784 * 1024 / t / 1e9, "timing": how}
+    return out
+
+
 def bench_fused(torch, cn, dev):
     """C = A . decode(W8) for A {32,128,512} x 4096, W 4096 x 4096: fused kernel against
     decompression_8bit followed by dot."""
@@ -393,6 +414,7 @@ def main():
         extra["gemm2_128x20000x40000"] = {"ms": g["gemm2_ms"], "TFLOPs": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12,
                                           "frac_mfma_peak": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS}
         extra["readme_pair_ms_reference_unknown_hw"] = 117.704285
+        extra["cfg1_layer_128x784x1024"] = bench_cfg1(torch, cn, dev)
         if not args.no_cpu and args.only is None:
             line["cpu_baseline"] = cpu_baseline(torch, g["tensors"])
         del g
