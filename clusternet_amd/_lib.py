@@ -436,6 +436,7 @@ def _declare_layers(L):
     L.cn_add_row_vector_f32.argtypes = [vp, vp, i64, i64, vp, vp]
     L.cn_maxout_f32.argtypes = [vp, i64, i64, C.c_int, vp, vp, vp]
     L.cn_bias_maxout_f32.argtypes = [vp, i64, vp, i64, i64, C.c_int, vp, vp, vp]
+    L.cn_gemm_f32_bias_maxout.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, C.c_int, vp, vp, vp]
     L.cn_csr_gemm_bias_maxout_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, C.c_int, vp, vp, vp]
     L.cn_expand_to_maxout_grad_f32.argtypes = [vp, vp, i64, i64, C.c_int, vp, vp]
     L.cn_softmax_f32.argtypes = [vp, i64, i64, vp, vp]
@@ -496,6 +497,24 @@ def bias_maxout(A, v, pool):
     arg = torch.empty_like(out)
     check(L.cn_bias_maxout_f32(A.data_ptr(), _ld(A), v.data_ptr(), A.shape[0], A.shape[1], int(pool), out.data_ptr(),
                                arg.data_ptr(), _stream()))
+    return out, arg
+
+
+def dot_bias_maxout(A, B, v, pool):
+    """maxout(A B + v): (values, winners' columns); bias and maxout ride on the product's chunk sum."""
+    import torch
+    L = _declare_layers(lib())
+    _need(A, torch.float32, "A")
+    _need(B, torch.float32, "B")
+    _contig(v, "v")
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2 or v.numel() != N or N % pool:
+        raise CnError(2, "Matrix size error: A %s, B %s, v %d, pool %d" % (tuple(A.shape), tuple(B.shape), v.numel(), pool))
+    out = torch.empty((M, N // pool), dtype=torch.float32, device=A.device)
+    arg = torch.empty_like(out)
+    check(L.cn_gemm_f32_bias_maxout(0, 0, M, N, K, A.data_ptr(), _ld(A), B.data_ptr(), _ld(B), v.data_ptr(), int(pool),
+                                    out.data_ptr(), arg.data_ptr(), _stream()))
     return out, arg
 
 

@@ -731,6 +731,38 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restr
     if (amax_out) publish_absmax(amax, amax_out);
 }
 
+// The chunk sum with the bias and maxout of the forward pass behind it: out, argmax = maxout(sum of planes +
+// bias) over `pool` consecutive columns.  The planes are added in ascending order and the bias last, so the
+// values compared are those of the chunk sum followed by add_row_vector.
+__global__ __launch_bounds__(256) void splitk_reduce_bias_maxout_kernel(const float *__restrict__ partial, int splits,
+                                                                        int64_t M, int64_t N, const float *__restrict__ bias,
+                                                                        int pool, float *__restrict__ out,
+                                                                        float *__restrict__ argmax) {
+    const int64_t plane = M * N, oc = N / pool, total = M * oc;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / oc, o = i % oc;
+        const float *src = partial + r * N + o * pool;
+        float best = 0.0f;
+        int arg = 0;
+        for (int p = 0; p < pool; ++p) {
+            float s = src[p];
+            int c = 1;
+            for (; c + 8 <= splits; c += 8) {
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) t[u] = src[p + (c + u) * plane];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s += t[u];
+            }
+            for (; c < splits; ++c) s += src[p + c * plane];
+            const float z = s + bias[o * pool + p];
+            if (p == 0 || best < z) { best = z; arg = p; }
+        }
+        out[i] = best;
+        argmax[i] = (float)(o * pool + arg);
+    }
+}
+
 __global__ void set_word_kernel(uint32_t *p, uint32_t value) {
     if (threadIdx.x == 0) *p = value;
 }
@@ -785,10 +817,17 @@ static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, 
 static int g_force_tile_n = 0;
 static bool g_wide_store = true;
 
+// Bias and maxout behind the product (the forward pass of a maxout layer): the product itself is not returned.
+struct BiasMaxout {
+    const float *bias;
+    int pool;
+    float *out, *argmax;  // M x N / pool, contiguous
+};
+
 static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_t K, const float *A,
                            int64_t lda, const void *B, int64_t ldb, float scale, float *C, int64_t ldc,
-                           float *absmax_out, void *stream) {
-    const char *who = w8 ? "gemm_f32_w8" : "gemm_f32";
+                           float *absmax_out, void *stream, const BiasMaxout *then = nullptr) {
+    const char *who = then ? "gemm_f32_bias_maxout" : (w8 ? "gemm_f32_w8" : "gemm_f32");
     if (M < 0 || N < 0 || K < 0) { set_error("%s: negative dimension", who); return CN_ERR_SHAPE; }
     if (lda < (ta ? M : K) || ldb < (tb ? K : N) || ldc < N) {
         set_error("%s: leading dimension too small (lda %lld, ldb %lld, ldc %lld for M %lld N %lld K %lld)",
@@ -800,7 +839,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         return CN_ERR_SHAPE;
     }
     if ((M == 0 || N == 0) && !absmax_out) return CN_OK;
-    if ((M > 0 && N > 0) && (!C || (K > 0 && (!A || !B)))) { set_error("%s: NULL operand", who); return CN_ERR_NULL; }
+    if ((M > 0 && N > 0) && ((!C && !then) || (K > 0 && (!A || !B)))) { set_error("%s: NULL operand", who); return CN_ERR_NULL; }
     Context *ctx;
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
@@ -814,11 +853,26 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     }
     if (M == 0 || N == 0) return CN_OK;
     if (K == 0) {
+        if (then) {
+            if ((size_t)M * (size_t)N * sizeof(float) > ctx->workspace_bytes) { set_error("%s: product does not fit the workspace", who); return CN_ERR_WORKSPACE; }
+            C = (float *)ctx->workspace;
+            ldc = N;
+        }
         hipLaunchKernelGGL(zero_matrix_kernel, dim3(ctx->num_cu * 4), dim3(256), 0, st, C, M, N, ldc);
         CN_HIP(hipGetLastError());
+        if (then) return cn_bias_maxout_f32(C, N, then->bias, M, N, then->pool, then->out, then->argmax, stream);
         return CN_OK;
     }
     GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->workspace_bytes, g_force_tile_n);
+    if (then && plan.splits == 1) {
+        // no chunk sum to fold into: the product goes to the workspace and one pass over it follows
+        if ((size_t)M * (size_t)N * sizeof(float) > ctx->workspace_bytes) {
+            set_error("%s: product does not fit the workspace", who);
+            return CN_ERR_WORKSPACE;
+        }
+        C = (float *)ctx->workspace;
+        ldc = N;
+    }
     if (plan.units <= 0 || plan.units > 0x7fffffffLL) {
         set_error("%s: %lld work units exceed the launch limit", who, (long long)plan.units);
         return CN_ERR_SHAPE;
@@ -847,6 +901,14 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     else                 s = launch<false, B_KC>(a, plan, ctx->device, st);
     if (s != CN_OK) return s;
 
+    if (then) {
+        if (plan.splits == 1) return cn_bias_maxout_f32(C, N, then->bias, M, N, then->pool, then->out, then->argmax, stream);
+        const int64_t work = M * (N / then->pool), blocks = (work + 255) / 256, cap = (int64_t)ctx->num_cu * 8;
+        hipLaunchKernelGGL(splitk_reduce_bias_maxout_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, st,
+                           (const float *)ctx->workspace, plan.splits, M, N, then->bias, then->pool, then->out, then->argmax);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
     if (plan.splits > 1) return add_chunk_planes(ctx, plan.splits, M, N, C, ldc, amax, st);
     return CN_OK;
 }
@@ -876,6 +938,18 @@ cn_status cn_gemm_f32_absmax(int trans_a, int trans_b, int64_t M, int64_t N, int
                              void *stream) {
     if (!absmax_out) { set_error("gemm_f32_absmax: NULL output for the maximum"); return CN_ERR_NULL; }
     return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, C, ldc, absmax_out, stream);
+}
+
+cn_status cn_gemm_f32_bias_maxout(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                                  const float *B, int64_t ldb, const float *bias, int pool, float *out, float *argmax,
+                                  void *stream) {
+    if (pool < 1 || N % (pool > 0 ? pool : 1) != 0) {
+        set_error("gemm_f32_bias_maxout: columns are not a multiple of the pool size");
+        return CN_ERR_SHAPE;
+    }
+    if (M > 0 && N > 0 && (!bias || !out || !argmax)) { set_error("gemm_f32_bias_maxout: NULL pointer"); return CN_ERR_NULL; }
+    const BiasMaxout then{bias, pool, out, argmax};
+    return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, nullptr, N, nullptr, stream, &then);
 }
 
 cn_status cn_gemm_f32_w8(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W,

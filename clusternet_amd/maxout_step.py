@@ -36,8 +36,8 @@ def forward(X, params, pool=2):
     if isinstance(X, SparseInput):
         h1, a1 = L.csr_gemm_bias_maxout(X.csr, W1, b1, pool)
     else:
-        h1, a1 = L.bias_maxout(L.dot(X, W1), b1, pool)
-    h2, a2 = L.bias_maxout(L.dot(h1, W2), b2, pool)
+        h1, a1 = L.dot_bias_maxout(X, W1, b1, pool)
+    h2, a2 = L.dot_bias_maxout(h1, W2, b2, pool)
     p = L.softmax(L.add_row_vector(L.dot(h2, W3), b3))
     return p, (h1, a1, h2, a2)
 

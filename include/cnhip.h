@@ -272,6 +272,14 @@ cn_status cn_sgd_update_f32(float *w_device, const float *grad_device, float rat
 /* out[r][c] = A[r][c] + v[c].  addMatrixVector, source/basicOps.cu:966-974. */
 cn_status cn_add_row_vector_f32(const float *A_device, const float *v_device, int64_t rows,
                                 int64_t cols, float *out_device, void *stream);
+/* out, argmax = maxout(op(A) op(B) + bias): cn_gemm_f32, cn_add_row_vector_f32 and cn_maxout_f32 as one call, the
+ * forward pass of a maxout layer (source/Layer.cpp:256-258: dot, addMatrixVector, maxout).  Where the product is
+ * summed over chunks of K, bias and maxout ride on that sum and the product never reaches memory as a whole;
+ * elsewhere it passes through the library's workspace (CN_ERR_WORKSPACE if it does not fit).  out and argmax are
+ * M x N / pool, contiguous; same bits as the three calls. */
+cn_status cn_gemm_f32_bias_maxout(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A_device,
+                                  int64_t lda, const float *B_device, int64_t ldb, const float *bias_device, int pool,
+                                  float *out_device, float *argmax_device, void *stream);
 /* out, argmax = maxout(A + v) as cn_add_row_vector_f32 followed by cn_maxout_f32 give them, in one pass and
  * without the sum in memory (A with leading dimension lda; out and argmax rows x cols/pool, contiguous).
  * The bias-and-maxout step behind every dot of the forward pass, source/Layer.cpp:256-258. */

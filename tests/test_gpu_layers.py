@@ -71,6 +71,34 @@ def test_bias_and_maxout_in_one_pass_equal_the_two_kernels(dev, rows, cols, pool
     assert np.array_equal(out.cpu().numpy().view(np.uint32), h.view(np.uint32)) and np.array_equal(arg.cpu().numpy(), a)
 
 
+@pytest.mark.parametrize("M,N,K,pool", [(128, 8192, 4096, 2), (128, 1024, 784, 2), (32, 512, 4096, 4), (7, 12, 33, 3),
+                                        (300, 260, 64, 2), (1, 2, 1, 1), (64, 4096, 100000, 2)])
+def test_product_with_bias_and_maxout_equals_the_three_calls(dev, M, N, K, pool):
+    """dot, add_row_vector and maxout as one call: where the product is summed over chunks of K the bias and
+    the maxout ride on that sum, elsewhere the product passes through the workspace; the same bits either
+    way, on every tile geometry."""
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev).manual_seed(M + N + K)
+    A = torch.randn((M, K), device=dev, generator=gen)
+    B = torch.randn((K, N), device=dev, generator=gen) * 0.05
+    v = torch.randn(N, device=dev, generator=gen) * 0.1
+    for force in (0, 32, 64, 128, 256):
+        cn.lib().cn_host_force_gemm_tile_n(force)
+        try:
+            out, arg = L.dot_bias_maxout(A, B, v, pool)
+            want_out, want_arg = L.maxout(L.add_row_vector(L.dot(A, B), v), pool)
+        finally:
+            cn.lib().cn_host_force_gemm_tile_n(0)
+        assert torch.equal(out.view(torch.int32), want_out.view(torch.int32)), force
+        assert torch.equal(arg, want_arg), force
+    with pytest.raises(L.CnError):
+        L.dot_bias_maxout(A, B, v[:-1] if N > 1 else torch.empty(0, device=dev), pool)
+    assert cn.lib().cn_gemm_f32_bias_maxout(0, 0, 4, 6, 4, None, 4, None, 6, None, 4, None, None, None) == 2  # 6 % 4
+    assert cn.lib().cn_gemm_f32_bias_maxout(0, 0, 4, 6, 4, None, 4, None, 6, None, 2, None, None, None) == 1  # NULL
+
+
 def _cpu_step(X, onehot, params, rate, pool):
     W1, b1, W2, b2, W3, b3 = params
     z1 = oracle.add_row_vector(oracle.gemm(X, W1), b1)
