@@ -437,6 +437,7 @@ def _declare_layers(L):
     L.cn_maxout_f32.argtypes = [vp, i64, i64, C.c_int, vp, vp, vp]
     L.cn_bias_maxout_f32.argtypes = [vp, i64, vp, i64, i64, C.c_int, vp, vp, vp]
     L.cn_gemm_f32_bias_maxout.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, C.c_int, vp, vp, vp]
+    L.cn_gemm_f32_expand_maxout_grad.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, C.c_int, vp, vp]
     L.cn_csr_gemm_bias_maxout_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, C.c_int, vp, vp, vp]
     L.cn_expand_to_maxout_grad_f32.argtypes = [vp, vp, i64, i64, C.c_int, vp, vp]
     L.cn_softmax_f32.argtypes = [vp, i64, i64, vp, vp]
@@ -516,6 +517,23 @@ def dot_bias_maxout(A, B, v, pool):
     check(L.cn_gemm_f32_bias_maxout(0, 0, M, N, K, A.data_ptr(), _ld(A), B.data_ptr(), _ld(B), v.data_ptr(), int(pool),
                                     out.data_ptr(), arg.data_ptr(), _stream()))
     return out, arg
+
+
+def dotT_expand_to_maxout_grad(E, W, argmax, pool):
+    """expand_to_maxout_grad(E W^T, argmax): the error of the layer below, in the winners' columns."""
+    import torch
+    L = _declare_layers(lib())
+    _need(E, torch.float32, "E")
+    _need(W, torch.float32, "W")
+    _contig(argmax, "argmax")
+    M, K = E.shape
+    N, K2 = W.shape
+    if K != K2 or tuple(argmax.shape) != (M, N):
+        raise CnError(2, "Matrix size error: E %s, W %s, argmax %s" % (tuple(E.shape), tuple(W.shape), tuple(argmax.shape)))
+    out = torch.empty((M, N * pool), dtype=torch.float32, device=E.device)
+    check(L.cn_gemm_f32_expand_maxout_grad(0, 1, M, N, K, E.data_ptr(), _ld(E), W.data_ptr(), _ld(W), argmax.data_ptr(),
+                                           int(pool), out.data_ptr(), _stream()))
+    return out
 
 
 def csr_gemm_bias_maxout(S, B, v, pool):

@@ -763,6 +763,25 @@ __global__ __launch_bounds__(256) void splitk_reduce_bias_maxout_kernel(const fl
     }
 }
 
+// The chunk sum with the backward step of a maxout layer behind it: out (M x N pool) receives the summed error
+// of a pooled unit in its winner's column and zero in the others.
+__global__ __launch_bounds__(256) void splitk_reduce_expand_kernel(const float *__restrict__ partial, int splits, int64_t M,
+                                                                   int64_t N, const float *__restrict__ argmax, int pool,
+                                                                   float *__restrict__ out) {
+    const int64_t plane = M * N, cols = N * pool, total = M * cols;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / cols, c = i % cols, o = c / pool;
+        float v = 0.0f;
+        if ((int64_t)argmax[r * N + o] == c) {
+            const float *src = partial + r * N + o;
+            float s = src[0];
+            for (int k = 1; k < splits; ++k) s += src[k * plane];
+            v = s;
+        }
+        out[i] = v;
+    }
+}
+
 __global__ void set_word_kernel(uint32_t *p, uint32_t value) {
     if (threadIdx.x == 0) *p = value;
 }
@@ -817,17 +836,23 @@ static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, 
 static int g_force_tile_n = 0;
 static bool g_wide_store = true;
 
-// Bias and maxout behind the product (the forward pass of a maxout layer): the product itself is not returned.
+// What follows the product instead of its delivery: bias and maxout (the forward pass of a maxout layer; `bias`
+// given, out and argmax M x N / pool), or the expansion of a pooled error to the winners' columns (its backward
+// pass; `bias` NULL, `argmax` M x N is read, out M x N pool).  All contiguous.
 struct BiasMaxout {
     const float *bias;
     int pool;
-    float *out, *argmax;  // M x N / pool, contiguous
+    float *out, *argmax;
 };
 
 static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_t K, const float *A,
                            int64_t lda, const void *B, int64_t ldb, float scale, float *C, int64_t ldc,
                            float *absmax_out, void *stream, const BiasMaxout *then = nullptr) {
-    const char *who = then ? "gemm_f32_bias_maxout" : (w8 ? "gemm_f32_w8" : "gemm_f32");
+    const char *who = then ? (then->bias ? "gemm_f32_bias_maxout" : "gemm_f32_expand_maxout_grad") : (w8 ? "gemm_f32_w8" : "gemm_f32");
+    auto finish_from = [&](const float *product) -> cn_status {  // `product` M x N contiguous
+        if (then->bias) return cn_bias_maxout_f32(product, N, then->bias, M, N, then->pool, then->out, then->argmax, stream);
+        return cn_expand_to_maxout_grad_f32(product, then->argmax, M, N, then->pool, then->out, stream);
+    };
     if (M < 0 || N < 0 || K < 0) { set_error("%s: negative dimension", who); return CN_ERR_SHAPE; }
     if (lda < (ta ? M : K) || ldb < (tb ? K : N) || ldc < N) {
         set_error("%s: leading dimension too small (lda %lld, ldb %lld, ldc %lld for M %lld N %lld K %lld)",
@@ -860,7 +885,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         }
         hipLaunchKernelGGL(zero_matrix_kernel, dim3(ctx->num_cu * 4), dim3(256), 0, st, C, M, N, ldc);
         CN_HIP(hipGetLastError());
-        if (then) return cn_bias_maxout_f32(C, N, then->bias, M, N, then->pool, then->out, then->argmax, stream);
+        if (then) return finish_from(C);
         return CN_OK;
     }
     GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->workspace_bytes, g_force_tile_n);
@@ -902,10 +927,16 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     if (s != CN_OK) return s;
 
     if (then) {
-        if (plan.splits == 1) return cn_bias_maxout_f32(C, N, then->bias, M, N, then->pool, then->out, then->argmax, stream);
-        const int64_t work = M * (N / then->pool), blocks = (work + 255) / 256, cap = (int64_t)ctx->num_cu * 8;
-        hipLaunchKernelGGL(splitk_reduce_bias_maxout_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, st,
-                           (const float *)ctx->workspace, plan.splits, M, N, then->bias, then->pool, then->out, then->argmax);
+        if (plan.splits == 1) return finish_from(C);
+        const int64_t work = then->bias ? M * (N / then->pool) : M * N * then->pool;
+        const int64_t blocks = (work + 255) / 256, cap = (int64_t)ctx->num_cu * 8;
+        const dim3 grid((unsigned)(blocks < cap ? blocks : cap));
+        if (then->bias)
+            hipLaunchKernelGGL(splitk_reduce_bias_maxout_kernel, grid, dim3(256), 0, st, (const float *)ctx->workspace,
+                               plan.splits, M, N, then->bias, then->pool, then->out, then->argmax);
+        else
+            hipLaunchKernelGGL(splitk_reduce_expand_kernel, grid, dim3(256), 0, st, (const float *)ctx->workspace, plan.splits,
+                               M, N, (const float *)then->argmax, then->pool, then->out);
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
@@ -949,6 +980,15 @@ cn_status cn_gemm_f32_bias_maxout(int trans_a, int trans_b, int64_t M, int64_t N
     }
     if (M > 0 && N > 0 && (!bias || !out || !argmax)) { set_error("gemm_f32_bias_maxout: NULL pointer"); return CN_ERR_NULL; }
     const BiasMaxout then{bias, pool, out, argmax};
+    return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, nullptr, N, nullptr, stream, &then);
+}
+
+cn_status cn_gemm_f32_expand_maxout_grad(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A,
+                                         int64_t lda, const float *B, int64_t ldb, const float *argmax, int pool, float *out,
+                                         void *stream) {
+    if (pool < 1) { set_error("gemm_f32_expand_maxout_grad: pool size below 1"); return CN_ERR_SHAPE; }
+    if (M > 0 && N > 0 && (!argmax || !out)) { set_error("gemm_f32_expand_maxout_grad: NULL pointer"); return CN_ERR_NULL; }
+    const BiasMaxout then{nullptr, pool, out, const_cast<float *>(argmax)};
     return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, nullptr, N, nullptr, stream, &then);
 }
 

@@ -52,9 +52,9 @@ def backward(X, onehot, params, p, cache, pool=2, absmax_out=None, defer_first=F
     m1, m2, m3 = absmax_out if absmax_out is not None else (None, None, None)
     e3 = L.sub(p, onehot)
     gW3 = L.Tdot(h2, e3, absmax_out=m3)
-    e2 = L.expand_to_maxout_grad(L.dotT(e3, W3), a2, pool)
+    e2 = L.dotT_expand_to_maxout_grad(e3, W3, a2, pool)
     gW2 = L.Tdot(h1, e2, absmax_out=m2)
-    e1 = L.expand_to_maxout_grad(L.dotT(e2, W2), a1, pool)
+    e1 = L.dotT_expand_to_maxout_grad(e2, W2, a1, pool)
     if isinstance(X, SparseInput) and defer_first:
         gW1 = e1
     elif isinstance(X, SparseInput):

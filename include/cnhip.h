@@ -280,6 +280,13 @@ cn_status cn_add_row_vector_f32(const float *A_device, const float *v_device, in
 cn_status cn_gemm_f32_bias_maxout(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A_device,
                                   int64_t lda, const float *B_device, int64_t ldb, const float *bias_device, int pool,
                                   float *out_device, float *argmax_device, void *stream);
+/* out = expand_to_maxout_grad(op(A) op(B), argmax): cn_gemm_f32 and cn_expand_to_maxout_grad_f32 as one call, the
+ * backward pass through a maxout layer (source/Layer.cpp:318-321 with source/basicOps.cu:1315-1321): the error of the
+ * pooled units, M x N, lands in the winners' columns of out, M x N pool, zero elsewhere.  Rides on the chunk sum
+ * like cn_gemm_f32_bias_maxout; same bits as the two calls. */
+cn_status cn_gemm_f32_expand_maxout_grad(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
+                                         const float *A_device, int64_t lda, const float *B_device, int64_t ldb,
+                                         const float *argmax_device, int pool, float *out_device, void *stream);
 /* out, argmax = maxout(A + v) as cn_add_row_vector_f32 followed by cn_maxout_f32 give them, in one pass and
  * without the sum in memory (A with leading dimension lda; out and argmax rows x cols/pool, contiguous).
  * The bias-and-maxout step behind every dot of the forward pass, source/Layer.cpp:256-258. */

@@ -99,6 +99,31 @@ def test_product_with_bias_and_maxout_equals_the_three_calls(dev, M, N, K, pool)
     assert cn.lib().cn_gemm_f32_bias_maxout(0, 0, 4, 6, 4, None, 4, None, 6, None, 2, None, None, None) == 1  # NULL
 
 
+@pytest.mark.parametrize("M,N,K,pool", [(128, 4096, 8192, 2), (128, 4096, 10, 2), (7, 5, 33, 3), (300, 130, 64, 4),
+                                        (1, 1, 1, 1), (32, 512, 4096, 2)])
+def test_product_with_expansion_equals_the_two_calls(dev, M, N, K, pool):
+    """dotT and expand_to_maxout_grad as one call (the expansion rides on the chunk sum, or follows the product
+    through the workspace): the same bits as the two calls on every tile geometry."""
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev).manual_seed(M * 3 + N + K)
+    E = torch.randn((M, K), device=dev, generator=gen)
+    W = torch.randn((N, K), device=dev, generator=gen) * 0.05
+    winners = (torch.arange(N, device=dev) * pool)[None, :] + torch.randint(0, pool, (M, N), device=dev, generator=gen)
+    argmax = winners.to(torch.float32)
+    for force in (0, 32, 64, 128, 256):
+        cn.lib().cn_host_force_gemm_tile_n(force)
+        try:
+            got = L.dotT_expand_to_maxout_grad(E, W, argmax, pool)
+            want = L.expand_to_maxout_grad(L.dotT(E, W), argmax, pool)
+        finally:
+            cn.lib().cn_host_force_gemm_tile_n(0)
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32)), force
+    assert cn.lib().cn_gemm_f32_expand_maxout_grad(0, 1, 4, 6, 4, None, 4, None, 4, None, 0, None, None) == 2
+    assert cn.lib().cn_gemm_f32_expand_maxout_grad(0, 1, 4, 6, 4, None, 4, None, 4, None, 2, None, None) == 1
+
+
 def _cpu_step(X, onehot, params, rate, pool):
     W1, b1, W2, b2, W3, b3 = params
     z1 = oracle.add_row_vector(oracle.gemm(X, W1), b1)
