@@ -620,13 +620,19 @@ __global__ void preset_word_kernel(uint32_t *p, uint32_t value) {
 // times.  Whether the second use finds the data in the L2 depends on how much is fetched in between:
 // the rows walk their nonzeros at about the same pace, some 2000 rows of B apart, so a B row comes back
 // after about 2000 other rows have been read.  With 1024 columns per workgroup that is 8 MB, twice an XCD's
-// L2.  Here a wavefront takes one row and a strip of 256 columns (1 KB of a B row) with sixteen B rows in
+// L2.  Here a wavefront takes one row and a strip of 256 columns (1 KB of a B row) with forty B rows in
 // flight, and all rows of a strip run on one XCD (workgroup index mod 8).  Measured on the 128 x 100000
-// batch against 100000 x 8192 weights: 0.90 ms instead of 1.06 ms, 6.7 GB fetched instead of 7.55 GB
-// (holding an XCD to one strip at a time brings that to 5.1 GB but leaves too few loads in flight to gain).
+// batch against 100000 x 8192 weights: 0.86 ms instead of 1.06 ms (0.90 ms with sixteen in flight, when
+// 6.7 GB were fetched instead of 7.55 GB; holding an XCD to one strip at a time brought that to 5.1 GB but
+// left too few loads in flight to gain).
 // Sums and results as in csr_gemm_kernel.
 constexpr int kStripColumns = 256;
-constexpr int kStripGather = 16;
+// Forty B rows in flight per wavefront.  That takes 215 registers, so a SIMD holds two wavefronts and an XCD
+// works on two strips at a time instead of four: deeper queues and a smaller working set in its L2 (0.86 ms
+// against 0.90 ms with sixteen in flight and every workgroup resident; 32 at the same occupancy is slower
+// than either, 56 and more spill).  What a multiple of forty leaves over goes eight at a time.
+constexpr int kStripGather = 40;
+constexpr int kStripGatherTail = 8;
 
 // kPool 0: out = S B (and optionally max |out|).  kPool 2 or 4: out = maxout(S B + bias) over kPool
 // consecutive columns, argmax = the winner's column as a float (first maximum wins): what add_row_vector
@@ -659,6 +665,17 @@ __global__ __launch_bounds__(kT) void csr_gemm_strip_kernel(int64_t R, int64_t N
             for (int u = 0; u < kStripGather; ++u) b[u] = *reinterpret_cast<const f32x4 *>(Bn + (int64_t)c[u] * ldb);
 #pragma unroll
             for (int u = 0; u < kStripGather; ++u) acc = acc + v[u] * b[u];
+        }
+        for (; j + kStripGatherTail <= j1; j += kStripGatherTail) {
+            int32_t c[kStripGatherTail];
+            float v[kStripGatherTail];
+            f32x4 b[kStripGatherTail];
+#pragma unroll
+            for (int u = 0; u < kStripGatherTail; ++u) { c[u] = col_idx[j + u]; v[u] = vals[j + u]; }
+#pragma unroll
+            for (int u = 0; u < kStripGatherTail; ++u) b[u] = *reinterpret_cast<const f32x4 *>(Bn + (int64_t)c[u] * ldb);
+#pragma unroll
+            for (int u = 0; u < kStripGatherTail; ++u) acc = acc + v[u] * b[u];
         }
         for (; j < j1; ++j) {
             const float v = vals[j];
