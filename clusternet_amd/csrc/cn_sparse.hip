@@ -647,7 +647,9 @@ __global__ __launch_bounds__(kT) void csr_gemm_strip_kernel(int64_t R, int64_t N
                                                             int64_t lda) {
     uint32_t amax = 0;
     const int64_t xcd = blockIdx.x % 8, local = blockIdx.x / 8;
-    const int64_t strip = (local / row_quads) * 8 + xcd;
+    // an XCD takes neighbouring strips, so that the two it has in flight read neighbouring kilobytes of the same
+    // B rows (0.82 ms instead of 0.845 ms with its strips eight apart)
+    const int64_t strip = xcd * ((strips + 7) / 8) + (local / row_quads);
     const int64_t r = (local % row_quads) * 4 + (threadIdx.x >> 6);
     const int64_t n = strip * kStripColumns + 4 * (int64_t)(threadIdx.x & 63);
     if (strip < strips && r < R && n < N) {
