@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/cnhip.h"
+#include "../../include/cnhip_hooks.h"
 
 namespace cn {
 

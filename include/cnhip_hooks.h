@@ -1,0 +1,57 @@
+/* libcnhip: host-side test and tuning hooks.
+ *
+ * None of these has a counterpart in the reference and none belongs to the drop-in surface of cnhip.h:
+ * they let the tests reach the library's host logic without a GPU (the work decomposition of a product,
+ * the encoder's bucket table evaluated on the CPU exactly as a workgroup evaluates it) and let tests and
+ * benchmarks pin a kernel choice that the library otherwise makes by itself.  The switches are process-wide
+ * and not synchronised: set them while no call of the library is in flight.
+ */
+#ifndef CNHIP_HOOKS_H
+#define CNHIP_HOOKS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* The decomposition cn_gemm_f32 would choose for an M x N x K product on `num_cu` compute units with
+ * `workspace_bytes` of partial-sum memory.  force_tile_n as in cn_host_force_gemm_tile_n.
+ * out = { tiles_m, tiles_n, k_iters, splits, iters_per_split, units, tile_n, tile_m }. */
+void cn_host_plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n,
+                       int64_t out[8]);
+
+/* 0 = the planner chooses the tile; 128 / 256 = that width of the 128-row tile; 32 / 64 = the 32 x 128 /
+ * 64 x 128 tile.  Any other value means 0. */
+void cn_host_force_gemm_tile_n(int tile_n);
+
+/* 0 = every output tile is written with 4-byte stores (the path that unaligned outputs take). */
+void cn_host_gemm_wide_store(int enabled);
+
+/* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
+void cn_host_codec_workgroups_per_cu(int per_cu);
+
+/* 0 = sparse products never take the strip kernel (few long rows) / the kernel that keeps a strip of B in
+ * LDS (maximum only); they then run on the general kernels, which the tests compare against. */
+void cn_host_csr_strip_kernel(int enabled);
+void cn_host_csr_lds_rows(int enabled);
+
+/* The encoder's bucket table on the host.  cn_host_xlut_entries: number of 8-byte entries of a table;
+ * cn_host_xlut_step_count: number of steps of the code function found at precision 1;
+ * cn_host_xlut_build: fills entries[cn_host_xlut_entries()] and *first for `precision` the way a workgroup
+ * does, returns 1 if the table must not be used for this precision (the encoder then runs the literal
+ * procedure per element), else 0;
+ * cn_host_xlut_encode_many: codes of x[0..n) as the device computes them, returns 1 if the table was used;
+ * cn_host_encode_exact: the literal procedure (division and pivot search) for one value. */
+int cn_host_xlut_entries(void);
+int cn_host_xlut_step_count(void);
+int cn_host_xlut_build(float precision, void *entries, uint32_t *first);
+int cn_host_xlut_encode_many(float precision, const float *x, size_t n, uint8_t *codes);
+int cn_host_encode_exact(float x, float precision);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CNHIP_HOOKS_H */

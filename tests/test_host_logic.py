@@ -16,13 +16,19 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_every_declared_symbol_is_exported():
-    hdr = open(os.path.join(ROOT, "include", "cnhip.h")).read()
+    inc = os.path.join(ROOT, "include")
+    hdr = "".join(open(os.path.join(inc, f)).read() for f in sorted(os.listdir(inc)) if f.endswith(".h"))
     names = set(re.findall(r"\b(cn_[a-z0-9_]+)\s*\(", hdr))
     assert {"cn_gemm_f32", "cn_gemm_f32_w8", "cn_compress_8bit", "cn_decompress_8bit",
             "cn_absmax_f32", "cn_init"} <= names
     L = cn.lib()
     for n in sorted(names):
         assert hasattr(L, n), n
+    # and nothing is exported that no header declares
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", L._name], capture_output=True, text=True, check=True).stdout
+    exported = {l.split()[2] for l in out.splitlines() if len(l.split()) == 3 and l.split()[1] == "T" and l.split()[2].startswith("cn_")}
+    assert exported <= names, sorted(exported - names)
 
 
 def test_no_device_is_reported_not_hidden():
