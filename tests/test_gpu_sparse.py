@@ -98,7 +98,7 @@ def test_gather_product_is_bit_exact(dev, R, Cc, N, density):
 
 
 @pytest.mark.parametrize("R,Cc,N,density", [(128, 3000, 4096, 0.02), (100, 700, 2052, 0.1), (3, 50, 2048, 0.5),
-                                            (128, 64, 8192, 1.0)])
+                                            (128, 64, 8192, 1.0), (64, 500, 2820, 0.05), (128, 200, 4612, 0.03)])
 def test_few_long_rows_take_the_strip_kernel_with_the_same_bits(dev, R, Cc, N, density):
     """Few rows and many columns run one column strip per L2 at a time; same sums, same bits, also with
     the maximum."""
