@@ -326,3 +326,51 @@ def test_coded_entries_report_bad_arguments_and_handle_empty_matrices(dev):
     got = L.csr_gemm_coded_update(Z, B, one, w=w, alpha=0.5)
     assert int(got.min()) == 254 and int(got.max()) == 254
     assert torch.equal(w, torch.full((40, 64), 0.5, device=dev))
+
+
+@pytest.mark.parametrize("seed", [5, 6])
+def test_random_shapes_of_every_kernel_choice(dev, seed):
+    """Shapes drawn at random over the three dispatch regimes (few long rows, many short rows, neither):
+    product with maximum, maximum alone, bias + maxout in one call, codes with the weight update, each
+    bit for bit against the checker."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(seed)
+    for it in range(18):
+        if it % 3 == 0:
+            R, Cc = int(rng.integers(1, 129)), int(rng.integers(1, 1500))
+            N = int(rng.choice([2048, 2052, 2304, 2820, 4100, 4612]))
+            density = float(rng.choice([0.01, 0.05, 0.3]))
+        elif it % 3 == 1:
+            R, Cc, N = int(rng.integers(1, 3000)), int(rng.integers(1, 129)), int(rng.integers(1, 1200))
+            density = float(rng.choice([0.0, 0.02, 0.1, 0.5]))
+        else:
+            R, Cc, N = int(rng.integers(1, 300)), int(rng.integers(1, 300)), int(rng.integers(1, 2500))
+            density = float(rng.choice([0.02, 0.2]))
+        case = "seed %d case %d: %d x %d times %d x %d, density %g" % (seed, it, R, Cc, Cc, N, density)
+        S_dense = (rng.normal(0, 1, (R, Cc)) * (rng.random((R, Cc)) < density)).astype(np.float32)
+        B = rng.normal(0, 1, (Cc, N)).astype(np.float32)
+        S, Bd = L.csr_from_dense(_t(S_dense, dev)), _t(B, dev)
+        want = oracle.csr_gemm(oracle.csr_from_dense(S_dense), B)
+        peak = float(oracle.absmax(want))
+        amax = torch.zeros(1, device=dev)
+        got = L.csr_gemm(S, Bd, absmax_out=amax).cpu().numpy()
+        assert np.array_equal(_bits(got), _bits(want)), case
+        assert float(amax.cpu()[0]) == peak, case
+        assert float(L.csr_gemm_absmax(S, Bd).cpu()[0]) == peak, case
+        pools = [p for p in (2, 3, 4) if N % p == 0]
+        if pools:
+            pool = pools[it % len(pools)]
+            v = rng.normal(0, 1, N).astype(np.float32)
+            out, arg = L.csr_gemm_bias_maxout(S, Bd, _t(v, dev), pool)
+            want_out, want_arg = oracle.maxout(oracle.add_row_vector(want, v), pool)
+            assert np.array_equal(_bits(out.cpu().numpy()), _bits(want_out)), case
+            assert np.array_equal(arg.cpu().numpy(), want_arg), case
+        if peak > 0:
+            w0 = rng.normal(0, 1, (R, N)).astype(np.float32)
+            w = _t(w0.copy(), dev)
+            codes = L.csr_gemm_coded_update(S, Bd, torch.full((1,), peak, device=dev), w=w, alpha=-0.01).cpu().numpy()
+            want_codes = np.asarray(oracle.compress(want, np.float32(peak))).reshape(R, N)
+            assert np.array_equal(codes, want_codes), case
+            want_w = oracle.decompress_axpy(want_codes, np.float32(peak), np.float32(-0.01), w0)
+            assert np.array_equal(_bits(w.cpu().numpy()), _bits(np.asarray(want_w).reshape(R, N))), case
