@@ -37,14 +37,26 @@ constexpr int64_t kSegment = 4096;
 
 // counts[r * segments + g] = nonzeros of columns [g kSegment, (g + 1) kSegment) of row r; one workgroup
 // per (row, segment).
+template <bool kVec>  // kVec: every row segment starts on a 16-byte boundary
 __global__ __launch_bounds__(kT) void count_segments_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
                                                             int64_t lda, int64_t segments, int32_t *__restrict__ counts) {
     __shared__ int partial[kT / 64];
     for (int64_t unit = blockIdx.x; unit < rows * segments; unit += gridDim.x) {
         const int64_t r = unit / segments, j0 = (unit % segments) * kSegment;
         const int64_t j1 = (j0 + kSegment < cols) ? j0 + kSegment : cols;
+        const float *row = A + r * lda;
         int c = 0;
-        for (int64_t j = j0 + threadIdx.x; j < j1; j += kT) c += (A[r * lda + j] != 0.0f) ? 1 : 0;
+        int64_t j = j0 + threadIdx.x;
+        if (kVec) {
+            const f32x4 *v4 = reinterpret_cast<const f32x4 *>(row + j0);
+            const int nv = (int)((j1 - j0) >> 2);
+            for (int i = threadIdx.x; i < nv; i += kT) {
+                const f32x4 v = v4[i];
+                c += ((v.x != 0.0f) ? 1 : 0) + ((v.y != 0.0f) ? 1 : 0) + ((v.z != 0.0f) ? 1 : 0) + ((v.w != 0.0f) ? 1 : 0);
+            }
+            j = j0 + 4 * (int64_t)nv + threadIdx.x;
+        }
+        for (; j < j1; j += kT) c += (row[j] != 0.0f) ? 1 : 0;
         for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
         if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = c;
         __syncthreads();
@@ -149,34 +161,57 @@ __global__ __launch_bounds__(kT) void block_scan_kernel(const int32_t *counts, i
 }
 
 // CSR of A: one workgroup per (row, segment), columns compacted in ascending order from the
-// segment's offset.
+// segment's offset.  A thread owns sixteen consecutive columns (four 16-byte loads when kVec says that
+// every row segment starts on a 16-byte boundary), counts its nonzeros, takes its place from a scan over the
+// workgroup and writes them out in order: one pass and two barriers per segment.
+static_assert(kSegment == 16 * kT, "a thread owns sixteen columns of a segment");
+template <bool kVec>
 __global__ __launch_bounds__(kT) void fill_segments_kernel(const float *__restrict__ A, int64_t rows, int64_t cols,
                                                            int64_t lda, int64_t segments,
                                                            const int32_t *__restrict__ offsets,
                                                            int32_t *__restrict__ col_idx, float *__restrict__ vals) {
     __shared__ int wave_count[kT / 64];
-    __shared__ int base;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int64_t unit = blockIdx.x; unit < rows * segments; unit += gridDim.x) {
         const int64_t r = unit / segments, s0 = (unit % segments) * kSegment;
         const int64_t s1 = (s0 + kSegment < cols) ? s0 + kSegment : cols;
-        if (threadIdx.x == 0) base = offsets[unit];
-        __syncthreads();
-        for (int64_t j0 = s0; j0 < s1; j0 += kT) {
-            const int64_t j = j0 + threadIdx.x;
-            const float v = (j < s1) ? A[r * lda + j] : 0.0f;
-            const bool keep = v != 0.0f;
-            const unsigned long long mask = __ballot(keep);
-            const int before = __popcll(mask & ((1ull << lane) - 1ull));
-            if (lane == 0) wave_count[wave] = __popcll(mask);
-            __syncthreads();
-            int offset = base + before;
-            for (int w = 0; w < wave; ++w) offset += wave_count[w];
-            if (keep) { col_idx[offset] = (int32_t)j; vals[offset] = v; }
-            __syncthreads();
-            if (threadIdx.x == 0) base += wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
-            __syncthreads();
+        const float *row = A + r * lda;
+        const int64_t mine = s0 + 16 * (int64_t)threadIdx.x;
+        const int base = offsets[unit];
+        float v[16];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int64_t j = mine + 4 * q;
+            if (kVec && j + 4 <= s1) {
+                const f32x4 x = *reinterpret_cast<const f32x4 *>(row + j);
+                v[4 * q] = x.x; v[4 * q + 1] = x.y; v[4 * q + 2] = x.z; v[4 * q + 3] = x.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[4 * q + e] = (j + e < s1) ? row[j + e] : 0.0f;
+            }
         }
+        uint32_t keep = 0;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) keep |= (v[e] != 0.0f) ? (1u << e) : 0u;
+        const int count = __popc(keep);
+        int inc = count;  // inclusive scan within the wavefront
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int up = __shfl_up(inc, off, 64);
+            if (lane >= off) inc += up;
+        }
+        if (lane == 63) wave_count[wave] = inc;
+        __syncthreads();
+        int at = base + inc - count;
+        for (int w = 0; w < wave; ++w) at += wave_count[w];
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            if (keep & (1u << e)) {
+                col_idx[at] = (int32_t)(mine + e);
+                vals[at] = v[e];
+                ++at;
+            }
+        __syncthreads();
     }
 }
 
@@ -910,6 +945,7 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
     const int wide = ctx->num_cu * 8;
     const int64_t segments = (cols + kSegment - 1) / kSegment;
     const int64_t units = rows * segments;
+    const bool vec_rows = aligned(A, 16) && lda % 4 == 0;  // segments start at multiples of 4096 columns
     int32_t *offsets = reinterpret_cast<int32_t *>(ctx->workspace);  // per (row, segment), transpose == 0 only
     if (!transpose && (size_t)(units + 1) * sizeof(int32_t) > ctx->workspace_bytes) {
         set_error("csr_from_dense_f32: matrix too large for the workspace");
@@ -922,8 +958,8 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
         CN_HIP(hipGetLastError());
         { cn_status sc = exclusive_scan(ctx, row_ptr, out_rows, row_ptr, total_dev, st); if (sc != CN_OK) return sc; }
     } else if (rows > 0 && cols > 0) {
-        hipLaunchKernelGGL(count_segments_kernel, dim3((unsigned)(units < wide ? units : wide)), dim3(kT), 0, st, A, rows, cols,
-                           lda, segments, offsets);
+        hipLaunchKernelGGL(vec_rows ? count_segments_kernel<true> : count_segments_kernel<false>,
+                           dim3((unsigned)(units < wide ? units : wide)), dim3(kT), 0, st, A, rows, cols, lda, segments, offsets);
         CN_HIP(hipGetLastError());
         { cn_status sc = exclusive_scan(ctx, offsets, units, offsets, total_dev, st); if (sc != CN_OK) return sc; }
         const int64_t blocks = (rows + kT) / kT;
@@ -950,8 +986,9 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
         hipLaunchKernelGGL(fill_cols_kernel, dim3((unsigned)(blocks < wide ? blocks : wide)), dim3(kT), 0, st, A, rows, cols,
                            lda, row_ptr, col_idx, vals);
     } else {
-        hipLaunchKernelGGL(fill_segments_kernel, dim3((unsigned)(units < wide ? units : wide)), dim3(kT), 0, st, A, rows, cols,
-                           lda, segments, offsets, col_idx, vals);
+        hipLaunchKernelGGL(vec_rows ? fill_segments_kernel<true> : fill_segments_kernel<false>,
+                           dim3((unsigned)(units < wide ? units : wide)), dim3(kT), 0, st, A, rows, cols, lda, segments, offsets,
+                           col_idx, vals);
     }
     CN_HIP(hipGetLastError());
     return CN_OK;
