@@ -374,3 +374,31 @@ def test_random_shapes_of_every_kernel_choice(dev, seed):
             assert np.array_equal(codes, want_codes), case
             want_w = oracle.decompress_axpy(want_codes, np.float32(peak), np.float32(-0.01), w0)
             assert np.array_equal(_bits(w.cpu().numpy()), _bits(np.asarray(want_w).reshape(R, N))), case
+
+
+@pytest.mark.parametrize("seed", [1, 2])
+def test_dense_to_csr_on_random_shapes_strides_and_alignments(dev, seed):
+    """The conversion reads rows with 16-byte loads when the base and the leading dimension allow it and
+    element by element otherwise: shapes, paddings and one-element offsets drawn at random, segments that
+    end inside a vector, each against the checker's arrays."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(100 + seed)
+    for it in range(24):
+        rows = int(rng.integers(1, 40))
+        cols = int(rng.choice([1, 3, 4, 5, 63, 64, 255, 256, 257, 4095, 4096, 4097, 4100, 8191, 8192, 9001, 12289]))
+        pad = int(rng.choice([0, 0, 1, 3, 4, 8]))
+        shift = int(rng.choice([0, 0, 1, 2]))
+        density = float(rng.choice([0.0, 0.01, 0.1, 0.6, 1.0]))
+        case = "seed %d case %d: %d x %d, pad %d, shift %d, density %g" % (seed, it, rows, cols, pad, shift, density)
+        A = (rng.normal(0, 1, (rows, cols)) * (rng.random((rows, cols)) < density)).astype(np.float32)
+        A[rng.random((rows, cols)) < 0.01] = -0.0  # a negative zero is no nonzero
+        store = torch.zeros(rows * (cols + pad) + shift, device=dev)
+        view = store[shift:].view(rows, cols + pad)[:, :cols]
+        view.copy_(_t(A, dev))
+        for transpose in (False, True):
+            S = L.csr_from_dense(view, transpose=transpose)
+            rp, ci, va = oracle.csr_from_dense(A, transpose=transpose)
+            assert np.array_equal(S.row_ptr.cpu().numpy(), rp), case
+            assert np.array_equal(S.col_idx.cpu().numpy(), ci), case
+            assert np.array_equal(_bits(S.vals.cpu().numpy()), _bits(va)), case
