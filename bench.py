@@ -10,7 +10,7 @@ against the fp32 matrix-core peak.  After the timed region the codec kernels (co
 decompression_8bit, absmax) and the fused 8-bit-weight GEMM are measured on their own workloads and
 reported under "extra"; the CPU port of the same arithmetic is timed on a bounded sample.
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|codec|fused] [--no-cpu]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|codec|fused|step] [--no-cpu] [--zero-operands]
 """
 import argparse
 import json
@@ -91,11 +91,18 @@ def time_replayed(torch, fn, calls, replays):
         return None
 
 
-def bench_gemm(torch, cn, dev, steps, warmup):
+def bench_gemm(torch, cn, dev, steps, warmup, zeros=False):
     gen = torch.Generator(device=dev).manual_seed(1234)
-    batch = torch.rand((M, K1), device=dev, generator=gen)
-    W1 = make_uniform(torch, (K1, N1), (6.0 / (K1 + N1)) ** 0.5, dev, gen)
-    W2 = make_uniform(torch, (N1, N2), (6.0 / (N1 + N2)) ** 0.5, dev, gen)
+    if zeros:
+        # same kernels, same schedule, no switching activity in the operands: separates what the code
+        # can issue from what the part sustains under the power of real data
+        batch = torch.zeros((M, K1), device=dev)
+        W1 = torch.zeros((K1, N1), device=dev)
+        W2 = torch.zeros((N1, N2), device=dev)
+    else:
+        batch = torch.rand((M, K1), device=dev, generator=gen)
+        W1 = make_uniform(torch, (K1, N1), (6.0 / (K1 + N1)) ** 0.5, dev, gen)
+        W2 = make_uniform(torch, (N1, N2), (6.0 / (N1 + N2)) ** 0.5, dev, gen)
     out1 = torch.empty((M, N1), device=dev)
     out2 = torch.empty((M, N2), device=dev)
 
@@ -381,6 +388,8 @@ def main():
     ap.add_argument("--only", choices=["gemm", "codec", "fused", "step"], default=None,
                     help="run one part only (for profiling); prints a reduced JSON line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--zero-operands", action="store_true",
+                    help="profiling aid: the two products run on all-zero operands (the line is marked; not a result)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build runs the un-sharded workload on a single "
@@ -413,7 +422,9 @@ def main():
                 pass
 
     if args.only in (None, "gemm"):
-        g = bench_gemm(torch, cn, dev, args.steps, args.warmup)
+        g = bench_gemm(torch, cn, dev, args.steps, args.warmup, zeros=args.zero_operands)
+        if args.zero_operands:
+            line["data"] = "all-zero operands (profiling aid, not a result)"
         line["value"] = (FLOP1 + FLOP2) / (g["wall_ms"] * 1e-3) / 1e12
         line["ms_per_step"] = g["wall_ms"]
         achieved = FLOP1 / (g["gemm1_ms"] * 1e-3) / 1e12
