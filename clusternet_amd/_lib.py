@@ -45,6 +45,7 @@ def lib():
     L.cn_synchronize.argtypes = [vp]
     L.cn_table_get.argtypes = [C.POINTER(f32)]
     L.cn_gemm_f32.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp]
+    L.cn_gemm_f32_noalloc.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp]
     L.cn_gemm_f32_absmax.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, vp]
     L.cn_gemm_f32_w8.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, vp, i64, vp]
     L.cn_csr_from_dense_f32.argtypes = [vp, i64, i64, i64, C.c_int, vp, vp, vp, i64, C.POINTER(i64), vp]
@@ -120,9 +121,10 @@ def _ld(t):
     return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
 
 
-def gemm(A, B, trans_a=False, trans_b=False, out=None, absmax_out=None):
+def gemm(A, B, trans_a=False, trans_b=False, out=None, absmax_out=None, noalloc=False):
     """out = op(A) op(B) on row-major fp32 matrices; mirrors ClusterNet::dot(A,B,out,T1,T2).
-    `absmax_out` (one-element fp32 device tensor) additionally receives max|out|."""
+    `absmax_out` (one-element fp32 device tensor) additionally receives max|out|.
+    `noalloc` (needs `out`): the entry point that allocates nothing, cn_gemm_f32_noalloc."""
     import torch
     _need(A, torch.float32, "A")
     _need(B, torch.float32, "B")
@@ -134,7 +136,10 @@ def gemm(A, B, trans_a=False, trans_b=False, out=None, absmax_out=None):
     if K != K2 or tuple(out.shape) != (M, N):
         raise CnError(2, "Matrix size error: op(A) %dx%d, op(B) %dx%d, out %dx%d"
                       % (M, K, K2, N, out.shape[0], out.shape[1]))
-    if absmax_out is not None:
+    if noalloc:
+        check(lib().cn_gemm_f32_noalloc(int(trans_a), int(trans_b), M, N, K, A.data_ptr(), _ld(A), B.data_ptr(),
+                                        _ld(B), out.data_ptr(), _ld(out), _stream()))
+    elif absmax_out is not None:
         _need(absmax_out, torch.float32, "absmax_out")
         check(lib().cn_gemm_f32_absmax(int(trans_a), int(trans_b), M, N, K, A.data_ptr(), _ld(A), B.data_ptr(),
                                        _ld(B), out.data_ptr(), _ld(out), absmax_out.data_ptr(), _stream()))

@@ -42,6 +42,8 @@
 //     contiguous range of work units and share their A/B panels in that XCD's L2
 //   * global addresses are a uniform buffer descriptor (scalar registers) plus a 32-bit per-lane
 //     byte offset, which is why leading dimensions are limited to 2^22 elements.
+#include <mutex>
+
 #include "cn_internal.h"
 
 namespace cn {
@@ -795,16 +797,16 @@ __global__ __launch_bounds__(256) void zero_matrix_kernel(float *__restrict__ C,
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// C = sum of the `splits` M x N planes at the start of the workspace, added in ascending order;
+// C = sum of the `splits` M x N planes at `planes`, added in ascending order;
 // optionally also max |C| (see publish_absmax).
-cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float *C, int64_t ldc, uint32_t *amax,
-                           hipStream_t st) {
+cn_status add_chunk_planes(const void *planes, int num_cu, int splits, int64_t M, int64_t N, float *C, int64_t ldc,
+                           uint32_t *amax, hipStream_t st) {
     int vec = (N % 4 == 0) && (ldc % 4 == 0) && aligned(C, 16);
     int64_t work = vec ? M * (N / 4) : M * N;
     int64_t blocks = (work + 255) / 256;
-    int64_t cap = (int64_t)ctx->num_cu * 8;
+    int64_t cap = (int64_t)num_cu * 8;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)(blocks < cap ? blocks : cap)), dim3(256), 0, st,
-                       (const float *)ctx->workspace, splits, M, N, C, ldc, vec, amax);
+                       (const float *)planes, splits, M, N, C, ldc, vec, amax);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -845,10 +847,13 @@ struct BiasMaxout {
     float *out, *argmax;
 };
 
+// `env` = NULL: the current device's context (initialised on first use) supplies the workspace.
 static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_t K, const float *A,
                            int64_t lda, const void *B, int64_t ldb, float scale, float *C, int64_t ldc,
-                           float *absmax_out, void *stream, const BiasMaxout *then = nullptr) {
-    const char *who = then ? (then->bias ? "gemm_f32_bias_maxout" : "gemm_f32_expand_maxout_grad") : (w8 ? "gemm_f32_w8" : "gemm_f32");
+                           float *absmax_out, void *stream, const BiasMaxout *then = nullptr,
+                           const GemmEnv *given = nullptr) {
+    const char *who = given ? "gemm_f32_noalloc"
+                            : then ? (then->bias ? "gemm_f32_bias_maxout" : "gemm_f32_expand_maxout_grad") : (w8 ? "gemm_f32_w8" : "gemm_f32");
     auto finish_from = [&](const float *product) -> cn_status {  // `product` M x N contiguous
         if (then->bias) return cn_bias_maxout_f32(product, N, then->bias, M, N, then->pool, then->out, then->argmax, stream);
         return cn_expand_to_maxout_grad_f32(product, then->argmax, M, N, then->pool, then->out, stream);
@@ -865,9 +870,15 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     }
     if ((M == 0 || N == 0) && !absmax_out) return CN_OK;
     if ((M > 0 && N > 0) && ((!C && !then) || (K > 0 && (!A || !B)))) { set_error("%s: NULL operand", who); return CN_ERR_NULL; }
-    Context *ctx;
-    cn_status s = current_context(&ctx);
-    if (s != CN_OK) return s;
+    cn_status s = CN_OK;
+    GemmEnv from_context;
+    if (!given) {
+        Context *c;
+        s = current_context(&c);
+        if (s != CN_OK) return s;
+        from_context = GemmEnv{c->device, c->num_cu, c->workspace, c->workspace_bytes, c->workspace_bytes, c->table};
+    }
+    const GemmEnv *ctx = given ? given : &from_context;
     hipStream_t st = (hipStream_t)stream;
     // The maximum is accumulated with atomics from +0.0 (|C| >= 0); an empty C reports -1.0f, the start
     // value of the reference's reduction, like cn_absmax_f32.
@@ -888,7 +899,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         if (then) return finish_from(C);
         return CN_OK;
     }
-    GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->workspace_bytes, g_force_tile_n);
+    GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->plan_bytes, g_force_tile_n);
     if (then && plan.splits == 1) {
         // no chunk sum to fold into: the product goes to the workspace and one pass over it follows
         if ((size_t)M * (size_t)N * sizeof(float) > ctx->workspace_bytes) {
@@ -903,7 +914,9 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         return CN_ERR_SHAPE;
     }
     if (plan.splits > 1 && (size_t)plan.splits * (size_t)M * (size_t)N * sizeof(float) > ctx->workspace_bytes) {
-        set_error("%s: split-K workspace too small", who);
+        set_error("%s: the %d K-chunks of this %lld x %lld product need %zu bytes of partial sums, %zu are there%s", who,
+                  plan.splits, (long long)M, (long long)N, (size_t)plan.splits * (size_t)M * (size_t)N * sizeof(float),
+                  ctx->workspace_bytes, given ? " (the limit of this entry point; cn_gemm_f32 serves larger products)" : "");
         return CN_ERR_WORKSPACE;
     }
     GemmArgs a;
@@ -940,7 +953,36 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
-    if (plan.splits > 1) return add_chunk_planes(ctx, plan.splits, M, N, C, ldc, amax, st);
+    if (plan.splits > 1) return add_chunk_planes(ctx->workspace, ctx->num_cu, plan.splits, M, N, C, ldc, amax, st);
+    return CN_OK;
+}
+
+// ---- the product for callers that must not allocate ----------------------------------------------------------
+// Its K-chunk partial sums go to an array that is part of the library's device image instead of the workspace that
+// cn_init allocates.  In host code the array's name stands for the symbol, not for a device address: the address
+// is asked for once per device (every device holds its own copy) and only that pointer is ever handed to a kernel.
+constexpr size_t kStaticPartialBytes = (size_t)64 << 20;
+static __device__ __align__(256) float scratch[kStaticPartialBytes / sizeof(float)];
+
+struct StaticPartials {
+    float *ptr = nullptr;
+    int num_cu = 0;
+};
+static StaticPartials g_static[kMaxDevices];
+static std::mutex g_static_mutex;
+
+cn_status gemm_static_setup(int device) {
+    if (device < 0 || device >= kMaxDevices) { set_error("device %d out of range", device); return CN_ERR_NO_DEVICE; }
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    StaticPartials &sp = g_static[device];
+    if (sp.ptr) return CN_OK;
+    float *ptr = nullptr;
+    CN_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    int cus = 0;
+    CN_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device));
+    if (!ptr || cus <= 0) { set_error("gemm_f32_noalloc: the partial-sum array could not be located on device %d", device); return CN_ERR_HIP; }
+    sp.num_cu = cus;
+    sp.ptr = ptr;
     return CN_OK;
 }
 
@@ -962,6 +1004,23 @@ void cn_host_force_gemm_tile_n(int tile_n) {
 cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
                       const float *B, int64_t ldb, float *C, int64_t ldc, void *stream) {
     return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, C, ldc, nullptr, stream);
+}
+
+cn_status cn_gemm_f32_noalloc(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                              const float *B, int64_t ldb, float *C, int64_t ldc, void *stream) {
+    int device = 0;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess || device < 0 || device >= kMaxDevices) {
+        set_error("gemm_f32_noalloc: no usable HIP device (%s)", e == hipSuccess ? "index out of range" : hipGetErrorString(e));
+        return CN_ERR_NO_DEVICE;
+    }
+    if (!g_static[device].ptr) {  // first call on this device without cn_init: locate the array now
+        cn_status s = gemm_static_setup(device);
+        if (s != CN_OK) return s;
+    }
+    const GemmEnv env{device, g_static[device].num_cu, g_static[device].ptr, kStaticPartialBytes,
+                      planning_workspace_bytes(device), nullptr};
+    return gemm_impl(trans_a != 0, trans_b != 0, false, M, N, K, A, lda, B, ldb, 1.0f, C, ldc, nullptr, stream, nullptr, &env);
 }
 
 cn_status cn_gemm_f32_absmax(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A,

@@ -59,6 +59,25 @@ struct OncePerDevice {
 // Returns the context of the current device, initialising it on first use.
 cn_status current_context(Context **out);
 
+// Bytes of split-K workspace cn_init allocates (CNHIP_WORKSPACE_MB, default 1 GiB), and the figure the planner
+// sees on `device`: the context's if it is initialised, else what initialisation would allocate.
+size_t default_workspace_bytes();
+size_t planning_workspace_bytes(int device);
+
+// What a product needs from its surroundings: where its K-chunk partial sums go, how much of that there is, and
+// the workspace size the planner is told (two entry points that plan with the same figure give the same bits).
+struct GemmEnv {
+    int device;
+    int num_cu;
+    void *workspace;
+    size_t workspace_bytes;
+    size_t plan_bytes;
+    const float *table;  // codebook, fused variant only
+};
+// The partial-sum array that is part of the library's device image (cn_gemm_f32_noalloc): resolves its address
+// on `device`, which must be the current device.  No allocation.
+cn_status gemm_static_setup(int device);
+
 // ---- GEMM planning (host, pure function; exported for tests) ---------------------------------
 struct GemmPlan {
     int tile_m;          // output tile is tile_m x tile_n: 128 x 128, 128 x 256, or 32 x 128 / 64 x 128 for a handful of rows
@@ -70,8 +89,8 @@ struct GemmPlan {
 };
 // force_tile_n: 0 = choose, 128 or 256 = use that tile width, 32 / 64 = use the 32 x 128 / 64 x 128 tile.
 // C = sum of `splits` M x N planes held at the start of the workspace (ascending order); optional max |C|.
-cn_status add_chunk_planes(Context *ctx, int splits, int64_t M, int64_t N, float *C, int64_t ldc, uint32_t *amax,
-                           hipStream_t st);
+cn_status add_chunk_planes(const void *planes, int num_cu, int splits, int64_t M, int64_t N, float *C, int64_t ldc,
+                           uint32_t *amax, hipStream_t st);
 
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 

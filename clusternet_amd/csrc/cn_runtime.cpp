@@ -31,6 +31,20 @@ void host_table(float out[126]);
 static Context g_ctx[kMaxDevices];
 static std::mutex g_mutex;
 
+size_t default_workspace_bytes() {
+    size_t mib = 1024;
+    if (const char *env = getenv("CNHIP_WORKSPACE_MB")) {
+        long v = atol(env);
+        if (v >= 16) mib = (size_t)v;
+    }
+    return mib << 20;
+}
+
+size_t planning_workspace_bytes(int device) {
+    if (device >= 0 && device < kMaxDevices && g_ctx[device].ready) return g_ctx[device].workspace_bytes;
+    return default_workspace_bytes();
+}
+
 static cn_status init_device(int device) {
     int count = 0;
     hipError_t e = hipGetDeviceCount(&count);
@@ -71,12 +85,7 @@ static cn_status init_device(int device) {
         CN_HIP(hipMemcpy(c.xsteps, steps, sizeof(steps), hipMemcpyHostToDevice));
     }
 
-    size_t mib = 1024;
-    if (const char *env = getenv("CNHIP_WORKSPACE_MB")) {
-        long v = atol(env);
-        if (v >= 16) mib = (size_t)v;
-    }
-    c.workspace_bytes = mib << 20;
+    c.workspace_bytes = default_workspace_bytes();
     CN_HIP(hipMalloc(&c.workspace, c.workspace_bytes));
 
     CN_HIP(hipMalloc((void **)&c.reduce_scratch, (kReduceSlots + 64) * sizeof(uint32_t)));
@@ -84,6 +93,10 @@ static cn_status init_device(int device) {
     CN_HIP(hipMalloc((void **)&c.tickets, kTicketWords * sizeof(uint32_t)));
     CN_HIP(hipMemset(c.tickets, 0, kTicketWords * sizeof(uint32_t)));
     CN_HIP(hipMalloc((void **)&c.sum_scratch, 1024 * sizeof(double)));
+    {
+        const cn_status located = gemm_static_setup(device);
+        if (located != CN_OK) return located;
+    }
     CN_HIP(hipDeviceSynchronize());
     CN_HIP(hipSetDevice(previous));
     c.ready = true;

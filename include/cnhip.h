@@ -81,6 +81,18 @@ cn_status cn_gemm_f32(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
                       const float *A_device, int64_t lda, const float *B_device, int64_t ldb,
                       float *C_device, int64_t ldc, void *stream);
 
+/* cn_gemm_f32 for callers that cannot allocate device memory (a stream under HIP graph capture, a serving loop, a
+ * harness that forbids hipMalloc); it has no counterpart in the reference.  Same arguments, same result bit for bit
+ * (it splits K exactly as cn_gemm_f32 does on this device), but the partial sums of a split K go to a 64 MiB array
+ * that is part of the library's device image, one copy per GPU, held until the process ends, and the call performs
+ * no hipMalloc / hipFree, with or without a preceding cn_init.  A product whose K-chunks need more than 64 MiB of
+ * partial sums (chunks x M x N x 4 bytes) is refused with CN_ERR_WORKSPACE and nothing is launched.  All calls on
+ * one GPU share the array: calls that may overlap on one GPU (streams without an ordering between them) race on it.
+ * The first call on a device looks the array's address up; make that call, or cn_init, outside a capture. */
+cn_status cn_gemm_f32_noalloc(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K,
+                              const float *A_device, int64_t lda, const float *B_device, int64_t ldb,
+                              float *C_device, int64_t ldc, void *stream);
+
 /* cn_gemm_f32 that also writes max |C[i][j]| to *absmax_out_device, taken in the kernel's write-out
  * (or in the addition of the K chunks): the value equals cn_absmax_f32 over the result bit for bit
  * (-1.0f for an empty C) and saves that pass over C.  It fuses dot / Tdot with the max(abs(grad)) that
