@@ -166,21 +166,11 @@ def bench_codec(torch, cn, dev):
                         "compress_us": time_replayed(torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50),
                         "decompress_us": time_replayed(torch, lambda: cn.decompression_8bit(codes, prec_t, back), 20, 50)}
             res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
-        if n % 4096 == 0 and n >= 100000 * 8192:
-            # the same bytes moved by kernels that do no arithmetic: best of six grid sizes each
-            from clusternet_amd import _lib as L
-            sink = torch.empty(256 * 64 * L.num_compute_units(), dtype=torch.int32, device=dev)
-            yard = {}
-            for label, kind, src, dst, nbytes in (("read_4B", 0, x, sink, 4.0), ("fp32_to_byte_4B_1B", 1, x, codes, 5.0),
-                                                  ("byte_to_fp32_1B_4B", 2, codes, back, 5.0), ("copy_4B_4B", 3, x, back, 8.0)):
-                best = min(time_region(torch, lambda: L.stream_yardstick(kind, src, dst, n, per_cu), 10, 2)
-                           for per_cu in (2, 3, 4, 6, 8, 16))
-                yard[label + "_GBps"] = nbytes * n / best / 1e6
-            res[name]["arithmetic_free_streams"] = yard
-            res[name]["compress_frac_of_stream"] = res[name]["compress_GBps"] / yard["fp32_to_byte_4B_1B_GBps"]
-            res[name]["decompress_frac_of_stream"] = res[name]["decompress_GBps"] / yard["byte_to_fp32_1B_4B_GBps"]
-            res[name]["absmax_frac_of_stream"] = res[name]["absmax_GBps"] / yard["read_4B_GBps"]
-            del sink
+        if n >= 100000 * 8192:
+            # movers that are not this library's: the runtime's device-to-device copy (above) and its fill, the latter a
+            # pure write stream.  What access patterns reach on this part at all is in profiles/ (stream_sweep).
+            t_fill = time_region(torch, lambda: back.fill_(1.0), iters, warm)
+            res[name]["fill_GBps"] = 4.0 * n / t_fill / 1e6
         del x, codes, back
     return res
 

@@ -52,7 +52,6 @@ def lib():
     L.cn_csr_gemm_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp]
     L.cn_csr_transpose.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp]
     L.cn_csr_gemm_f32_absmax.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp, vp]
-    L.cn_stream_yardstick.argtypes = [C.c_int, vp, vp, sz, C.c_int, vp]
     L.cn_csr_gemm_coded_update.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, i64, f32, vp]
     L.cn_csr_gemm_coded_rmsprop.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, vp, vp, vp, i64, f32, f32, vp]
     L.cn_compress_8bit_axpy.argtypes = [vp, f32, sz, vp, f32, vp, vp]
@@ -313,11 +312,6 @@ def csr_transpose(S):
                                  t_row_ptr.data_ptr(), t_col_idx.data_ptr(), t_vals.data_ptr(), scratch.data_ptr(),
                                  _stream()))
     return Csr(S.cols, S.rows, t_row_ptr, t_col_idx[:S.nnz], t_vals[:S.nnz])
-
-
-def stream_yardstick(kind, src, dst, n, workgroups_per_cu):
-    """Launches the arithmetic-free stream kernel `kind` (0 read, 1 fp32->byte, 2 byte->fp32, 3 copy) over n elements."""
-    check(lib().cn_stream_yardstick(kind, src.data_ptr(), dst.data_ptr(), n, workgroups_per_cu, _stream()))
 
 
 def absmax(x, out=None):

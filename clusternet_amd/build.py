@@ -1,6 +1,6 @@
 """Compiles the HIP sources under clusternet_amd/csrc into clusternet_amd/libcnhip.so (gfx950).
 
-Usage: python -m clusternet_amd.build [--facade]
+Usage: python -m clusternet_amd.build [--facade] [--stream-sweep]
 The library is built in-tree so that it travels with the source tree; nothing is installed.
 """
 import os
@@ -24,7 +24,7 @@ HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-contr
              # the direct-to-LDS loads set M0 inside their inline assembly and say so
              "-Wno-inline-asm"]
 SOURCES = ["cn_runtime.cpp", "cn_encode_lut.cpp", "cn_gemm_plan.cpp", "cn_codec.hip", "cn_gemm.hip",
-           "cn_layers.hip", "cn_update.hip", "cn_sparse.hip", "cn_yardstick.hip"]
+           "cn_layers.hip", "cn_update.hip", "cn_sparse.hip"]
 
 
 def hipcc():
@@ -80,11 +80,37 @@ def build_facade(verbose=False):
     return FACADE_LIB
 
 
+def build_stream_sweep(verbose=False):
+    """The stand-alone measurement program under csrc/stream_sweep (not part of the library)."""
+    d = os.path.join(CSRC, "stream_sweep")
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    flags = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-Wno-unused-command-line-argument"]
+    procs, objs = [], []
+    for kind in range(7):
+        obj = os.path.join(objdir, "stream_sweep_kind%d.o" % kind)
+        objs.append(obj)
+        procs.append(subprocess.Popen([hipcc()] + flags + ["-DSWEEP_KIND=%d" % kind, "-c", os.path.join(d, "kind.hip"), "-o", obj],
+                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+    main_obj = os.path.join(objdir, "stream_sweep_main.o")
+    _run([hipcc()] + flags + ["-c", os.path.join(d, "main.hip"), "-o", main_obj])
+    for p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            raise RuntimeError("build failed: stream_sweep\n%s" % out)
+    exe = os.path.join(HERE, "stream_sweep")
+    _run([hipcc(), "--offload-arch=" + ARCH, "-o", exe, main_obj] + objs)
+    return exe
+
+
 def main(argv=None):
     argv = sys.argv[1:] if argv is None else argv
     print(build_library(verbose=True))
     if "--facade" in argv:
         print(build_facade(verbose=True))
+    if "--stream-sweep" in argv:
+        print(build_stream_sweep(verbose=True))
 
 
 if __name__ == "__main__":

@@ -4,6 +4,15 @@
 //   absmax      4 B read per element
 // Each lane moves 16-byte vectors laid out so that one wavefront instruction touches one
 // contiguous 1 KiB (fp32 side) / 256 B (code side) span.
+//
+// Large tensors take the *_stream_kernel forms.  What a stream that also writes reaches on this part depends
+// sharply on how many bytes a compute unit keeps in flight: about 48 KB of loads (compression) or 64 KB of stores
+// (decompression) per compute unit, one workgroup each, is the optimum; twice that, or as much again left in
+// flight by not waiting for the stores, costs 10 to 15 %.  So these kernels run one workgroup per compute unit,
+// address memory through a buffer descriptor per tile (a uniform base and a 32-bit lane offset; the descriptor's
+// range replaces the bounds test of the last tile), read with the non-temporal hint and write with it too.
+#include <type_traits>
+
 #include "cn_internal.h"
 #include "cn_xlut.h"
 #include "cn_encode_table.h"
@@ -134,6 +143,119 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
             codes[i] = (uint8_t)c;
             if (kUpdate) y[i] = y[i] + dlut[c];
         }
+    }
+}
+
+// ---- streaming forms for large tensors ---------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr int kAuxNt = 2;            // cache policy bits of the buffer instructions: nt
+constexpr int kAuxSc0Sc1Nt = 19;     // sc0 sc1 nt
+__device__ __forceinline__ rsrc_t tile_rsrc(const void *base, uint32_t bytes) {
+    // 0x00020000: 32-bit untyped data; accesses at or beyond `bytes` read zero and write nothing
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+// Compression of whole float4 groups: a tile is T * U float4, all of its loads are issued at once and awaited
+// together, then encoded and stored; the next tile's loads go out right behind the stores.  Two shapes: 256 x 12
+// (48 KiB of input per tile) with one workgroup per compute unit for tensors that stream from HBM, 512 x 10 with two
+// for tensors that the Infinity Cache can hold, where more bytes in flight pay.
+template <int T, int U>
+__global__ __launch_bounds__(T) void compress_stream_kernel(
+    const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr, size_t n,
+    uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    constexpr uint32_t kVecs = T * U;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
+    const size_t nvec = n / 4;
+    const size_t tiles = (nvec + kVecs - 1) / kVecs;
+    const uint32_t tid = threadIdx.x;
+    u32x4 v[U];
+    auto load = [&](size_t tile) {
+        const size_t left = nvec - tile * kVecs;
+        const rsrc_t r = tile_rsrc(x + tile * (size_t)kVecs * 4, (uint32_t)(left < kVecs ? left : kVecs) * 16u);
+#pragma unroll
+        for (int j = 0; j < U; ++j) v[j] = __builtin_amdgcn_raw_buffer_load_b128(r, (j * T + tid) * 16u, 0, kAuxNt);
+    };
+    size_t tile = blockIdx.x;
+    if (tile < tiles) load(tile);  // on their way while the table is built
+    const bool exact_only = !build_table(sh, steps, step_count, precision, table);
+    const uint32_t first = xlut_first(precision);
+    // `exact` is a type: the table look-up, or (where no table can be trusted) the literal procedure per element
+    auto run = [&](auto exact) {
+        auto encode = [&](uint32_t bits) -> uint32_t {
+            if (decltype(exact)::value) return encode_exact(__uint_as_float(bits), precision, sh.slot);
+            return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
+        };
+        while (tile < tiles) {
+            const size_t left = nvec - tile * kVecs;
+            const rsrc_t r = tile_rsrc(codes + tile * (size_t)kVecs * 4, (uint32_t)(left < kVecs ? left : kVecs) * 4u);
+            uint32_t packed[U];
+            // the whole tile has arrived before the first element is encoded: while a wavefront encodes it has
+            // nothing in flight, which is what keeps the bytes in flight per compute unit at the optimum
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+#pragma unroll
+            for (int j = 0; j < U; ++j)
+                packed[j] = encode(v[j].x) | (encode(v[j].y) << 8) | (encode(v[j].z) << 16) | (encode(v[j].w) << 24);
+#pragma unroll
+            for (int j = 0; j < U; ++j) __builtin_amdgcn_raw_buffer_store_b32(packed[j], r, (j * T + tid) * 4u, 0, kAuxNt);
+            tile += gridDim.x;
+            if (tile < tiles) load(tile);
+        }
+        if (blockIdx.x == 0) {  // ragged tail (n % 4 elements)
+            const size_t i = nvec * 4 + tid;
+            if (i < n) codes[i] = (uint8_t)encode(__float_as_uint(x[i]));
+        }
+    };
+    if (exact_only) run(std::true_type{}); else run(std::false_type{});
+}
+
+// Decompression of whole code words: a tile is kT * kU words (64 KiB of output for 512 x 8); the workgroup waits
+// for its stores before it starts the next tile, which holds the bytes in flight at one tile per compute unit.
+constexpr int kStreamDT = 512, kStreamDU = 8;
+__global__ __launch_bounds__(kStreamDT) void decompress_stream_kernel(
+    const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr, size_t n,
+    float *__restrict__ out, const float *__restrict__ table) {
+    constexpr int T = kStreamDT, U = kStreamDU;
+    constexpr uint32_t kVecs = T * U;
+    __shared__ float lut[256];
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
+    const uint32_t tid = threadIdx.x;
+    if (tid < 126) {
+        const float v = table[tid] * precision;
+        lut[tid] = v;
+        lut[tid + 128] = -v;
+    } else if (tid == 126) {
+        lut[126] = precision;
+        lut[127] = precision;
+        lut[254] = precision;
+        lut[255] = -precision;
+    }
+    __syncthreads();
+    const size_t nvec = n / 4;
+    const size_t tiles = (nvec + kVecs - 1) / kVecs;
+    for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const size_t left = nvec - tile * kVecs;
+        const uint32_t vecs = (uint32_t)(left < kVecs ? left : kVecs);
+        const rsrc_t rc = tile_rsrc(codes + tile * (size_t)kVecs * 4, vecs * 4u);
+        const rsrc_t ro = tile_rsrc(out + tile * (size_t)kVecs * 4, vecs * 16u);
+        uint32_t w[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j) w[j] = __builtin_amdgcn_raw_buffer_load_b32(rc, (j * T + tid) * 4u, 0, 0);
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            u32x4 o;
+            o.x = __float_as_uint(lut[w[j] & 0xffu]);
+            o.y = __float_as_uint(lut[(w[j] >> 8) & 0xffu]);
+            o.z = __float_as_uint(lut[(w[j] >> 16) & 0xffu]);
+            o.w = __float_as_uint(lut[w[j] >> 24]);
+            __builtin_amdgcn_raw_buffer_store_b128(o, ro, (j * T + tid) * 16u, 0, kAuxSc0Sc1Nt);
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this tile's stores have been acknowledged
+    }
+    if (blockIdx.x == 0) {
+        const size_t i = nvec * 4 + tid;
+        if (i < n) out[i] = lut[codes[i]];
     }
 }
 
@@ -311,7 +433,12 @@ __global__ __launch_bounds__(kThreads) void fill_kernel(float *__restrict__ dst,
 
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-static int g_workgroups_per_cu = 0;  // tuning hook: nonzero overrides every kernel's own figure
+static int g_workgroups_per_cu = 0;  // tuning hook: nonzero overrides every kernel's own figure (and keeps the tile kernels)
+// Tensors of at least this many elements take the streaming forms: enough tiles for every compute unit to have
+// several, so that the uneven last round does not show.
+constexpr size_t kStreamFrom = (size_t)1 << 24;
+// Tensors of at least this many elements (256 MiB of fp32) do not fit the 256 MB Infinity Cache.
+constexpr size_t kBeyondCacheFrom = (size_t)1 << 26;
 
 static int stream_grid(const Context *ctx, size_t n, int per_cu) {
     size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
@@ -349,6 +476,23 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
                                    hipFuncAttributeMaxDynamicSharedMemorySize, most));
     }
     const bool vec = aligned(x, 16) && aligned(codes, 4) && (!y || aligned(y, 16));
+    if (vec && !y && n >= kStreamFrom && g_workgroups_per_cu == 0) {
+        static OncePerDevice stream_configured;
+        if (stream_configured.first(ctx->device)) {
+            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<256, 12>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
+            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<512, 10>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
+        }
+        if (n >= kBeyondCacheFrom)
+            hipLaunchKernelGGL((compress_stream_kernel<256, 12>), dim3(ctx->num_cu), dim3(256), sizeof(EncodeShared), st, x,
+                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
+        else
+            hipLaunchKernelGGL((compress_stream_kernel<512, 10>), dim3(ctx->num_cu * 2), dim3(512), sizeof(EncodeShared), st, x,
+                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
     auto kernel = y ? (vec ? compress_kernel<true, true> : compress_kernel<false, true>)
                     : (vec ? compress_kernel<true, false> : compress_kernel<false, false>);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, st, x, precision, precision_dev, n, codes, ctx->xsteps,
@@ -366,7 +510,10 @@ static cn_status decompress_impl(const uint8_t *codes, float precision, const fl
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
     int grid = stream_grid(ctx, n, 8);
-    if (aligned(codes, 4) && aligned(out, 16))
+    if (aligned(codes, 4) && aligned(out, 16) && n >= kStreamFrom && g_workgroups_per_cu == 0)
+        hipLaunchKernelGGL(decompress_stream_kernel, dim3(ctx->num_cu), dim3(kStreamDT), 0, st, codes, precision,
+                           precision_dev, n, out, ctx->table);
+    else if (aligned(codes, 4) && aligned(out, 16))
         hipLaunchKernelGGL(decompress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
                            precision_dev, n, out, ctx->table);
     else

@@ -119,14 +119,6 @@ cn_status cn_absmax_f32(const float *x_device, size_t n, float *out_device, void
  * reduction starts from -1.  NaN inputs are ordered by their bit pattern. */
 cn_status cn_max_f32(const float *x_device, size_t n, float *out_device, void *stream);
 
-/* Measurement aid, no counterpart in the reference: a kernel that only moves bytes in one of the
- * codec's access patterns.  kind 0 reads n fp32 (writes one word per lane: out needs
- * 256 * workgroups_per_cu * compute units words), 1 reads n fp32 and writes n bytes (compression's
- * pattern), 2 reads n bytes and writes n fp32 (decompression's), 3 copies n fp32.  n must be a multiple
- * of 4096; buffers 16-byte aligned.  bench.py reports the codec against these. */
-cn_status cn_stream_yardstick(int kind, const void *in_device, void *out_device, size_t n, int workgroups_per_cu,
-                              void *stream);
-
 /* codes[i] = 8-bit code of x[i] / precision, bit-exact with kCompression_8bit
  * (source/clusterKernels.cu:1163-1232; launcher source/basicOps.cu:1163-1168), flat over n
  * elements.  Inputs whose scaled magnitude falls in (0.99140614, 0.995703], for which the

@@ -195,23 +195,43 @@ def test_large_tensor_by_tiling(dev):
     assert torch.equal(back.view(reps, -1).view(torch.int32), bt.view(torch.int32).unsqueeze(0).expand(reps, -1))
 
 
-def test_stream_yardstick_moves_the_bytes_it_claims(dev):
-    """The arithmetic-free streams the bench compares the codec with: each does what its label says."""
+def test_streaming_forms_ragged_sizes_offsets_and_fallback(dev):
+    """Tensors of 2^24 elements and more take the one-workgroup-per-compute-unit streaming kernels, whose last tile
+    is bounded by a buffer descriptor instead of a per-element test: sizes round a tile boundary, tails of 1 to 3
+    elements, starts that are not 16-byte aligned (which fall back to the element-wise kernel), and a precision for
+    which no table can be built (the literal procedure per element), all against the CPU checker."""
     import torch
-    from clusternet_amd import _lib as L
-    n = 4096 * 37
-    x = torch.randn(n, device=dev)
-    bits = x.view(torch.int32)
-    sink = torch.zeros(256 * 2 * L.num_compute_units(), dtype=torch.int32, device=dev)
-    L.stream_yardstick(0, x, sink, n, 2)
-    assert int(sink.view(torch.int32).to(torch.int64).__and__(0xffffffff).max()) == int(bits.to(torch.int64).__and__(0xffffffff).max())
-    top = torch.empty(n, dtype=torch.uint8, device=dev)
-    L.stream_yardstick(1, x, top, n, 4)
-    assert torch.equal(top, ((bits.to(torch.int64) & 0xffffffff) >> 24).to(torch.uint8))
-    back = torch.empty(n, device=dev)
-    L.stream_yardstick(2, top, back, n, 8)
-    assert torch.equal(back, top.float())
-    L.stream_yardstick(3, x, back, n, 16)
-    assert torch.equal(back, x)
-    with pytest.raises(L.CnError):
-        L.stream_yardstick(1, x, top, n - 1, 2)
+    import clusternet_amd as cn
+    rng = np.random.default_rng(31)
+    base_n = (1 << 24) + 12288 * 3 + 64
+    mag = np.exp(rng.uniform(np.log(1e-7), np.log(1.3), base_n)).astype(np.float32)
+    base = (mag * rng.choice(np.array([-1.0, 1.0], np.float32), base_n)).astype(np.float32)
+    base[:5] = [0.0, -0.0, np.inf, -np.inf, np.nan]
+    want_all = oracle.port_compress(base, 0.77)
+    bt = _t(base, dev)
+    ct = _t(want_all, dev)
+    for n in (1 << 24, (1 << 24) + 1, (1 << 24) + 2, (1 << 24) + 3, (1 << 24) + 4, (1 << 24) + 12288 - 4,
+              (1 << 24) + 12288, (1 << 24) + 12288 * 3 + 61):
+        for off in (0, 4, 1):
+            if off + n > base_n:
+                continue
+            got = cn.compression_8bit(bt[off:off + n], 0.77)
+            assert torch.equal(got, ct[off:off + n]), ("compress", n, off)
+            canary = torch.full((n + 8,), 7.0, device=dev)
+            back = cn.decompression_8bit(ct[off:off + n], 0.77, out=canary[4:4 + n] if off != 1 else canary[1:1 + n])
+            want = _t(oracle.decompress(want_all[off:off + n], 0.77), dev)
+            assert torch.equal(back.view(torch.int32), want.view(torch.int32)), ("decompress", n, off)
+            lo = 4 if off != 1 else 1
+            assert float(canary[:lo].min()) == 7.0 and float(canary[lo + n:].max()) == 7.0 and float(canary[lo + n:].min()) == 7.0
+    # codes written past the end would show here
+    n = (1 << 24) + 5
+    canary = torch.full((n + 64,), 0xAB, dtype=torch.uint8, device=dev)
+    cn.compression_8bit(bt[:n], 0.77, out=canary[32:32 + n])
+    assert torch.equal(canary[32:32 + n], ct[:n]) and int(canary[:32].min()) == 0xAB and int(canary[32 + n:].min()) == 0xAB
+    # no table for these precisions: every element goes through the literal procedure
+    small = base[:(1 << 24) + 7]
+    for prec in (0.0, float("inf"), 1e-42):
+        with np.errstate(all="ignore"):
+            want = oracle.port_compress(small, prec)
+        got = cn.compression_8bit(bt[:small.size], prec).cpu().numpy()
+        assert np.array_equal(got, want), prec
