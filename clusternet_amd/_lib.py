@@ -4,7 +4,9 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_PATH = os.path.join(_HERE, "libcnhip.so")
+# CNHIP_LIB names another build of the same library (the host-sanitizer build of `python -m clusternet_amd.build
+# --host-asan`); CNHIP_NO_TORCH=1 keeps a host-only process from loading PyTorch first.
+_PATH = os.environ.get("CNHIP_LIB") or os.path.join(_HERE, "libcnhip.so")
 _lib = None
 
 
@@ -25,10 +27,11 @@ def lib():
         return _lib
     if not os.path.exists(_PATH):
         raise ImportError("%s is not built; run `python -m clusternet_amd.build`" % _PATH)
-    try:
-        import torch  # noqa: F401  (loads the HIP runtime that owns the tensors we are handed)
-    except ImportError:
-        pass
+    if not os.environ.get("CNHIP_NO_TORCH"):
+        try:
+            import torch  # noqa: F401  (loads the HIP runtime that owns the tensors we are handed)
+        except ImportError:
+            pass
     L = C.CDLL(_PATH)
     i64, vp, f32, sz = C.c_int64, C.c_void_p, C.c_float, C.c_size_t
     L.cn_status_string.restype = C.c_char_p
@@ -62,6 +65,7 @@ def lib():
     L.cn_compress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
     L.cn_decompress_8bit.argtypes = [vp, f32, sz, vp, vp]
     L.cn_decompress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
+    L.cn_decode_8bit_lut.argtypes = [vp, vp, sz, vp, vp]
     L.cn_decompress_8bit_axpy.argtypes = [vp, f32, f32, sz, vp, vp]
     L.cn_decompress_8bit_axpy_dp.argtypes = [vp, vp, f32, sz, vp, vp]
     L.cn_rmsprop_update_f32.argtypes = [vp, vp, vp, f32, f32, sz, vp]
@@ -74,6 +78,8 @@ def lib():
     L.cn_host_force_gemm_tile_n.restype = None
     L.cn_host_gemm_wide_store.argtypes = [C.c_int]
     L.cn_host_gemm_wide_store.restype = None
+    L.cn_host_reduction_fences.argtypes = [C.c_int]
+    L.cn_host_reduction_fences.restype = None
     L.cn_host_csr_strip_kernel.argtypes = [C.c_int]
     L.cn_host_csr_strip_kernel.restype = None
     L.cn_host_csr_lds_rows.argtypes = [C.c_int]
@@ -376,6 +382,20 @@ def decompression_8bit(codes, precision, out=None):
         check(lib().cn_decompress_8bit_dp(codes.data_ptr(), precision.data_ptr(), codes.numel(), out.data_ptr(), _stream()))
     else:
         check(lib().cn_decompress_8bit(codes.data_ptr(), float(precision), codes.numel(), out.data_ptr(), _stream()))
+    return out
+
+
+def decode_8bit_lut(codes, lut, out=None):
+    """out[i] = lut[codes[i]] for a 256-entry fp32 device table."""
+    import torch
+    _need(codes, torch.uint8, "codes")
+    _need(lut, torch.float32, "lut")
+    if not codes.is_contiguous() or lut.numel() != 256 or not lut.is_contiguous():
+        raise ValueError("codes must be contiguous and lut a contiguous tensor of 256 floats")
+    if out is None:
+        out = torch.empty(codes.shape, dtype=torch.float32, device=codes.device)
+    _need(out, torch.float32, "out")
+    check(lib().cn_decode_8bit_lut(codes.data_ptr(), lut.data_ptr(), codes.numel(), out.data_ptr(), _stream()))
     return out
 
 

@@ -215,13 +215,15 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
 constexpr int kStreamDT = 512, kStreamDU = 8;
 __global__ __launch_bounds__(kStreamDT) void decompress_stream_kernel(
     const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr, size_t n,
-    float *__restrict__ out, const float *__restrict__ table) {
+    float *__restrict__ out, const float *__restrict__ table, const float *__restrict__ given_lut) {
     constexpr int T = kStreamDT, U = kStreamDU;
     constexpr uint32_t kVecs = T * U;
     __shared__ float lut[256];
     const float precision = precision_ptr ? *precision_ptr : precision_value;
     const uint32_t tid = threadIdx.x;
-    if (tid < 126) {
+    if (given_lut) {  // the caller's own 256-entry table instead of the codec's
+        if (tid < 256) lut[tid] = given_lut[tid];
+    } else if (tid < 126) {
         const float v = table[tid] * precision;
         lut[tid] = v;
         lut[tid + 128] = -v;
@@ -264,10 +266,12 @@ __global__ __launch_bounds__(kStreamDT) void decompress_stream_kernel(
 template <bool kVector>
 __global__ __launch_bounds__(kThreads) void decompress_kernel(
     const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr,
-    size_t n, float *__restrict__ out, const float *__restrict__ table) {
+    size_t n, float *__restrict__ out, const float *__restrict__ table, const float *__restrict__ given_lut) {
     __shared__ float lut[256];
     const float precision = precision_ptr ? *precision_ptr : precision_value;
-    if (threadIdx.x < 126) {
+    if (given_lut) {  // the caller's own 256-entry table instead of the codec's
+        lut[threadIdx.x] = given_lut[threadIdx.x];
+    } else if (threadIdx.x < 126) {
         float v = table[threadIdx.x] * precision;
         lut[threadIdx.x] = v;
         lut[threadIdx.x + 128] = -v;
@@ -351,7 +355,7 @@ __device__ __forceinline__ float max_unkey(uint32_t key) {
 template <bool kVector, bool kAbs>
 __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restrict__ x, size_t n,
                                                           float *__restrict__ out,
-                                                          uint32_t *__restrict__ tickets) {
+                                                          uint32_t *__restrict__ tickets, int fenced) {
     __shared__ uint32_t smem[kThreads / 64];
     const uint32_t start = kAbs ? 0u : max_key<false>(0xbf800000u);
     uint32_t m = start;
@@ -394,20 +398,27 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
     // ordering by data dependence instead of by fences, which cost far more here (a release fence per
     // workgroup writes the L2 back; nothing in this kernel needs that).  Atomics on one word are performed one
     // after the other, about 12 ns each, hence the groups: their words lie on lines of their own.
+    // The writer side therefore rests on a property of this part (a returning atomic has been performed at the
+    // device's coherence point before an instruction that consumes its result issues), not on the memory model;
+    // the reader side is model-correct: whoever arrives last issues an acquire fence at agent scope before it
+    // reads.  `fenced` (cn_host_reduction_fences) switches the writer to the model's own form, a release fence
+    // between the fold and the count; the tests hold the two forms to the same bits.
     if (threadIdx.x == 0) {
         const uint32_t groups = (gridDim.x + kTicketGroup - 1) / kTicketGroup;
         const uint32_t group = blockIdx.x / kTicketGroup;
         const uint32_t left = gridDim.x - group * kTicketGroup;
         const uint32_t members = left < (uint32_t)kTicketGroup ? left : (uint32_t)kTicketGroup;
         uint32_t *first = tickets + (1 + group) * kTicketStride, *second = tickets;
-        auto fold_and_count = [](uint32_t *line, uint32_t value) -> uint32_t {
+        auto fold_and_count = [fenced](uint32_t *line, uint32_t value) -> uint32_t {
             const uint32_t before = atomicMax(line, value);
             uint32_t one = 1u;
             asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
+            if (fenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             return atomicAdd(line + 1, one);
         };
         auto take = [](uint32_t *line, uint32_t ticket) -> uint32_t {
             asm volatile("" : "+v"(line) : "v"(ticket));  // the read is not issued before the ticket is known
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             const uint32_t v = __hip_atomic_load(line, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(line, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __hip_atomic_store(line + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -502,9 +513,9 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
 }
 
 static cn_status decompress_impl(const uint8_t *codes, float precision, const float *precision_dev,
-                                 size_t n, float *out, void *stream) {
+                                 size_t n, float *out, void *stream, const float *given_lut = nullptr) {
     if (n == 0) return CN_OK;
-    if (!codes || !out) { set_error("decompress_8bit: NULL pointer"); return CN_ERR_NULL; }
+    if (!codes || !out) { set_error("%s: NULL pointer", given_lut ? "decode_8bit_lut" : "decompress_8bit"); return CN_ERR_NULL; }
     Context *ctx;
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
@@ -512,13 +523,13 @@ static cn_status decompress_impl(const uint8_t *codes, float precision, const fl
     int grid = stream_grid(ctx, n, 8);
     if (aligned(codes, 4) && aligned(out, 16) && n >= kStreamFrom && g_workgroups_per_cu == 0)
         hipLaunchKernelGGL(decompress_stream_kernel, dim3(ctx->num_cu), dim3(kStreamDT), 0, st, codes, precision,
-                           precision_dev, n, out, ctx->table);
+                           precision_dev, n, out, ctx->table, given_lut);
     else if (aligned(codes, 4) && aligned(out, 16))
         hipLaunchKernelGGL(decompress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
-                           precision_dev, n, out, ctx->table);
+                           precision_dev, n, out, ctx->table, given_lut);
     else
         hipLaunchKernelGGL(decompress_kernel<false>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
-                           precision_dev, n, out, ctx->table);
+                           precision_dev, n, out, ctx->table, given_lut);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -564,6 +575,11 @@ cn_status cn_decompress_8bit_dp(const uint8_t *codes, const float *precision_dev
     return decompress_impl(codes, 0.0f, precision_device, n, out, stream);
 }
 
+cn_status cn_decode_8bit_lut(const uint8_t *codes, const float *lut256_device, size_t n, float *out, void *stream) {
+    if (n != 0 && !lut256_device) { set_error("decode_8bit_lut: NULL table"); return CN_ERR_NULL; }
+    return decompress_impl(codes, 0.0f, nullptr, n, out, stream, lut256_device);
+}
+
 cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
     if (!out) { set_error("absmax_f32: NULL output"); return CN_ERR_NULL; }
     Context *ctx;
@@ -579,9 +595,9 @@ cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
     if (!x) { set_error("absmax_f32: NULL input"); return CN_ERR_NULL; }
     int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16))
-        hipLaunchKernelGGL((absmax_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
+        hipLaunchKernelGGL((absmax_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets, g_reduction_fences);
     else
-        hipLaunchKernelGGL((absmax_kernel<false, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
+        hipLaunchKernelGGL((absmax_kernel<false, true>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets, g_reduction_fences);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -600,9 +616,9 @@ cn_status cn_max_f32(const float *x, size_t n, float *out, void *stream) {
     if (!x) { set_error("max_f32: NULL input"); return CN_ERR_NULL; }
     int grid = stream_grid(ctx, n, 2);
     if (aligned(x, 16))
-        hipLaunchKernelGGL((absmax_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
+        hipLaunchKernelGGL((absmax_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets, g_reduction_fences);
     else
-        hipLaunchKernelGGL((absmax_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets);
+        hipLaunchKernelGGL((absmax_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, x, n, out, ctx->tickets, g_reduction_fences);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

@@ -109,11 +109,14 @@ __device__ __forceinline__ void publish_absmax(uint32_t v, uint32_t *amax) {
 // LDS image of one operand tile (ROWS index values x BK k; ROWS = 128 for A, TN for B):
 //   KC (memory [index][k]): float offset lds_offset(index, k / 4) + k % 4   (swizzled 16-byte columns)
 //   IC (memory [k][index]): float offset k * ROWS + index
-// The swizzle makes the 16-byte reads of eight consecutive rows at one k quad hit eight different
-// 16-byte bank groups: rows are 128 bytes (BK 32) or 64 bytes (BK 16) apart.
+// The swizzle makes the 16-byte reads of consecutive rows at one k quad hit different 16-byte bank groups, for
+// eight consecutive rows over 128 bytes of banks and for sixteen over 256 bytes (the LDS of this part serves
+// 16-byte reads sixteen lanes at a time: with a swizzle that only separated eight rows, the counters showed a
+// third of the LDS cycles of the 64-byte-row tile as bank conflicts).  Rows are 128 bytes (BK 32) or 64 bytes
+// (BK 16) apart.
 template <int BK>
 __device__ __forceinline__ int swizzle_of(int row) {
-    return BK == 32 ? ((row & 7) ^ ((row >> 3) & 3)) : ((row >> 1) & 3);
+    return BK == 32 ? ((row & 7) ^ ((row >> 3) & 3)) : (((row >> 1) & 3) ^ ((row >> 3) & 1));
 }
 template <int BK>
 __device__ __forceinline__ int lds_offset(int row, int quad) {

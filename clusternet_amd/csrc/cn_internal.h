@@ -56,6 +56,10 @@ struct OncePerDevice {
     }
 };
 
+// Test switch (cn_host_reduction_fences): nonzero makes the single-launch reductions order their partial results
+// with a release fence per workgroup instead of by data dependence.
+extern int g_reduction_fences;
+
 // Returns the context of the current device, initialising it on first use.
 cn_status current_context(Context **out);
 

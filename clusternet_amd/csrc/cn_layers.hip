@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kT) void softmax_kernel(const float *__restrict__ A
 // to depend on what the exchange returned, so the partial has been stored before the workgroup is counted:
 // ordering by data dependence, which costs far less than a fence per workgroup.
 __global__ __launch_bounds__(kT) void sum_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ out,
-                                                 double *__restrict__ partial, uint32_t *__restrict__ counter) {
+                                                 double *__restrict__ partial, uint32_t *__restrict__ counter, int fenced) {
     __shared__ double sm[kT];
     __shared__ uint32_t s_last;
     double s = 0.0;
@@ -185,8 +185,12 @@ __global__ __launch_bounds__(kT) void sum_kernel(const float *__restrict__ x, in
         const unsigned long long before = atomicExch(&slots[blockIdx.x], (unsigned long long)__double_as_longlong(sm[0]));
         uint32_t one = 1u;
         asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
+        // writer side: ordered by that dependence (see absmax_kernel), or by a release fence when `fenced`
+        if (fenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         const uint32_t ticket = atomicAdd(counter, one);
         s_last = (ticket == gridDim.x - 1) ? 1u : 0u;
+        // reader side: the last to arrive acquires before any of its lanes reads the partial sums
+        if (s_last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
     __syncthreads();
     if (s_last) {
@@ -343,7 +347,7 @@ cn_status cn_sum_f32(const float *x, size_t n, float *out_device, void *stream) 
     if (grid > 1024) grid = 1024;
     // arrival counter: the slot after the abs-max kernel's counter
     hipLaunchKernelGGL(sum_kernel, dim3(grid), dim3(kT), 0, st, x, (int64_t)n, out_device, ctx->sum_scratch,
-                       ctx->reduce_scratch + kReduceSlots + 1);
+                       ctx->reduce_scratch + kReduceSlots + 1, g_reduction_fences);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

@@ -28,6 +28,8 @@ cn_status hip_fail(hipError_t e, const char *what, const char *file, int line) {
 
 void host_table(float out[126]);
 
+int g_reduction_fences = 0;
+
 static Context g_ctx[kMaxDevices];
 static std::mutex g_mutex;
 
@@ -62,6 +64,24 @@ static cn_status init_device(int device) {
     int previous = 0;
     CN_HIP(hipGetDevice(&previous));
     CN_HIP(hipSetDevice(device));
+    // On any failure below: what was allocated so far is released, the context stays unready and the caller's
+    // device is current again, so that a later attempt starts from nothing instead of leaking another set.
+    struct Undo {
+        Context &c;
+        int previous;
+        bool armed = true;
+        ~Undo() {
+            if (!armed) return;
+            (void)hipFree(c.table);
+            (void)hipFree(c.xsteps);
+            (void)hipFree(c.workspace);
+            (void)hipFree(c.reduce_scratch);
+            (void)hipFree(c.tickets);
+            (void)hipFree(c.sum_scratch);
+            c = Context();
+            (void)hipSetDevice(previous);
+        }
+    } undo{c, previous};
     hipDeviceProp_t prop;
     CN_HIP(hipGetDeviceProperties(&prop, device));
     c.device = device;
@@ -99,6 +119,7 @@ static cn_status init_device(int device) {
     }
     CN_HIP(hipDeviceSynchronize());
     CN_HIP(hipSetDevice(previous));
+    undo.armed = false;
     c.ready = true;
     return CN_OK;
 }
@@ -143,6 +164,8 @@ const char *cn_status_string(cn_status s) {
 }
 
 const char *cn_last_error(void) { return g_error; }
+
+void cn_host_reduction_fences(int enabled) { g_reduction_fences = enabled != 0; }
 
 cn_status cn_init(int device) {
     std::lock_guard<std::mutex> lock(g_mutex);

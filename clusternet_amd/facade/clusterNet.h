@@ -47,6 +47,19 @@ public:
     void decompression_8bit(Matrix *A, float precision, Matrix *out);
     // out = A decode(B codes, precisionB): the fused kernel that takes the place of the
     // dot8bit prototypes (source/clusterNet.cpp:1409-1431).  A is fp32, B is a char matrix.
+    // The 8-bit products of the reference (source/clusterNet.h:146-149, source/clusterNet.cpp:1409-1431): A and B are
+    // char matrices, out += decodeA(A) decodeB(B) in fp32.  As in kDot8bit (source/clusterKernels.cu:1717-1762) the
+    // result is ADDED to what out holds, and each operand is decoded through that kernel's own table, whose special
+    // codes are not the codec's: 126 -> 0 and 254 -> -0 on both sides, 127 -> precisionA (A) / -precisionA (B),
+    // 255 -> precisionB (A) / -precisionB (B) -- the reference's literal, evidently mixed-up, assignments.  Here the
+    // operands are decoded and multiplied on the matrix cores, so sums differ from the reference's sequential fp32
+    // accumulation within the usual product tolerance; dot8bit_shared (tiles + atomicAdd in the reference, whose
+    // order of additions is not defined) is the same computation.  The value-returning forms start from zeros of
+    // A->rows x B->cols (the reference allocates A->rows x A->cols without clearing it).
+    void dot8bit(Matrix *A, Matrix *B, float precisionA, float precisionB, Matrix *out);
+    Matrix *dot8bit(Matrix *A, Matrix *B, float precisionA, float precisionB);
+    void dot8bit_shared(Matrix *A, Matrix *B, float precisionA, float precisionB, Matrix *out);
+    Matrix *dot8bit_shared(Matrix *A, Matrix *B, float precisionA, float precisionB);
     Matrix *dot8bit_weights(Matrix *A, Matrix *B, float precisionB);
     void dot8bit_weights(Matrix *A, Matrix *B, float precisionB, Matrix *out);
 

@@ -148,6 +148,12 @@ cn_status cn_decompress_8bit(const uint8_t *codes_device, float precision, size_
 cn_status cn_decompress_8bit_dp(const uint8_t *codes_device, const float *precision_device,
                                 size_t n, float *out_device, void *stream);
 
+/* out[i] = lut[codes[i]] for a 256-entry fp32 table the caller keeps in device memory.  It is the table look-up that
+ * the 8-bit products kDot8bit / kDot8bit_shared apply to both coded operands, each with a table of its own whose
+ * special codes differ from the codec's (source/clusterKernels.cu:1722-1739, 1775-1792). */
+cn_status cn_decode_8bit_lut(const uint8_t *codes_device, const float *lut256_device, size_t n, float *out_device,
+                             void *stream);
+
 /* ---- fused passes that follow the 8-bit exchange of a gradient ------------------------------- */
 
 /* y[i] = y[i] + alpha * decode(codes[i]) in one pass (9 bytes per element instead of 17), decode as

@@ -32,6 +32,11 @@ void cn_host_gemm_wide_store(int enabled);
 /* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
 void cn_host_codec_workgroups_per_cu(int per_cu);
 
+/* Nonzero: the single-launch reductions (abs-max, max, sum) put a release fence at device scope between a
+ * workgroup's partial result and its arrival count, the form the memory model prescribes, instead of ordering the
+ * two by a data dependence; the last workgroup acquires either way.  Same results; for tests of that equality. */
+void cn_host_reduction_fences(int enabled);
+
 /* 0 = sparse products never take the strip kernel (few long rows) / the kernel that keeps a strip of B in
  * LDS (maximum only); they then run on the general kernels, which the tests compare against. */
 void cn_host_csr_strip_kernel(int enabled);

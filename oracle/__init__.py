@@ -11,7 +11,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_SO = os.path.join(_HERE, "liboracle.so")
+# CN_ORACLE_LIB names another build of the same sources (the sanitizer build, oracle/_asan/liboracle.so)
+_SO = os.environ.get("CN_ORACLE_LIB") or os.path.join(_HERE, "liboracle.so")
 
 _c = ctypes
 _f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")

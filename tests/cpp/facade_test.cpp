@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "clusterNet.h"
+#include "cnhip.h"
 
 extern "C" {
 void cn_oracle_compress_literal(const float *x, float precision, size_t n, uint8_t *codes, int sliver_rule);
@@ -269,6 +270,61 @@ static void run_codec_test(ClusterNet gpu) {
     CHECK(worst <= 1e-4f * scale, "fused 8-bit-weight product matches decompress + dot");
 }
 
+// dot8bit / dot8bit_shared (source/clusterNet.cpp:1409-1431) against a brute-force loop over kDot8bit's own decode
+// tables (source/clusterKernels.cu:1725-1739), written out here from the source text: out += decA(A) decB(B).
+static void run_dot8bit_test(ClusterNet gpu) {
+    const int M = 37, K = 150, N = 29;
+    const float pA = 0.75f, pB = 2.5f;
+    float t[126];
+    CHECK(cn_table_get(t) == 0, "table");
+    double ta[256], tb[256];
+    for (int i = 0; i < 126; ++i) {
+        ta[i] = (double)(t[i] * pA); ta[i + 128] = -ta[i];
+        tb[i] = (double)(t[i] * pB); tb[i + 128] = -tb[i];
+    }
+    ta[126] = 0; tb[126] = 0; ta[127] = pA; tb[127] = -pA; ta[254] = -0.0; tb[254] = -0.0; ta[255] = pB; tb[255] = -pB;
+    Matrix *A = empty_char(M, K), *B = empty_char(K, N);
+    std::vector<uint8_t> a(M * K), b(K * N);
+    uint32_t seed = 12345;
+    auto next = [&]() { seed = seed * 1664525u + 1013904223u; return (uint8_t)(seed >> 24); };
+    for (auto &c : a) c = next();
+    for (auto &c : b) c = next();
+    // every special code on both sides
+    const uint8_t special[4] = {126, 127, 254, 255};
+    for (int i = 0; i < 4; ++i) { a[i * 7] = special[i]; b[i * 11 + 3] = special[i]; a[K + i] = special[i]; b[N * 2 + i] = special[i]; }
+    CHECK(cn_memcpy_h2d(A->char_data, a.data(), a.size()) == 0, "upload A");
+    CHECK(cn_memcpy_h2d(B->char_data, b.data(), b.size()) == 0, "upload B");
+    std::vector<double> want(M * N), scale(M * N);
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j) {
+            double s = 0, sa = 0;
+            for (int k = 0; k < K; ++k) { const double p = ta[a[i * K + k]] * tb[b[k * N + j]]; s += p; sa += fabs(p); }
+            want[i * N + j] = s; scale[i * N + j] = sa;
+        }
+    // accumulation into what `out` holds, twice in a row, through both names
+    Matrix *out = fill_matrix(M, N, 1.5f);
+    gpu.dot8bit(A, B, pA, pB, out);
+    Matrix *h1 = to_host(out);
+    gpu.dot8bit_shared(A, B, pA, pB, out);
+    Matrix *h2 = to_host(out);
+    double worst1 = 0, worst2 = 0;
+    for (int i = 0; i < M * N; ++i) {
+        worst1 = fmax(worst1, fabs((double)h1->data[i] - (1.5 + want[i])) / (scale[i] + 1.5));
+        worst2 = fmax(worst2, fabs((double)h2->data[i] - (1.5 + 2 * want[i])) / (2 * scale[i] + 1.5));
+    }
+    CHECK(worst1 <= 1e-5, "dot8bit adds the decoded product to out");
+    CHECK(worst2 <= 1e-5, "dot8bit_shared adds it again");
+    Matrix *fresh = gpu.dot8bit(A, B, pA, pB);
+    CHECK(test_matrix(fresh, M, N), "dot8bit returns A->rows x B->cols");
+    Matrix *hf = to_host(fresh);
+    double worst3 = 0;
+    for (int i = 0; i < M * N; ++i) worst3 = fmax(worst3, fabs((double)hf->data[i] - want[i]) / (scale[i] + 1e-30));
+    CHECK(worst3 <= 1e-5, "value-returning dot8bit starts from zeros");
+    bool thrown = false;
+    try { gpu.dot8bit(A, A, pA, pB, out); } catch (const char *msg) { thrown = strcmp(msg, "Matrix *size error:\n") == 0; }
+    CHECK(thrown, "dot8bit throws the reference's message on a shape mismatch");
+}
+
 static void run_basicOps_test(ClusterNet gpu) {
     // layout round trips (reference tests/basicOps_test.cu:20-57,200-247)
     Matrix *m1 = gpu.rand(37, 53);
@@ -366,6 +422,7 @@ int main() {
         run_basicOps_test(gpus);
         run_clusterNet_test(gpus);
         run_codec_test(gpus);
+        run_dot8bit_test(gpus);
     } catch (const char *e) {
         printf("uncaught error: %s\n", e);
         return 2;

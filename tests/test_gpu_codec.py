@@ -55,6 +55,36 @@ def test_absmax_matches_numpy(dev):
         assert float(cn.absmax(xt).cpu()[0]) == oracle.absmax(xt.cpu().numpy())
 
 
+def test_reductions_with_and_without_writer_fences(dev):
+    """The single-launch reductions order a workgroup's partial result and its arrival count by a data dependence
+    (the last workgroup acquires); cn_host_reduction_fences switches the writers to a release fence, the form the
+    memory model prescribes.  Both forms must give the same bits, over grid sizes from one workgroup to the cap,
+    and on repeated calls (every ticket word is put back to zero by the last to arrive)."""
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(123)
+    x = rng.normal(0, 3, 6_000_011).astype(np.float32)
+    xt = _t(x, dev)
+    try:
+        for n in (1, 4096, 4097, 70_000, 1_000_003, 6_000_011):
+            want_max = float(np.abs(x[:n]).max())
+            want_sum = None
+            for per_cu in (0, 1, 3, 16):
+                L.lib().cn_host_codec_workgroups_per_cu(per_cu)
+                for fenced in (0, 1, 0):
+                    L.lib().cn_host_reduction_fences(fenced)
+                    assert float(cn.absmax(xt[:n]).cpu()[0]) == want_max, (n, per_cu, fenced)
+                    assert float(L.reduce_max(xt[:n]).cpu()[0]) == max(float(x[:n].max()), -1.0), (n, per_cu, fenced)
+                    got = float(L.reduce_sum(xt[:n]).cpu()[0])
+                    want_sum = got if want_sum is None else want_sum
+                    assert got == want_sum, (n, per_cu, fenced)
+            assert abs(want_sum - float(x[:n].astype(np.float64).sum())) <= 1e-6 * np.abs(x[:n]).astype(np.float64).sum()
+    finally:
+        L.lib().cn_host_reduction_fences(0)
+        L.lib().cn_host_codec_workgroups_per_cu(0)
+
+
 def test_compress_config2_bit_exact(dev):
     import clusternet_amd as cn
     x = cfg2_tensor(np.random.default_rng(42))
@@ -235,3 +265,21 @@ def test_streaming_forms_ragged_sizes_offsets_and_fallback(dev):
             want = oracle.port_compress(small, prec)
         got = cn.compression_8bit(bt[:small.size], prec).cpu().numpy()
         assert np.array_equal(got, want), prec
+
+
+def test_decode_through_a_given_table(dev):
+    """cn_decode_8bit_lut: out[i] = lut[codes[i]] for any 256-entry table, on both kernels (tile and streaming),
+    ragged sizes and unaligned starts."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(8)
+    lut = rng.normal(0, 1, 256).astype(np.float32)
+    lut[126], lut[254] = 0.0, -0.0
+    codes = rng.integers(0, 256, (1 << 24) + 4103, dtype=np.uint8)
+    ct, lt = _t(codes, dev), _t(lut, dev)
+    for n in (0, 1, 5, 4096, 65_539, (1 << 24), (1 << 24) + 4103):
+        for off in (0, 1, 4):
+            if off + n > codes.size:
+                continue
+            got = L.decode_8bit_lut(ct[off:off + n], lt).cpu().numpy()
+            assert np.array_equal(got.view(np.uint32), lut[codes[off:off + n]].view(np.uint32)), (n, off)

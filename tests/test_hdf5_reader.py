@@ -13,8 +13,10 @@ DATA = os.path.join(HERE, "golden", "hdf5")
 
 @pytest.fixture(scope="module")
 def reader():
-    import torch  # noqa: F401  (the facade links the HIP runtime; load torch's copy first)
-    lib = C.CDLL(os.path.join(os.path.dirname(HERE), "clusternet_amd", "libclusternet.so"))
+    if not os.environ.get("CNHIP_NO_TORCH"):
+        import torch  # noqa: F401  (the facade links the HIP runtime; load torch's copy first)
+    # CN_FACADE_LIB: another build of the facade (the host-sanitizer build)
+    lib = C.CDLL(os.environ.get("CN_FACADE_LIB") or os.path.join(os.path.dirname(HERE), "clusternet_amd", "libclusternet.so"))
     fn = lib.cn_facade_read_hdf5
     fn.argtypes = [C.c_char_p, C.c_char_p, C.POINTER(C.c_longlong), C.POINTER(C.c_longlong),
                    C.POINTER(C.POINTER(C.c_float)), C.POINTER(C.c_char_p)]
