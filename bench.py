@@ -164,7 +164,15 @@ def bench_codec(torch, cn, dev):
             # small buffers: the kernels take a few microseconds, so also time them replayed from a graph
             replayed = {"absmax_us": time_replayed(torch, lambda: cn.absmax(x, prec_t), 20, 50),
                         "compress_us": time_replayed(torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50),
-                        "decompress_us": time_replayed(torch, lambda: cn.decompression_8bit(codes, prec_t, back), 20, 50)}
+                        "decompress_us": time_replayed(torch, lambda: cn.decompression_8bit(codes, prec_t, back), 20, 50),
+                        "absmax_then_compress_us": time_replayed(
+                            torch, lambda: (cn.absmax(x, prec_t), cn.compression_8bit(x, prec_t, codes)), 20, 50),
+                        "absmax_compress_one_call_us": time_replayed(
+                            torch, lambda: cn.absmax_compression_8bit(x, codes, prec_t), 20, 50)}
+            cn.lib().cn_host_absmax_compress_single_launch(1)
+            replayed["absmax_compress_single_launch_us"] = time_replayed(
+                torch, lambda: cn.absmax_compression_8bit(x, codes, prec_t), 20, 50)
+            cn.lib().cn_host_absmax_compress_single_launch(0)
             res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
         if n >= 100000 * 8192:
             # movers that are not this library's: the runtime's device-to-device copy (above) and its fill, the latter a

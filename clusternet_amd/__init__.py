@@ -3,9 +3,9 @@ path.  The product is the C-ABI library libcnhip.so (see include/cnhip.h) and th
 ClusterNet / Matrix facade over it; this package is the thin Python host binding used by the
 tests and the benchmark.  PyTorch appears only as the owner of device memory and streams.
 """
-from ._lib import (CnError, absmax, compression_8bit, compression_8bit_axpy, decompression_8bit, decompression_8bit_axpy, dot, dotT,
+from ._lib import (CnError, absmax, absmax_compression_8bit, compression_8bit, compression_8bit_axpy, decompression_8bit, decompression_8bit_axpy, dot, dotT,
                    Tdot, gemm, gemm_w8, init, lib, lib_path, num_compute_units, rmsprop_update, table)
 
-__all__ = ["CnError", "absmax", "compression_8bit", "compression_8bit_axpy", "decompression_8bit", "decompression_8bit_axpy", "dot",
+__all__ = ["CnError", "absmax", "absmax_compression_8bit", "compression_8bit", "compression_8bit_axpy", "decompression_8bit", "decompression_8bit_axpy", "dot",
            "dotT", "Tdot", "gemm", "gemm_w8", "init", "lib", "lib_path", "num_compute_units", "rmsprop_update",
            "table"]

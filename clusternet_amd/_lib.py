@@ -66,6 +66,11 @@ def lib():
     L.cn_decompress_8bit.argtypes = [vp, f32, sz, vp, vp]
     L.cn_decompress_8bit_dp.argtypes = [vp, vp, sz, vp, vp]
     L.cn_decode_8bit_lut.argtypes = [vp, vp, sz, vp, vp]
+    L.cn_absmax_compress_8bit.argtypes = [vp, sz, vp, vp, vp]
+    L.cn_host_absmax_compress_single_launch.argtypes = [C.c_int]
+    L.cn_host_absmax_compress_single_launch.restype = None
+    L.cn_host_absmax_compress_spin_limit.argtypes = [C.c_int]
+    L.cn_host_absmax_compress_spin_limit.restype = None
     L.cn_decompress_8bit_axpy.argtypes = [vp, f32, f32, sz, vp, vp]
     L.cn_decompress_8bit_axpy_dp.argtypes = [vp, vp, f32, sz, vp, vp]
     L.cn_rmsprop_update_f32.argtypes = [vp, vp, vp, f32, f32, sz, vp]
@@ -346,6 +351,22 @@ def compression_8bit(A, precision, out=None):
     else:
         check(lib().cn_compress_8bit(A.data_ptr(), float(precision), A.numel(), out.data_ptr(), _stream()))
     return out
+
+
+def absmax_compression_8bit(A, out=None, precision_out=None):
+    """(codes, precision): precision = max|A| as a one-element device tensor and the codes of A under it, one call."""
+    import torch
+    _need(A, torch.float32, "A")
+    if not A.is_contiguous():
+        raise ValueError("A must be contiguous")
+    if out is None:
+        out = torch.empty(A.shape, dtype=torch.uint8, device=A.device)
+    _need(out, torch.uint8, "out")
+    if precision_out is None:
+        precision_out = torch.empty(1, dtype=torch.float32, device=A.device)
+    _need(precision_out, torch.float32, "precision_out")
+    check(lib().cn_absmax_compress_8bit(A.data_ptr(), A.numel(), out.data_ptr(), precision_out.data_ptr(), _stream()))
+    return out, precision_out
 
 
 def compression_8bit_axpy(A, precision, alpha, y, out=None):

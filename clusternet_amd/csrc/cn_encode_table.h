@@ -24,10 +24,18 @@ struct EncodeShared {
     int step_index[kXMaxSteps];
     XEntry step_entry[kXMaxSteps];
     uint8_t mark[(kXEntries + 3) / 4 * 4];  // 1 + number of the step that sits in this entry's bucket, 0 if none
+    uint32_t sentinel_code[8];              // literal codes at the eight patterns that define the two sentinel entries
 };
 static_assert(kXMaxSteps < 255, "a step's number plus one fits a byte");
 
 // Returns true when the table in sh.lut may be used.
+//
+// The build is a chain of latencies (a workgroup of a small call does little else), so it is laid out for a short
+// critical path: a thread's own step comes from global memory together with the codebook and is located in
+// registers before the first barrier; the eight literal evaluations behind the two sentinel entries run one per
+// lane on wavefronts that locate no step; every group of LDS reads is issued as a whole before its first use
+// (unconditional loads, conditions applied to the values), because a conditional read costs a full LDS round
+// trip each.  Measured at the shader clock: about 4 800 cycles, against 11 000 with dependent reads.
 __device__ __forceinline__ bool build_table(EncodeShared &sh, const XStep *__restrict__ steps, int count,
                                             float precision, const float *__restrict__ table) {
     const int t = threadIdx.x;
@@ -38,28 +46,57 @@ __device__ __forceinline__ bool build_table(EncodeShared &sh, const XStep *__res
     if (t < 126) sh.slot[t] = table[t];
     if (t == 126) sh.slot[126] = 1.0f;
     if (t == 127) sh.slot[127] = 0.0f;
-    __syncthreads();
     const uint32_t first = xlut_first(precision);
+    // the own step: registers only, needs nothing of the above
     bool bad = false;
     XEntry e{};
     int index = 0;
     if (t < count) {
-        bad = !xlut_locate_step(mine, precision, sh.slot, &e);
+        bad = !xlut_locate_step(mine, precision, nullptr, &e);
         index = (int)(e.boundary >> kXShift) - (int)first + 1;
         if (bad || index < 1 || index > kXBuckets) { bad = true; index = 0; }
+    }
+    __syncthreads();  // the codebook copy and the cleared marks are there
+    if (t < count) {
         sh.step_index[t] = index;
+        sh.step_entry[t] = e;
         if (index > 0) sh.mark[index] = (uint8_t)(t + 1);
-    } else if (t == kEncodeThreads / 2) {       // the two sentinels: lanes of wavefronts that locate no step,
-        sh.lut[0] = xlut_entry(0, precision, sh.slot, &bad);
-    } else if (t == 3 * kEncodeThreads / 4) {   // so that they run beside the steps and not after them
-
-        sh.lut[kXEntries - 1] = xlut_entry(kXEntries - 1, precision, sh.slot, &bad);
+    }
+    // The sentinels (xlut_entry for the entries 0 and kXEntries - 1) take literal evaluations at eight patterns:
+    // lane j of the third wavefront evaluates pattern j, one lane assembles the two entries behind the barrier.
+    const uint32_t kSign = 0x80000000u;
+    const uint32_t top = first > 0 ? (first << kXShift) - 1 : 0u;
+    const uint64_t start64 = ((uint64_t)first + kXBuckets) << kXShift;
+    const uint32_t start = start64 > 0x7f800000u ? 0x7f800000u : (uint32_t)start64;
+    constexpr int kSentinelLane = kEncodeThreads / 2;
+    if (t >= kSentinelLane && t < kSentinelLane + 8) {
+        const uint32_t pattern[8] = {top, top | kSign, 0x7fc00000u, 0xffc00000u, start, start | kSign, 0x7f800000u, 0xff800000u};
+        uint32_t mine_bits = pattern[0];
+#pragma unroll
+        for (int j = 1; j < 8; ++j) mine_bits = (t - kSentinelLane == j) ? pattern[j] : mine_bits;
+        sh.sentinel_code[t - kSentinelLane] = encode_exact(x_from_bits(mine_bits), precision, sh.slot);
+    }
+    __syncthreads();
+    // the steps must come in ascending buckets, one per bucket
+    if (t > 0 && t < count) bad = bad || (index <= sh.step_index[t - 1]);
+    if (t == kSentinelLane) {
+        uint32_t c[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c[j] = sh.sentinel_code[j];
+        // entry 0: everything below bucket `first` must be code 254, up to its largest pattern
+        if (first > 0 && (c[0] != 254u || c[1] != 254u)) bad = true;
+        sh.lut[0] = XEntry{0xffffffffu, pack_codes(254, 254, 254, 254)};
+        // last entry: one code from the end of the last bucket up to infinity, then the code of a NaN
+        XEntry last;
+        if (start64 > 0x7f800000u) {
+            last = XEntry{0u, pack_codes(c[2], c[2], c[3], c[3])};  // only NaNs left
+        } else {
+            if (c[4] != c[6] || c[5] != c[7]) bad = true;
+            last = XEntry{0x7f800001u, pack_codes(c[4], c[2], c[5], c[3])};
+        }
+        sh.lut[kXEntries - 1] = last;
         if ((uint64_t)first + kXBuckets > 0xff00u) bad = true;  // infinity / NaN inside the window
     }
-    if (t < count) sh.step_entry[t] = e;
-    if (__syncthreads_or(bad ? 1 : 0)) return false;
-    // the steps must come in ascending buckets, one per bucket
-    bad = (t > 0 && t < count) ? (index <= sh.step_index[t - 1]) : false;
     if (__syncthreads_or(bad ? 1 : 0)) return false;
     // Every thread fills a run of consecutive entries.  An entry whose bucket holds a step is that step's
     // entry; any other carries the codes above the nearest step below it (below the first step: the codes
@@ -68,36 +105,45 @@ __device__ __forceinline__ bool build_table(EncodeShared &sh, const XStep *__res
     // 4) words apart and spread over all banks.
     constexpr int kRun = ((kXBuckets + kEncodeThreads - 1) / kEncodeThreads) | 1;
     const int i0 = 1 + t * kRun;
-    // steps whose bucket lies before entry i0: a count over every sixteenth step, then over the sixteen behind
-    // the last of those that qualify (two rounds of independent reads instead of a chain of eight)
+    // steps whose bucket lies before entry i0: a count over every sixteenth step, then over the fifteen behind
+    // the last of those that qualify: two rounds of independent reads
     static_assert(kXMaxSteps % 16 == 0, "coarse stride");
+    int every16th[kXMaxSteps / 16];
+#pragma unroll
+    for (int c = 0; c < kXMaxSteps / 16; ++c) every16th[c] = sh.step_index[16 * c + 15];
     int coarse = 0;
 #pragma unroll
-    for (int c = 16; c <= kXMaxSteps; c += 16) coarse += (c <= count && sh.step_index[c - 1] < i0) ? 1 : 0;
-    int below = 16 * coarse;
-    {
-        int fine = 0;
+    for (int c = 0; c < kXMaxSteps / 16; ++c) coarse += ((16 * c + 16 <= count) & (every16th[c] < i0)) ? 1 : 0;
+    int behind[15];
 #pragma unroll
-        for (int f = 0; f < 15; ++f) {
-            const int k = 16 * coarse + f;
-            fine += (k < count && sh.step_index[k < kXMaxSteps ? k : kXMaxSteps - 1] < i0) ? 1 : 0;
-        }
-        below += fine;
+    for (int f = 0; f < 15; ++f) {
+        const int k = 16 * coarse + f;
+        behind[f] = sh.step_index[k < kXMaxSteps ? k : kXMaxSteps - 1];
     }
+    int below = 16 * coarse;
+#pragma unroll
+    for (int f = 0; f < 15; ++f) below += ((16 * coarse + f < count) & (behind[f] < i0)) ? 1 : 0;
     // Entries past the last bucket are clamped to it: those lanes compute and store the last bucket's own
     // entry again, which keeps the loop free of branches.
     uint32_t marks[kRun];
 #pragma unroll
     for (int m = 0; m < kRun; ++m) marks[m] = sh.mark[i0 + m <= kXBuckets ? i0 + m : kXBuckets];
-    uint32_t nearest = (uint32_t)below;  // 1 + number of the nearest step at or below the entry, 0 if none
+    uint32_t nearest[kRun];  // 1 + number of the nearest step at or below the entry, 0 if none
+    uint32_t running = (uint32_t)below;
 #pragma unroll
     for (int m = 0; m < kRun; ++m) {
-        nearest = marks[m] ? marks[m] : nearest;
-        const XEntry of_step = sh.step_entry[nearest ? nearest - 1 : 0];
-        const XEntry flat = xlut_flat_entry(of_step, nearest != 0);
+        running = marks[m] ? marks[m] : running;
+        nearest[m] = running;
+    }
+    XEntry of_step[kRun];
+#pragma unroll
+    for (int m = 0; m < kRun; ++m) of_step[m] = sh.step_entry[nearest[m] ? nearest[m] - 1 : 0];
+#pragma unroll
+    for (int m = 0; m < kRun; ++m) {
+        const XEntry flat = xlut_flat_entry(of_step[m], nearest[m] != 0);
         XEntry e_m;
-        e_m.boundary = marks[m] ? of_step.boundary : flat.boundary;
-        e_m.codes = marks[m] ? of_step.codes : flat.codes;
+        e_m.boundary = marks[m] ? of_step[m].boundary : flat.boundary;
+        e_m.codes = marks[m] ? of_step[m].codes : flat.codes;
         sh.lut[i0 + m <= kXBuckets ? i0 + m : kXBuckets] = e_m;
     }
     __syncthreads();

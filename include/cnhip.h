@@ -130,6 +130,15 @@ cn_status cn_compress_8bit(const float *x_device, float precision, size_t n,
 cn_status cn_compress_8bit_dp(const float *x_device, const float *precision_device, size_t n,
                               uint8_t *codes_device, void *stream);
 
+/* *precision_out_device = max_i |x_i| and codes = the codes of x under that precision, in one call and without a
+ * round trip to the host: the same bits as cn_absmax_f32 followed by cn_compress_8bit_dp.  The pair of calls in front
+ * of every exchange of a gradient, max(abs(grad)) then compression_8bit (source/DeepNeuralNetwork.cpp:334-339,
+ * source/test.cu:2108-2111).  It runs as those two kernels, one behind the other on the stream; a form that does both
+ * phases in one launch (a wait across the grid between them) exists and measures slower on this part, see
+ * cn_host_absmax_compress_single_launch. */
+cn_status cn_absmax_compress_8bit(const float *x_device, size_t n, uint8_t *codes_device,
+                                  float *precision_out_device, void *stream);
+
 /* cn_compress_8bit followed by cn_decompress_8bit_axpy on its codes, in one pass: codes[i] as above and
  * y[i] += alpha * (decoded value of codes[i]).  A gradient's codes for the exchange and the own weight
  * update (source/Layer.cpp:365, 430-433) at 13 bytes per element instead of 5 + 9; same bits.  x, codes and y

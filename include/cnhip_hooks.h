@@ -37,6 +37,14 @@ void cn_host_codec_workgroups_per_cu(int per_cu);
  * two by a data dependence; the last workgroup acquires either way.  Same results; for tests of that equality. */
 void cn_host_reduction_fences(int enabled);
 
+/* Nonzero: cn_absmax_compress_8bit runs as one launch (abs-max, a wait across the resident grid, compression) for
+ * aligned tensors below 2^26 elements instead of as two kernels.  Same bits. */
+void cn_host_absmax_compress_single_launch(int enabled);
+
+/* How often a workgroup of the single-launch cn_absmax_compress_8bit looks for the rest of the grid before it takes the maximum
+ * by itself; negative = the library's figure.  0 lets the tests reach that path: every workgroup then gives up at once. */
+void cn_host_absmax_compress_spin_limit(int spins);
+
 /* 0 = sparse products never take the strip kernel (few long rows) / the kernel that keeps a strip of B in
  * LDS (maximum only); they then run on the general kernels, which the tests compare against. */
 void cn_host_csr_strip_kernel(int enabled);

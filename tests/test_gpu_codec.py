@@ -283,3 +283,51 @@ def test_decode_through_a_given_table(dev):
                 continue
             got = L.decode_8bit_lut(ct[off:off + n], lt).cpu().numpy()
             assert np.array_equal(got.view(np.uint32), lut[codes[off:off + n]].view(np.uint32)), (n, off)
+
+
+def test_absmax_and_compression_in_one_call(dev):
+    """cn_absmax_compress_8bit against cn_absmax_f32 followed by cn_compress_8bit_dp and against the CPU checker, as
+    the two kernels it runs by default and as the single launch behind cn_host_absmax_compress_single_launch: sizes on
+    both sides of every dispatch boundary, unaligned starts, all-zero and NaN-bearing data, calls in a row, and with
+    the single launch's wait for the rest of the grid cut to nothing, so that every workgroup that would have
+    waited takes the maximum by itself."""
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(77)
+    big = (1 << 26) + 8
+    base = rng.normal(0, 0.02, big + 4).astype(np.float32)
+    base[::101] *= 20
+    bt = _t(base, dev)
+    try:
+        for single, spins in ((0, -1), (1, -1), (1, 0), (1, -1)):
+            L.lib().cn_host_absmax_compress_single_launch(single)
+            L.lib().cn_host_absmax_compress_spin_limit(spins)
+            for n, off in ((1, 0), (3, 0), (5, 4), (4096, 0), (4097, 0), (70_001, 0), (128 * 40000, 0), (128 * 40000, 1),
+                           ((1 << 24) + 3, 4), (big, 0)):
+                if spins == 0 and n > (1 << 23):
+                    continue  # a workgroup on its own reads the whole tensor: keep that to small inputs
+                x = bt[off:off + n]
+                codes, prec = cn.absmax_compression_8bit(x)
+                want_prec = cn.absmax(x)
+                want = cn.compression_8bit(x, want_prec)
+                assert torch.equal(prec.view(torch.int32), want_prec.view(torch.int32)), (spins, n, off)
+                assert torch.equal(codes, want), (spins, n, off)
+                if n <= 128 * 40000:
+                    p = float(np.abs(base[off:off + n]).max())
+                    assert float(prec.cpu()[0]) == p
+                    assert np.array_equal(codes.cpu().numpy(), oracle.port_compress(base[off:off + n], p)), (spins, n, off)
+            z = torch.zeros(10_000, device=dev)
+            codes, prec = cn.absmax_compression_8bit(z)
+            assert float(prec.cpu()[0]) == 0.0 and np.array_equal(codes.cpu().numpy(), oracle.compress(np.zeros(10_000, np.float32), 0.0))
+            y = bt[:50_000].clone()
+            y[12_345] = float("nan")
+            codes, prec = cn.absmax_compression_8bit(y)
+            assert np.isnan(float(prec.cpu()[0]))
+            with np.errstate(all="ignore"):
+                assert np.array_equal(codes.cpu().numpy(), oracle.compress(y.cpu().numpy(), float("nan")))
+            codes, prec = cn.absmax_compression_8bit(bt[:0])
+            assert float(prec.cpu()[0]) == -1.0 and codes.numel() == 0
+    finally:
+        L.lib().cn_host_absmax_compress_spin_limit(-1)
+        L.lib().cn_host_absmax_compress_single_launch(0)
