@@ -124,6 +124,88 @@ def test_product_with_expansion_equals_the_two_calls(dev, M, N, K, pool):
     assert cn.lib().cn_gemm_f32_expand_maxout_grad(0, 1, 4, 6, 4, None, 4, None, 4, None, 2, None, None) == 1
 
 
+def _maxout_against_checker(out, arg, z64, tol_abs, pool):
+    """out / arg of a fused product + bias + maxout against the pre-activations z64 of the CPU checker (float64,
+    M x N): the value is the maximum of its pool within the product tolerance, the stored winner lies in its pool and
+    is a maximiser up to that tolerance, and the value is the pre-activation at the stored winner."""
+    M, N = z64.shape
+    groups = z64.reshape(M, N // pool, pool)
+    best = groups.max(axis=2)
+    assert np.all(np.abs(out.astype(np.float64) - best) <= tol_abs), float(np.abs(out - best).max())
+    a = arg.astype(np.int64)
+    base = (np.arange(N // pool, dtype=np.int64) * pool)[None, :]
+    assert np.array_equal(arg, a.astype(np.float32)) and np.all(a >= base) and np.all(a < base + pool)
+    at_winner = np.take_along_axis(z64, a.reshape(M, -1), axis=1).reshape(M, N // pool)
+    assert np.all(best - at_winner <= 2 * tol_abs)
+    assert np.all(np.abs(out.astype(np.float64) - at_winner) <= tol_abs)
+    # where the pool has a clear winner (margin above the tolerance) the stored winner is that one
+    order = np.sort(groups, axis=2)
+    clear = (order[:, :, -1] - order[:, :, -2]) > 2 * tol_abs
+    assert np.array_equal(a[clear], (base + groups.argmax(axis=2))[clear])
+    assert clear.mean() > 0.9
+
+
+def test_forward_of_a_maxout_layer_against_the_checker_at_full_size(dev):
+    """cn_gemm_f32_bias_maxout at the shapes of the training configuration, straight against the CPU checker (fp64
+    product + bias + maxout) instead of against the unfused HIP calls: the second layer 128 x 8192 x 4096 in full,
+    and a first layer at a quarter of its depth, 128 x 8192 x 25000, on 512 sampled pools."""
+    import torch
+    from clusternet_amd import _lib as L
+    from util import gemm_tolerance
+    rng = np.random.default_rng(2027)
+    pool = 2
+    M, N, K = 128, 8192, 4096
+    A = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = rng.uniform(-0.022, 0.022, (K, N)).astype(np.float32)
+    b = rng.normal(0, 0.05, N).astype(np.float32)
+    out, arg = L.dot_bias_maxout(_t(A, dev), _t(W, dev), _t(b, dev), pool)
+    C, Cabs = oracle.gemm_with_abs(A, W)
+    z = C.astype(np.float64) + b.astype(np.float64)[None, :]
+    tol = gemm_tolerance(K) * float(Cabs.max())
+    _maxout_against_checker(out.cpu().numpy(), arg.cpu().numpy(), z, tol, pool)
+
+    K = 25000
+    A = (rng.uniform(0, 1, (M, K)) * (rng.uniform(0, 1, (M, K)) < 0.02)).astype(np.float32)
+    W = rng.uniform(-0.0074, 0.0074, (K, N)).astype(np.float32)
+    out, arg = L.dot_bias_maxout(_t(A, dev), _t(W, dev), _t(b, dev), pool)
+    pools = np.sort(rng.choice(N // pool, 512, replace=False))
+    cols = (pools[:, None] * pool + np.arange(pool)[None, :]).reshape(-1)
+    C, Cabs = oracle.gemm_cols(A, W, cols)
+    z = C + b.astype(np.float64)[cols][None, :]
+    tol = gemm_tolerance(K) * float(Cabs.max())
+    got_out = out.cpu().numpy()[:, pools]
+    got_arg = arg.cpu().numpy()[:, pools]
+    # renumber the sampled pools' winners into the sampled column space
+    local = (got_arg.astype(np.int64) - (pools * pool)[None, :]) + (np.arange(pools.size) * pool)[None, :]
+    _maxout_against_checker(got_out, local.astype(np.float32), z, tol, pool)
+
+
+def test_backward_through_a_maxout_layer_against_the_checker_at_full_size(dev):
+    """cn_gemm_f32_expand_maxout_grad at the training configuration's 128 x 4096 x 8192 (the input-gradient product
+    of the second layer, scattered to the winners of the first), straight against the CPU checker."""
+    import torch
+    from clusternet_amd import _lib as L
+    from util import gemm_errors, gemm_tolerance
+    rng = np.random.default_rng(2028)
+    pool = 2
+    M, N, K = 128, 4096, 8192
+    E = rng.normal(0, 0.01, (M, K)).astype(np.float32)
+    W = rng.uniform(-0.022, 0.022, (N, K)).astype(np.float32)
+    winners = (np.arange(N) * pool)[None, :] + rng.integers(0, pool, (M, N))
+    argmax = winners.astype(np.float32)
+    got = L.dotT_expand_to_maxout_grad(_t(E, dev), _t(W, dev), _t(argmax, dev), pool).cpu().numpy()
+    C, Cabs = oracle.gemm_with_abs(E, W, False, True)
+    assert got.shape == (M, N * pool)
+    at = np.take_along_axis(got, winners, axis=1)
+    e1, e2 = gemm_errors(at, C, Cabs)
+    assert e1 <= gemm_tolerance(K) and e2 <= gemm_tolerance(K), (e1, e2)
+    mask = np.ones_like(got, bool)
+    np.put_along_axis(mask, winners, False, axis=1)
+    assert np.all(got[mask].view(np.uint32) == 0)            # +0.0 everywhere else
+    want = oracle.expand_to_maxout_grad(C.astype(np.float32), argmax, pool)
+    assert np.array_equal(want != 0, (~mask) & (want != 0))   # the checker scatters to the same places
+
+
 def _cpu_step(X, onehot, params, rate, pool):
     W1, b1, W2, b2, W3, b3 = params
     z1 = oracle.add_row_vector(oracle.gemm(X, W1), b1)
