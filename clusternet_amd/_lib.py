@@ -81,6 +81,8 @@ def lib():
     L.cn_host_plan_gemm.restype = None
     L.cn_host_force_gemm_tile_n.argtypes = [C.c_int]
     L.cn_host_force_gemm_tile_n.restype = None
+    L.cn_host_gemm_epilogue_in_kernel.argtypes = [C.c_int]
+    L.cn_host_gemm_epilogue_in_kernel.restype = None
     L.cn_host_gemm_wide_store.argtypes = [C.c_int]
     L.cn_host_gemm_wide_store.restype = None
     L.cn_host_reduction_fences.argtypes = [C.c_int]

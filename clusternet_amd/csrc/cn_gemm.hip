@@ -92,7 +92,16 @@ struct GemmArgs {
     const float *table;  // fused: 126-entry codebook
     uint32_t *amax;      // optional: receives max |C| as the bit pattern of a non-negative float
     int wide_store;      // the destination of the write-out (C, or the partial planes) allows 16-byte stores
+    // What the write-out does instead of storing C when the kernel is instantiated with an epilogue (whole tiles
+    // only, K not split): bias + maxout over epi_pool consecutive columns into epi_out / epi_arg_out (M x N / pool),
+    // or the expansion of the product (M x N) to the winners' columns epi_arg_in names, into epi_out (M x N pool).
+    const float *epi_bias;
+    const float *epi_arg_in;
+    float *epi_out;
+    float *epi_arg_out;
+    int epi_pool;
 };
+enum Epilogue { EPI_NONE = 0, EPI_BIAS_MAXOUT = 1, EPI_EXPAND = 2 };
 
 // max over the wavefront of a non-negative float's bit pattern, then one atomic per wavefront.
 // Bit patterns of non-negative floats order like the floats, so the unsigned maximum is exact and
@@ -278,7 +287,7 @@ struct GuardedIC {
     }
 };
 
-template <bool A_KC, int B_KIND, int TN, int TM>
+template <bool A_KC, int B_KIND, int TN, int TM, int EPI = EPI_NONE>
 __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
     using G = Geo<TM, TN>;
     constexpr int BM = TM;
@@ -654,16 +663,87 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
                     const uint32_t bits = __float_as_uint(acc[mi][ni][r]) & 0x7fffffffu;
                     amax = bits > amax ? bits : amax;
                 }
-                float *corner = dst + (m0 + wave_m * (32 * FM) + mi * 32) * ldd + n0 + wave_n * (32 * FN) + ni * 32 + pcol;
+                if (EPI == EPI_NONE) {
+                    float *corner = dst + (m0 + wave_m * (32 * FM) + mi * 32) * ldd + n0 + wave_n * (32 * FN) + ni * 32 + pcol;
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(patch + (prow + 8 * k) * kPatchLd + pcol);
-                    // the result itself is not read again soon; the partial planes are, by the chunk sum
-                    if (g.splits == 1) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(corner + (int64_t)(prow + 8 * k) * ldd));
-                    else               *reinterpret_cast<f32x4 *>(corner + (int64_t)(prow + 8 * k) * ldd) = v;
+                    for (int k = 0; k < 4; ++k) {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(patch + (prow + 8 * k) * kPatchLd + pcol);
+                        // the result itself is not read again soon; the partial planes are, by the chunk sum
+                        if (g.splits == 1) __builtin_nontemporal_store(v, reinterpret_cast<f32x4 *>(corner + (int64_t)(prow + 8 * k) * ldd));
+                        else               *reinterpret_cast<f32x4 *>(corner + (int64_t)(prow + 8 * k) * ldd) = v;
+                    }
+                } else {
+                    // The lane holds four consecutive columns of a row: the pools of 2 or 4 columns that the bias
+                    // and the maximum go over, or the four pooled units whose error is spread to their winners,
+                    // lie inside its own 16 bytes.  Same operations, in the same order, as the kernels that would
+                    // follow the stored product (add_row_vector then maxout; expand_to_maxout_grad).
+                    const int64_t col = n0 + wave_n * (32 * FN) + ni * 32 + pcol;
+                    const int pool = g.epi_pool;
+                    f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
+                    if (EPI == EPI_BIAS_MAXOUT) bias4 = *reinterpret_cast<const f32x4 *>(g.epi_bias + col);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int64_t row = m0 + wave_m * (32 * FM) + mi * 32 + prow + 8 * k;
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(patch + (prow + 8 * k) * kPatchLd + pcol);
+                        if (EPI == EPI_BIAS_MAXOUT) {
+                            const f32x4 z = {v.x + bias4.x, v.y + bias4.y, v.z + bias4.z, v.w + bias4.w};
+                            const int64_t at = row * (g.N / pool) + col / pool;
+                            if (pool == 2) {
+                                float b0 = z.x, b1 = z.z;
+                                int a0 = 0, a1 = 0;
+                                if (b0 < z.y) { b0 = z.y; a0 = 1; }
+                                if (b1 < z.w) { b1 = z.w; a1 = 1; }
+                                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                                __builtin_nontemporal_store(f32x2{b0, b1}, reinterpret_cast<f32x2 *>(g.epi_out + at));
+                                __builtin_nontemporal_store(f32x2{(float)(col + a0), (float)(col + 2 + a1)},
+                                                            reinterpret_cast<f32x2 *>(g.epi_arg_out + at));
+                            } else if (pool == 4) {
+                                float b = z.x;
+                                int a = 0;
+                                if (b < z.y) { b = z.y; a = 1; }
+                                if (b < z.z) { b = z.z; a = 2; }
+                                if (b < z.w) { b = z.w; a = 3; }
+                                g.epi_out[at] = b;
+                                g.epi_arg_out[at] = (float)(col + a);
+                            } else {  // pool 1: every column its own winner
+                                __builtin_nontemporal_store(z, reinterpret_cast<f32x4 *>(g.epi_out + at));
+                                __builtin_nontemporal_store(f32x4{(float)col, (float)(col + 1), (float)(col + 2), (float)(col + 3)},
+                                                            reinterpret_cast<f32x4 *>(g.epi_arg_out + at));
+                            }
+                        } else {
+                            const f32x4 winner = *reinterpret_cast<const f32x4 *>(g.epi_arg_in + row * g.N + col);
+                            float *to = g.epi_out + (row * g.N + col) * pool;
+                            if (pool == 2) {
+                                f32x4 lo, hi;
+                                lo.x = ((int64_t)winner.x == col * 2 + 0) ? v.x : 0.0f;
+                                lo.y = ((int64_t)winner.x == col * 2 + 1) ? v.x : 0.0f;
+                                lo.z = ((int64_t)winner.y == col * 2 + 2) ? v.y : 0.0f;
+                                lo.w = ((int64_t)winner.y == col * 2 + 3) ? v.y : 0.0f;
+                                hi.x = ((int64_t)winner.z == col * 2 + 4) ? v.z : 0.0f;
+                                hi.y = ((int64_t)winner.z == col * 2 + 5) ? v.z : 0.0f;
+                                hi.z = ((int64_t)winner.w == col * 2 + 6) ? v.w : 0.0f;
+                                hi.w = ((int64_t)winner.w == col * 2 + 7) ? v.w : 0.0f;
+                                __builtin_nontemporal_store(lo, reinterpret_cast<f32x4 *>(to));
+                                __builtin_nontemporal_store(hi, reinterpret_cast<f32x4 *>(to + 4));
+                            } else if (pool == 4) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) {
+                                    const int64_t c0 = (col + e) * 4;
+                                    const int64_t w = (int64_t)winner[e];
+                                    const f32x4 o = {w == c0 ? v[e] : 0.0f, w == c0 + 1 ? v[e] : 0.0f, w == c0 + 2 ? v[e] : 0.0f,
+                                                     w == c0 + 3 ? v[e] : 0.0f};
+                                    __builtin_nontemporal_store(o, reinterpret_cast<f32x4 *>(to + 4 * e));
+                                }
+                            } else {  // pool 1
+                                const f32x4 o = {(int64_t)winner.x == col ? v.x : 0.0f, (int64_t)winner.y == col + 1 ? v.y : 0.0f,
+                                                 (int64_t)winner.z == col + 2 ? v.z : 0.0f, (int64_t)winner.w == col + 3 ? v.w : 0.0f};
+                                __builtin_nontemporal_store(o, reinterpret_cast<f32x4 *>(to));
+                            }
+                        }
+                    }
                 }
             }
-    } else {
+    } else if (EPI == EPI_NONE) {  // a kernel with an epilogue is only launched on whole tiles
 #pragma unroll
         for (int mi = 0; mi < FM; ++mi)
 #pragma unroll
@@ -814,7 +894,7 @@ cn_status add_chunk_planes(const void *planes, int num_cu, int splits, int64_t M
     return CN_OK;
 }
 
-template <bool A_KC, int B_KIND, int TN, int TM>
+template <bool A_KC, int B_KIND, int TN, int TM, int EPI = EPI_NONE>
 static cn_status launch_tile(const GemmArgs &args, int device, hipStream_t st) {
     using G = Geo<TM, TN>;
     // the stages, the decode table of the fused variant, and at least the four write-out patches
@@ -822,10 +902,10 @@ static cn_status launch_tile(const GemmArgs &args, int device, hipStream_t st) {
     if (lds < NW * 32 * 36 * sizeof(float)) lds = NW * 32 * 36 * sizeof(float);
     static OncePerDevice configured;
     if (configured.first(device)) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN, TM>),
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_kernel<A_KC, B_KIND, TN, TM, EPI>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     }
-    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN, TM>), dim3(args.units), dim3(NT), lds, st, args);
+    hipLaunchKernelGGL((gemm_kernel<A_KC, B_KIND, TN, TM, EPI>), dim3(args.units), dim3(NT), lds, st, args);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -840,6 +920,7 @@ static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, 
 
 static int g_force_tile_n = 0;
 static bool g_wide_store = true;
+static bool g_epilogue_in_kernel = true;  // test hook: false sends every fused product through the workspace
 
 // What follows the product instead of its delivery: bias and maxout (the forward pass of a maxout layer; `bias`
 // given, out and argmax M x N / pool), or the expansion of a pooled error to the winners' columns (its backward
@@ -903,7 +984,14 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         return CN_OK;
     }
     GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->plan_bytes, g_force_tile_n);
-    if (then && plan.splits == 1) {
+    // K not split, whole 128-row tiles and pools of 1, 2 or 4: bias + maxout, or the expansion, happen in the
+    // product's own write-out and the product never exists in memory (dot for the forward pass, dotT for the
+    // backward one; the other transpositions go through the workspace like ragged shapes).
+    const bool in_write_out =
+        then && g_epilogue_in_kernel && !w8 && plan.splits == 1 && plan.tile_m == kTileM && M % kTileM == 0 && N % plan.tile_n == 0 &&
+        (then->pool == 1 || then->pool == 2 || then->pool == 4) && !ta && (then->bias ? !tb : tb) && aligned(then->out, 16) &&
+        aligned(then->argmax, 16) && (!then->bias || aligned(then->bias, 16));
+    if (then && plan.splits == 1 && !in_write_out) {
         // no chunk sum to fold into: the product goes to the workspace and one pass over it follows
         if ((size_t)M * (size_t)N * sizeof(float) > ctx->workspace_bytes) {
             set_error("%s: product does not fit the workspace", who);
@@ -934,6 +1022,19 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.amax = amax;
     a.wide_store = g_wide_store && (plan.splits > 1 ? (N % 4 == 0 && (M * N) % 4 == 0)
                                                      : (aligned(C, 16) && ldc % 4 == 0));
+    a.epi_bias = nullptr; a.epi_arg_in = nullptr; a.epi_out = nullptr; a.epi_arg_out = nullptr; a.epi_pool = 1;
+    if (in_write_out) {
+        a.wide_store = 1;  // the tiles leave through the LDS patch whatever C would have allowed
+        a.epi_pool = then->pool;
+        a.epi_out = then->out;
+        if (then->bias) { a.epi_bias = then->bias; a.epi_arg_out = then->argmax; }
+        else            { a.epi_arg_in = then->argmax; }
+        if (then->bias)
+            return plan.tile_n == 256 ? launch_tile<true, B_IC, 256, kTileM, EPI_BIAS_MAXOUT>(a, ctx->device, st)
+                                      : launch_tile<true, B_IC, 128, kTileM, EPI_BIAS_MAXOUT>(a, ctx->device, st);
+        return plan.tile_n == 256 ? launch_tile<true, B_KC, 256, kTileM, EPI_EXPAND>(a, ctx->device, st)
+                                  : launch_tile<true, B_KC, 128, kTileM, EPI_EXPAND>(a, ctx->device, st);
+    }
 
     if (w8)              s = launch<true, B_CODES>(a, plan, ctx->device, st);
     else if (!ta && !tb) s = launch<true, B_IC>(a, plan, ctx->device, st);
@@ -997,6 +1098,9 @@ extern "C" {
 
 // Test hook: 0 = write every tile with 4-byte stores.
 void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
+
+// Test hook: 0 = bias + maxout and the maxout expansion never run inside the product's write-out.
+void cn_host_gemm_epilogue_in_kernel(int enabled) { g_epilogue_in_kernel = enabled != 0; }
 
 // Test and tuning hook: 0 = let the planner choose the tile, 128 / 256 = force that width of the 128-row
 // tile, 32 / 64 = force the 32 x 128 / 64 x 128 tile.

@@ -40,28 +40,65 @@ __global__ __launch_bounds__(kT) void transpose_kernel(const float *__restrict__
     }
 }
 
-__global__ __launch_bounds__(kT) void affine_kernel(const float *__restrict__ x, float mul, float add, int64_t n,
-                                                    float *__restrict__ out) {
-    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
-        out[i] = x[i] * mul + add;
+// Flat element-wise passes: out[i] = f(a[i], b[i]).  With 16-byte aligned arrays every lane moves 16-byte vectors
+// (non-temporal: nothing is reused), four of each input in flight before the first is consumed; otherwise, and
+// for the last n % 4 elements, element by element.  Each f is the single fp32 expression of its reference routine.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+struct AffineOp { float mul, add; __device__ float operator()(float x, float) const { return x * mul + add; } };
+struct AbsOp { __device__ float operator()(float x, float) const { return fabsf(x); } };
+struct SubOp { __device__ float operator()(float a, float b) const { return a - b; } };
+struct SgdOp { float rate; __device__ float operator()(float w, float g) const { return w - rate * g; } };
+
+template <class Op, bool kTwo, bool kVector>
+__global__ __launch_bounds__(kT) void flat_kernel(const float *a, const float *b, int64_t n, float *out, Op f) {
+    if (kVector) {
+        constexpr int kU = 4;
+        const int64_t nvec = n / 4, tiles = (nvec + kT * kU - 1) / (kT * kU);
+        const f32x4_t *a4 = reinterpret_cast<const f32x4_t *>(a), *b4 = reinterpret_cast<const f32x4_t *>(b);
+        f32x4_t *o4 = reinterpret_cast<f32x4_t *>(out);
+        for (int64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+            const int64_t base = tile * (kT * kU) + threadIdx.x;
+            f32x4_t va[kU], vb[kU];
+#pragma unroll
+            for (int j = 0; j < kU; ++j) {
+                const int64_t i = base + (int64_t)j * kT;
+                va[j] = i < nvec ? __builtin_nontemporal_load(&a4[i]) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+                if (kTwo) vb[j] = i < nvec ? __builtin_nontemporal_load(&b4[i]) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int j = 0; j < kU; ++j) {
+                const int64_t i = base + (int64_t)j * kT;
+                f32x4_t o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = f(va[j][e], kTwo ? vb[j][e] : 0.0f);
+                if (i < nvec) __builtin_nontemporal_store(o, &o4[i]);
+            }
+        }
+        if (blockIdx.x == 0) {
+            const int64_t i = nvec * 4 + threadIdx.x;
+            if (i < n) out[i] = f(a[i], kTwo ? b[i] : 0.0f);
+        }
+    } else {
+        for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
+            out[i] = f(a[i], kTwo ? b[i] : 0.0f);
+    }
 }
 
-__global__ __launch_bounds__(kT) void abs_kernel(const float *__restrict__ x, int64_t n, float *__restrict__ out) {
-    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
-        out[i] = fabsf(x[i]);
-}
-
-__global__ __launch_bounds__(kT) void sub_kernel(const float *__restrict__ a, const float *__restrict__ b, int64_t n,
-                                                 float *__restrict__ out) {
-    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
-        out[i] = a[i] - b[i];
-}
-
-// w[i] -= rate * g[i]
-__global__ __launch_bounds__(kT) void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, float rate,
-                                                 int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT)
-        w[i] = w[i] - rate * g[i];
+template <class Op, bool kTwo>
+static cn_status launch_flat(Context *ctx, hipStream_t st, const float *a, const float *b, int64_t n, float *out, Op f) {
+    auto ok16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    const bool vec = ok16(a) && ok16(out) && (!kTwo || ok16(b));
+    if (vec) {
+        int64_t tiles = (n / 4 + kT * 4 - 1) / (kT * 4), cap = (int64_t)ctx->num_cu * 8;
+        const int64_t grid = tiles < 1 ? 1 : (tiles < cap ? tiles : cap);
+        hipLaunchKernelGGL((flat_kernel<Op, kTwo, true>), dim3((unsigned)grid), dim3(kT), 0, st, a, b, n, out, f);
+    } else {
+        int64_t blocks = (n + kT - 1) / kT, cap = (int64_t)ctx->num_cu * 8;
+        const int64_t grid = blocks < 1 ? 1 : (blocks < cap ? blocks : cap);
+        hipLaunchKernelGGL((flat_kernel<Op, kTwo, false>), dim3((unsigned)grid), dim3(kT), 0, st, a, b, n, out, f);
+    }
+    CN_HIP(hipGetLastError());
+    return CN_OK;
 }
 
 // out[r][c] = A[r][c] + v[c]
@@ -248,36 +285,28 @@ cn_status cn_affine_f32(const float *x, float mul, float add, size_t n, float *o
     if (n == 0) return CN_OK;
     CN_REQUIRE(x && out, CN_ERR_NULL, "affine_f32: NULL pointer");
     CN_ENTER();
-    hipLaunchKernelGGL(affine_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, x, mul, add, (int64_t)n, out);
-    CN_HIP(hipGetLastError());
-    return CN_OK;
+    return launch_flat<AffineOp, false>(ctx, st, x, nullptr, (int64_t)n, out, AffineOp{mul, add});
 }
 
 cn_status cn_abs_f32(const float *x, size_t n, float *out, void *stream) {
     if (n == 0) return CN_OK;
     CN_REQUIRE(x && out, CN_ERR_NULL, "abs_f32: NULL pointer");
     CN_ENTER();
-    hipLaunchKernelGGL(abs_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, x, (int64_t)n, out);
-    CN_HIP(hipGetLastError());
-    return CN_OK;
+    return launch_flat<AbsOp, false>(ctx, st, x, nullptr, (int64_t)n, out, AbsOp{});
 }
 
 cn_status cn_sub_f32(const float *a, const float *b, size_t n, float *out, void *stream) {
     if (n == 0) return CN_OK;
     CN_REQUIRE(a && b && out, CN_ERR_NULL, "sub_f32: NULL pointer");
     CN_ENTER();
-    hipLaunchKernelGGL(sub_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, a, b, (int64_t)n, out);
-    CN_HIP(hipGetLastError());
-    return CN_OK;
+    return launch_flat<SubOp, true>(ctx, st, a, b, (int64_t)n, out, SubOp{});
 }
 
 cn_status cn_sgd_update_f32(float *w, const float *grad, float rate, size_t n, void *stream) {
     if (n == 0) return CN_OK;
     CN_REQUIRE(w && grad, CN_ERR_NULL, "sgd_update_f32: NULL pointer");
     CN_ENTER();
-    hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(ctx, (int64_t)n)), dim3(kT), 0, st, w, grad, rate, (int64_t)n);
-    CN_HIP(hipGetLastError());
-    return CN_OK;
+    return launch_flat<SgdOp, true>(ctx, st, w, grad, (int64_t)n, w, SgdOp{rate});
 }
 
 cn_status cn_add_row_vector_f32(const float *A, const float *v, int64_t rows, int64_t cols, float *out, void *stream) {

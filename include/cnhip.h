@@ -293,8 +293,9 @@ cn_status cn_add_row_vector_f32(const float *A_device, const float *v_device, in
                                 int64_t cols, float *out_device, void *stream);
 /* out, argmax = maxout(op(A) op(B) + bias): cn_gemm_f32, cn_add_row_vector_f32 and cn_maxout_f32 as one call, the
  * forward pass of a maxout layer (source/Layer.cpp:256-258: dot, addMatrixVector, maxout).  Where the product is
- * summed over chunks of K, bias and maxout ride on that sum and the product never reaches memory as a whole;
- * elsewhere it passes through the library's workspace (CN_ERR_WORKSPACE if it does not fit).  out and argmax are
+ * summed over chunks of K, bias and maxout ride on that sum; where K is not split, the tiles are whole and the pool
+ * is 1, 2 or 4, they happen in the product's own write-out; either way the product never reaches memory as a whole.
+ * Other shapes pass through the library's workspace (CN_ERR_WORKSPACE if it does not fit).  out and argmax are
  * M x N / pool, contiguous; same bits as the three calls. */
 cn_status cn_gemm_f32_bias_maxout(int trans_a, int trans_b, int64_t M, int64_t N, int64_t K, const float *A_device,
                                   int64_t lda, const float *B_device, int64_t ldb, const float *bias_device, int pool,

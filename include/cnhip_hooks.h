@@ -29,6 +29,11 @@ void cn_host_force_gemm_tile_n(int tile_n);
 /* 0 = every output tile is written with 4-byte stores (the path that unaligned outputs take). */
 void cn_host_gemm_wide_store(int enabled);
 
+/* 0 = cn_gemm_f32_bias_maxout / cn_gemm_f32_expand_maxout_grad never take the kernel that applies them in the
+ * product's own write-out (K not split, whole tiles): they then pass through the workspace, which the tests compare
+ * against. */
+void cn_host_gemm_epilogue_in_kernel(int enabled);
+
 /* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
 void cn_host_codec_workgroups_per_cu(int per_cu);
 

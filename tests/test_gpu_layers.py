@@ -53,6 +53,26 @@ def test_helpers_match_checker(dev):
     assert arg.cpu().numpy().tolist() == [[0.0, 3.0]]
 
 
+def test_flat_passes_on_ragged_sizes_and_unaligned_starts(dev):
+    """sub and the plain update on 16-byte vectors where the arrays allow it and element by element where they do
+    not: every size around a vector and a tile boundary, starts that are and are not 16-byte aligned, in place."""
+    import torch
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(4)
+    A = rng.normal(0, 1, 70_000).astype(np.float32)
+    B = rng.normal(0, 1, 70_000).astype(np.float32)
+    At, Bt = _t(A, dev), _t(B, dev)
+    for n in (1, 3, 4, 5, 1023, 1024, 4095, 4096, 4097, 16_385, 65_537):
+        for oa, ob in ((0, 0), (4, 8), (1, 0), (0, 3), (2, 2)):
+            got = L.sub(At[oa:oa + n], Bt[ob:ob + n]).cpu().numpy()
+            assert np.array_equal(got, A[oa:oa + n] - B[ob:ob + n]), (n, oa, ob)
+            w = At.clone()
+            L.sgd_update(w[oa:oa + n], Bt[ob:ob + n], 0.375)
+            want = A.copy()
+            want[oa:oa + n] = A[oa:oa + n] - np.float32(0.375) * B[ob:ob + n]
+            assert np.array_equal(w.cpu().numpy(), want), (n, oa, ob)
+
+
 @pytest.mark.parametrize("rows,cols,pool", [(128, 8192, 2), (7, 12, 3), (33, 260, 4), (1, 2, 1), (5, 64, 64)])
 def test_bias_and_maxout_in_one_pass_equal_the_two_kernels(dev, rows, cols, pool):
     import torch
@@ -124,6 +144,59 @@ def test_product_with_expansion_equals_the_two_calls(dev, M, N, K, pool):
     assert cn.lib().cn_gemm_f32_expand_maxout_grad(0, 1, 4, 6, 4, None, 4, None, 4, None, 2, None, None) == 1
 
 
+@pytest.mark.parametrize("M,N,K,pool", [(256, 512, 64, 2), (128, 1024, 100, 4), (384, 256, 33, 1), (2048, 4096, 64, 2),
+                                        (1024, 2048, 120, 4)])
+def test_bias_maxout_and_expansion_inside_the_write_out_of_an_unsplit_product(dev, M, N, K, pool):
+    """Where K is not split and the tiles are whole, bias + maxout (forward, dot) and the expansion to the winners'
+    columns (backward, dotT) happen in the product kernel's own write-out.  Same bits as the path through the
+    workspace (the hook switches the write-out form off) and as the separate calls, on both 128-row tile widths;
+    values against the CPU checker."""
+    import ctypes
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    from util import gemm_errors
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    gen = torch.Generator(device=dev).manual_seed(M + 7 * N + K)
+    A = torch.randn((M, K), device=dev, generator=gen)
+    B = torch.randn((K, N), device=dev, generator=gen) * 0.05
+    v = torch.randn(N, device=dev, generator=gen) * 0.1
+    NE = N // 4                                   # pooled units of the backward case
+    E = torch.randn((M, K), device=dev, generator=gen)
+    W = torch.randn((NE, K), device=dev, generator=gen) * 0.05
+    winners = (torch.arange(NE, device=dev) * pool)[None, :] + torch.randint(0, pool, (M, NE), device=dev, generator=gen)
+    argmax = winners.to(torch.float32)
+    try:
+        for force in (128, 256, 0):
+            plan = (ctypes.c_int64 * 8)()
+            cn.lib().cn_host_plan_gemm(M, N, K, cus, 1 << 30, force, plan)
+            assert plan[3] == 1, "the case is meant not to split K"
+            cn.lib().cn_host_force_gemm_tile_n(force)
+            results = []
+            for in_kernel in (1, 0):
+                cn.lib().cn_host_gemm_epilogue_in_kernel(in_kernel)
+                out, arg = L.dot_bias_maxout(A, B, v, pool)
+                back = L.dotT_expand_to_maxout_grad(E, W, argmax, pool)
+                results.append((out, arg, back))
+            for a, b in zip(results[0], results[1]):
+                assert torch.equal(a.view(torch.int32), b.view(torch.int32)), force
+            want_out, want_arg = L.maxout(L.add_row_vector(L.dot(A, B), v), pool)
+            assert torch.equal(results[0][0].view(torch.int32), want_out.view(torch.int32)) and torch.equal(results[0][1], want_arg)
+            want_back = L.expand_to_maxout_grad(L.dotT(E, W), argmax, pool)
+            assert torch.equal(results[0][2].view(torch.int32), want_back.view(torch.int32)), force
+    finally:
+        cn.lib().cn_host_gemm_epilogue_in_kernel(1)
+        cn.lib().cn_host_force_gemm_tile_n(0)
+    if M * N <= 1 << 20:
+        C, Cabs = oracle.gemm_with_abs(A.cpu().numpy(), B.cpu().numpy())
+        z = C.astype(np.float64) + v.cpu().numpy().astype(np.float64)[None, :]
+        _maxout_against_checker(results[0][0].cpu().numpy(), results[0][1].cpu().numpy(), z, 1e-4 * float(Cabs.max()), pool)
+        Cb, Cbabs = oracle.gemm_with_abs(E.cpu().numpy(), W.cpu().numpy(), False, True)
+        at = np.take_along_axis(results[0][2].cpu().numpy(), winners.cpu().numpy(), axis=1)
+        e1, e2 = gemm_errors(at, Cb, Cbabs)
+        assert e1 <= 1e-4 and e2 <= 1e-4
+
+
 def _maxout_against_checker(out, arg, z64, tol_abs, pool):
     """out / arg of a fused product + bias + maxout against the pre-activations z64 of the CPU checker (float64,
     M x N): the value is the maximum of its pool within the product tolerance, the stored winner lies in its pool and
@@ -139,10 +212,11 @@ def _maxout_against_checker(out, arg, z64, tol_abs, pool):
     assert np.all(best - at_winner <= 2 * tol_abs)
     assert np.all(np.abs(out.astype(np.float64) - at_winner) <= tol_abs)
     # where the pool has a clear winner (margin above the tolerance) the stored winner is that one
-    order = np.sort(groups, axis=2)
-    clear = (order[:, :, -1] - order[:, :, -2]) > 2 * tol_abs
-    assert np.array_equal(a[clear], (base + groups.argmax(axis=2))[clear])
-    assert clear.mean() > 0.9
+    if pool > 1:
+        order = np.sort(groups, axis=2)
+        clear = (order[:, :, -1] - order[:, :, -2]) > 2 * tol_abs
+        assert np.array_equal(a[clear], (base + groups.argmax(axis=2))[clear])
+        assert clear.mean() > 0.9
 
 
 def test_forward_of_a_maxout_layer_against_the_checker_at_full_size(dev):
