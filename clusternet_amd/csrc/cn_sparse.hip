@@ -92,22 +92,24 @@ __global__ __launch_bounds__(kT) void zero_counts_kernel(int32_t *__restrict__ c
 // table across wavefronts.
 __global__ __launch_bounds__(kT) void scan_kernel(const int32_t *counts, int64_t n, int32_t *row_ptr,
                                                   int64_t *__restrict__ total) {
-    __shared__ int wave_sum[kT / 64];
+    // Sums are carried in 64 bits throughout: the entries may themselves be sums of blocks (up to 2^24 each), so a
+    // tile of 256 can pass 2^31, and *total must stay exact for the callers that refuse more than 2^31 - 1 nonzeros.
+    __shared__ long long wave_sum[kT / 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     int64_t carry = 0;
     for (int64_t i0 = 0; i0 < n; i0 += kT) {
         const int64_t i = i0 + threadIdx.x;
-        const int c = (i < n) ? counts[i] : 0;
-        int inc = c;  // inclusive scan within the wavefront
+        const long long c = (i < n) ? counts[i] : 0;
+        long long inc = c;  // inclusive scan within the wavefront
         for (int off = 1; off < 64; off <<= 1) {
-            const int up = __shfl_up(inc, off, 64);
+            const long long up = __shfl_up(inc, off, 64);
             if (lane >= off) inc += up;
         }
         if (lane == 63) wave_sum[wave] = inc;
         __syncthreads();
-        int before = 0;
+        long long before = 0;
         for (int w = 0; w < wave; ++w) before += wave_sum[w];
-        const int tile_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+        const long long tile_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
         if (i < n) row_ptr[i] = (int32_t)(carry + before + inc - c);
         carry += tile_total;
         __syncthreads();
@@ -837,40 +839,43 @@ __global__ __launch_bounds__(kCodedThreads) void csr_gemm_coded_kernel(
 }
 
 // ---- CSR(S) -> CSR(S^T) ------------------------------------------------------------------------------------
-// Histogram of the column indices, prefix sums, a fill in arbitrary order, then every row of the
-// result is sorted by its (few) column indices: the result does not depend on the order of the fill.
-__global__ __launch_bounds__(kT) void histogram_kernel(const int32_t *__restrict__ col_idx, int64_t nnz,
-                                                       int32_t *__restrict__ counts) {
-    for (int64_t j = (int64_t)blockIdx.x * kT + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kT)
-        atomicAdd(&counts[col_idx[j]], 1);
+// Transposition as a counting sort whose result does not depend on scheduling and needs no sorting afterwards.
+// The rows of S are cut into `blocks` blocks of `rows_per_block` consecutive rows; cursor[c * blocks + b] counts the
+// nonzeros of column c inside block b, and after a prefix sum over that array (column-major: all blocks of column 0,
+// then of column 1, ...) holds where block b's part of result row c starts.  One workgroup per block then walks its
+// rows in ascending order, a barrier between rows, so that every result row comes out in ascending column (= source
+// row) order whatever the lengths of its parts; within one source row the columns are distinct, so its nonzeros
+// take their places without atomics.  A result row of any length costs what its nonzeros cost.
+__global__ __launch_bounds__(kT) void transpose_count_kernel(int64_t R, const int32_t *__restrict__ row_ptr,
+                                                             const int32_t *__restrict__ col_idx, int64_t blocks,
+                                                             int64_t rows_per_block, int32_t *__restrict__ cursor) {
+    for (int64_t r = blockIdx.x; r < R; r += gridDim.x) {
+        const int64_t b = r / rows_per_block;
+        for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) atomicAdd(&cursor[(int64_t)col_idx[j] * blocks + b], 1);
+    }
+}
+
+__global__ __launch_bounds__(kT) void transpose_row_ptr_kernel(const int32_t *__restrict__ cursor, int64_t Cc, int64_t blocks,
+                                                               int32_t *__restrict__ t_row_ptr) {
+    for (int64_t c = (int64_t)blockIdx.x * kT + threadIdx.x; c <= Cc; c += (int64_t)gridDim.x * kT) t_row_ptr[c] = cursor[c * blocks];
 }
 
 __global__ __launch_bounds__(kT) void transpose_fill_kernel(int64_t R, const int32_t *__restrict__ row_ptr,
                                                             const int32_t *__restrict__ col_idx,
-                                                            const float *__restrict__ vals,
-                                                            int32_t *__restrict__ cursor, int32_t *__restrict__ out_col,
-                                                            float *__restrict__ out_val) {
-    // one workgroup per row of S; cursor[c] starts at the first slot of row c of the result
-    for (int64_t r = blockIdx.x; r < R; r += gridDim.x)
-        for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) {
-            const int32_t at = atomicAdd(&cursor[col_idx[j]], 1);
-            out_col[at] = (int32_t)r;
-            out_val[at] = vals[j];
-        }
-}
-
-__global__ __launch_bounds__(kT) void sort_rows_kernel(int64_t R, const int32_t *__restrict__ row_ptr,
-                                                       int32_t *__restrict__ col_idx, float *__restrict__ vals) {
-    // insertion sort of every row by column index, one thread per row
-    for (int64_t r = (int64_t)blockIdx.x * kT + threadIdx.x; r < R; r += (int64_t)gridDim.x * kT) {
-        const int32_t j0 = row_ptr[r], j1 = row_ptr[r + 1];
-        for (int32_t j = j0 + 1; j < j1; ++j) {
-            const int32_t c = col_idx[j];
-            const float v = vals[j];
-            int32_t i = j - 1;
-            while (i >= j0 && col_idx[i] > c) { col_idx[i + 1] = col_idx[i]; vals[i + 1] = vals[i]; --i; }
-            col_idx[i + 1] = c;
-            vals[i + 1] = v;
+                                                            const float *__restrict__ vals, int64_t blocks,
+                                                            int64_t rows_per_block, int32_t *cursor,
+                                                            int32_t *__restrict__ out_col, float *__restrict__ out_val) {
+    for (int64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
+        const int64_t r_end = (b + 1) * rows_per_block < R ? (b + 1) * rows_per_block : R;
+        for (int64_t r = b * rows_per_block; r < r_end; ++r) {
+            for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) {
+                int32_t *slot = &cursor[(int64_t)col_idx[j] * blocks + b];
+                const int32_t at = *slot;
+                *slot = at + 1;
+                out_col[at] = (int32_t)r;
+                out_val[at] = vals[j];
+            }
+            __syncthreads();  // the next row of the block sees the places this one took
         }
     }
 }
@@ -886,10 +891,6 @@ __global__ __launch_bounds__(kT) void csr_to_dense_kernel(int64_t R, int64_t Cc,
         for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) out[r * ldo + col_idx[j]] = vals[j];
         __syncthreads();
     }
-}
-
-__global__ __launch_bounds__(kT) void copy_i32_kernel(const int32_t *__restrict__ src, int32_t *__restrict__ dst, int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * kT + threadIdx.x; i < n; i += (int64_t)gridDim.x * kT) dst[i] = src[i];
 }
 
 // row_ptr[0 .. n] = exclusive prefix sums of counts[0 .. n - 1] (in place allowed), *total_dev = their sum.
@@ -1214,7 +1215,8 @@ cn_status cn_csr_transpose(int64_t R, int64_t Cc, int64_t nnz, const int32_t *ro
         set_error("csr_transpose: bad dimensions");
         return CN_ERR_SHAPE;
     }
-    if (!row_ptr || !t_row_ptr || (Cc > 0 && !scratch) || (nnz > 0 && (!col_idx || !vals || !t_col_idx || !t_vals))) {
+    (void)scratch;  // kept in the signature; the transposition counts in the library's workspace
+    if (!row_ptr || !t_row_ptr || (nnz > 0 && (!col_idx || !vals || !t_col_idx || !t_vals))) {
         set_error("csr_transpose: NULL pointer");
         return CN_ERR_NULL;
     }
@@ -1224,20 +1226,34 @@ cn_status cn_csr_transpose(int64_t R, int64_t Cc, int64_t nnz, const int32_t *ro
     hipStream_t st = (hipStream_t)stream;
     const int wide = ctx->num_cu * 8;
     int64_t *total_dev = reinterpret_cast<int64_t *>(ctx->sum_scratch);
-    hipLaunchKernelGGL(zero_counts_kernel, dim3(wide), dim3(kT), 0, st, t_row_ptr, Cc + 1);
-    CN_HIP(hipGetLastError());
-    if (nnz > 0) {
-        hipLaunchKernelGGL(histogram_kernel, dim3(wide), dim3(kT), 0, st, col_idx, nnz, t_row_ptr);
+    if (nnz == 0 || R == 0 || Cc == 0) {
+        hipLaunchKernelGGL(zero_counts_kernel, dim3(wide), dim3(kT), 0, st, t_row_ptr, Cc + 1);
         CN_HIP(hipGetLastError());
+        return CN_OK;
     }
-    { cn_status sc = exclusive_scan(ctx, t_row_ptr, Cc, t_row_ptr, total_dev, st); if (sc != CN_OK) return sc; }
-    if (nnz == 0) return CN_OK;
-    hipLaunchKernelGGL(copy_i32_kernel, dim3(wide), dim3(kT), 0, st, t_row_ptr, scratch, Cc);
+    // as many row blocks as a cursor array of about four million entries allows (a scan of that size is a few
+    // microseconds); one block per row where that fits
+    constexpr int64_t kCursorEntries = (int64_t)4 << 20;
+    int64_t blocks = R;
+    if (blocks * Cc > kCursorEntries) blocks = kCursorEntries / Cc > 1 ? kCursorEntries / Cc : 1;
+    const int64_t rows_per_block = (R + blocks - 1) / blocks;
+    blocks = (R + rows_per_block - 1) / rows_per_block;
+    const int64_t entries = Cc * blocks;
+    if ((size_t)(entries + 1) * sizeof(int32_t) > ctx->workspace_bytes) {
+        set_error("csr_transpose: %lld columns need a cursor array beyond the workspace", (long long)Cc);
+        return CN_ERR_WORKSPACE;
+    }
+    int32_t *cursor = reinterpret_cast<int32_t *>(ctx->workspace);
+    hipLaunchKernelGGL(zero_counts_kernel, dim3(wide), dim3(kT), 0, st, cursor, entries + 1);
     CN_HIP(hipGetLastError());
-    hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)(R < wide ? (R > 0 ? R : 1) : wide)), dim3(kT), 0, st, R, row_ptr,
-                       col_idx, vals, scratch, t_col_idx, t_vals);
+    hipLaunchKernelGGL(transpose_count_kernel, dim3((unsigned)(R < wide ? R : wide)), dim3(kT), 0, st, R, row_ptr, col_idx, blocks,
+                       rows_per_block, cursor);
     CN_HIP(hipGetLastError());
-    hipLaunchKernelGGL(sort_rows_kernel, dim3(wide), dim3(kT), 0, st, Cc, t_row_ptr, t_col_idx, t_vals);
+    { cn_status sc = exclusive_scan(ctx, cursor, entries, cursor, total_dev, st); if (sc != CN_OK) return sc; }
+    hipLaunchKernelGGL(transpose_row_ptr_kernel, dim3(wide), dim3(kT), 0, st, cursor, Cc, blocks, t_row_ptr);
+    CN_HIP(hipGetLastError());
+    hipLaunchKernelGGL(transpose_fill_kernel, dim3((unsigned)(blocks < 65535 * 16 ? blocks : 65535 * 16)), dim3(kT), 0, st, R, row_ptr,
+                       col_idx, vals, blocks, rows_per_block, cursor, t_col_idx, t_vals);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

@@ -260,8 +260,9 @@ cn_status cn_csr_to_dense_f32(int64_t R, int64_t C, const int32_t *row_ptr_devic
                               const float *vals_device, float *out_device, int64_t ldo, void *stream);
 
 /* CSR of S^T from the CSR of the R x C matrix S with nnz nonzeros (t_row_ptr: C + 1 entries, t_col_idx
- * and t_vals: nnz entries, column indices ascending within a row).  `scratch` is C int32 of device
- * memory.  With it Tdot_sparse (the transposed operand of cusparseScsrmm2, source/clusterNet.cpp:304,307)
+ * and t_vals: nnz entries, column indices ascending within a row).  A counting sort over (column, block of rows) in
+ * the library's workspace: the result does not depend on scheduling, and a column of any number of nonzeros costs
+ * what its nonzeros cost.  `scratch` is not used any more and may be NULL.  With it Tdot_sparse (the transposed operand of cusparseScsrmm2, source/clusterNet.cpp:304,307)
  * is cn_csr_gemm_f32 on the transposed arrays. */
 cn_status cn_csr_transpose(int64_t R, int64_t C, int64_t nnz, const int32_t *row_ptr_device,
                            const int32_t *col_idx_device, const float *vals_device, int32_t *t_row_ptr_device,

@@ -260,6 +260,46 @@ def test_csr_transpose_equals_csr_of_the_transpose(dev, shape, density):
     assert np.array_equal(_bits(T.vals.cpu().numpy()), _bits(vals))
 
 
+def test_csr_transpose_with_a_dense_column_and_long_rows(dev):
+    """A column that every one of 60 000 rows uses, beside sparse ones, and a short wide matrix whose transposition
+    has a hundred thousand short rows: the result rows come out in ascending column order whatever their length
+    (a counting sort over blocks of rows; nothing is sorted afterwards), twice in a row with the same bits."""
+    import scipy.sparse as sp
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(90)
+    R, C = 60_000, 300
+    A = (rng.uniform(0, 1, (R, C)) * (rng.uniform(0, 1, (R, C)) < 0.01)).astype(np.float32)
+    A[:, 7] = rng.uniform(0.5, 1, R).astype(np.float32)       # fully dense column -> a result row of 60 000 entries
+    A[::3, 123] = 2.0
+    for M in (A, np.ascontiguousarray(A[:128].T), (rng.uniform(0, 1, (128, 100_000)) * (rng.uniform(0, 1, (128, 100_000)) < 0.02)).astype(np.float32)):
+        S = L.csr_from_dense(_t(M, dev))
+        want = sp.csr_matrix(M.T)
+        want.sort_indices()
+        for _ in range(2):
+            T = L.csr_transpose(S)
+            assert (T.rows, T.cols) == (M.shape[1], M.shape[0])
+            assert np.array_equal(T.row_ptr.cpu().numpy(), want.indptr)
+            assert np.array_equal(T.col_idx.cpu().numpy(), want.indices)
+            assert np.array_equal(_bits(T.vals.cpu().numpy()), _bits(want.data.astype(np.float32)))
+
+
+def test_more_than_2_to_31_nonzeros_are_refused_not_truncated(dev):
+    """8.6 GB of ones: the count of nonzeros passes 2^31 - 1, which the 32-bit row pointers cannot hold.  The
+    prefix sums carry 64 bits, so the count arrives exact and the call answers CN_ERR_SHAPE."""
+    import ctypes
+    import torch
+    import clusternet_amd as cn
+    rows, cols = 65_536, 32_800
+    A = torch.ones((rows, cols), device=dev)
+    row_ptr = torch.empty(rows + 1, dtype=torch.int32, device=dev)
+    nnz = ctypes.c_int64(-1)
+    status = cn.lib().cn_csr_from_dense_f32(A.data_ptr(), rows, cols, cols, 0, row_ptr.data_ptr(), None, None, 0, ctypes.byref(nnz), None)
+    torch.cuda.synchronize()
+    assert nnz.value == rows * cols and status == 2, (status, nnz.value, cn.lib().cn_last_error())
+    del A
+    torch.cuda.empty_cache()
+
+
 def test_batch_products(dev):
     """The two products of the training step on a 2 % dense batch: X W = CSR(X) W and
     X^T E = CSR(X^T) E; against the dense kernels of this library, the fp64 product and the checker."""
