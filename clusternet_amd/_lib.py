@@ -89,6 +89,8 @@ def lib():
     L.cn_host_reduction_fences.restype = None
     L.cn_host_csr_strip_kernel.argtypes = [C.c_int]
     L.cn_host_csr_strip_kernel.restype = None
+    L.cn_host_csr_rows_workgroups_per_cu.argtypes = [C.c_int]
+    L.cn_host_csr_rows_workgroups_per_cu.restype = None
     L.cn_host_csr_lds_rows.argtypes = [C.c_int]
     L.cn_host_csr_lds_rows.restype = None
     _lib = L

@@ -996,6 +996,7 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
 }
 
 static bool g_strip_kernel = true;  // the test hooks below switch these kernels off to compare
+static int g_rows_per_cu = 0;  // tuning hook: workgroups per compute unit of the fused row passes, 0 = their own figure
 static bool g_lds_rows = true;
 
 static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
@@ -1071,6 +1072,7 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
 }
 
 void cn_host_csr_strip_kernel(int enabled) { g_strip_kernel = enabled != 0; }
+void cn_host_csr_rows_workgroups_per_cu(int per_cu) { g_rows_per_cu = per_cu > 0 ? per_cu : 0; }
 void cn_host_csr_lds_rows(int enabled) { g_lds_rows = enabled != 0; }
 
 cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
@@ -1158,7 +1160,7 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
         const int threads = codes_only ? row_threads<2>() : kRowThreads;
         const int64_t per_wg = threads / 64;
         // the encoder table allows three workgroups of 256 threads per compute unit, the registers two of 512
-        int64_t grid = (int64_t)ctx->num_cu * (codes_only ? 2 : 3);
+        int64_t grid = (int64_t)ctx->num_cu * (g_rows_per_cu > 0 ? g_rows_per_cu : (codes_only ? 2 : 3));
         if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
         auto kernel = rms ? csr_rows_kernel<4> : (w ? csr_rows_kernel<3> : csr_rows_kernel<2>);
         hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), lds, st, R, N, row_ptr, col_idx, vals, B, ldb, col_blocks,

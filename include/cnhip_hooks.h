@@ -54,6 +54,8 @@ void cn_host_absmax_compress_spin_limit(int spins);
  * LDS (maximum only); they then run on the general kernels, which the tests compare against. */
 void cn_host_csr_strip_kernel(int enabled);
 void cn_host_csr_lds_rows(int enabled);
+/* Workgroups per compute unit of the passes that turn a sparse product into codes (and updates); 0 = their own. */
+void cn_host_csr_rows_workgroups_per_cu(int per_cu);
 
 /* The encoder's bucket table on the host.  cn_host_xlut_entries: number of 8-byte entries of a table;
  * cn_host_xlut_step_count: number of steps of the code function found at precision 1;
