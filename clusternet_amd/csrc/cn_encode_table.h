@@ -13,8 +13,8 @@ constexpr int kEncodeThreads = 256;  // threads that build the table; a workgrou
 // Every workgroup builds the table of cn_xlut.h for the call's precision in LDS (one thread per step
 // of the code function: ten divisions around the step's estimated position; then every thread a run of
 // LDS stores), then looks every element up: shift, clamp, one 8-byte LDS read, one compare, one byte select.
-// The build is what a call on a small input costs (about 4 us of the 7 us that a call on 4096 elements takes
-// at the clocks such calls run at), so its phases keep their LDS reads independent of one another and the
+// The build is what a call on a small input costs (about 3.6 us of the 7 us that a call on 4096 elements
+// takes), so its phases keep their LDS reads independent of one another and the
 // two sentinel entries, which take full evaluations of the literal procedure, are computed by lanes of
 // wavefronts that locate no step.
 
@@ -35,7 +35,7 @@ static_assert(kXMaxSteps < 255, "a step's number plus one fits a byte");
 // registers before the first barrier; the eight literal evaluations behind the two sentinel entries run one per
 // lane on wavefronts that locate no step; every group of LDS reads is issued as a whole before its first use
 // (unconditional loads, conditions applied to the values), because a conditional read costs a full LDS round
-// trip each.  Measured at the shader clock: about 4 800 cycles, against 11 000 with dependent reads.
+// trip each.  Measured at the shader clock: about 9 000 cycles, against 11 000 with dependent reads.
 __device__ __forceinline__ bool build_table(EncodeShared &sh, const XStep *__restrict__ steps, int count,
                                             float precision, const float *__restrict__ table) {
     const int t = threadIdx.x;
