@@ -137,7 +137,7 @@ def bench_codec(torch, cn, dev):
     res = {}
     gen = torch.Generator(device=dev).manual_seed(99)
     for name, n, iters in (("grad_100000x8192", 100000 * 8192, 20), ("cfg2_128x40000", 128 * 40000, 200),
-                           ("ref_microbench_5120x5120", 5120 * 5120, 100)):
+                           ("ref_microbench_5120x5120", 5120 * 5120, 100), ("layer_784x1024", 784 * 1024, 200)):
         x = torch.empty(n, device=dev).normal_(0.0, 0.02, generator=gen)
         idx = torch.randint(0, n, (n // 100,), device=dev, generator=gen)
         x[idx] = torch.empty(idx.numel(), device=dev).normal_(0.0, 0.5, generator=gen)
@@ -173,6 +173,12 @@ def bench_codec(torch, cn, dev):
             replayed["absmax_compress_single_launch_us"] = time_replayed(
                 torch, lambda: cn.absmax_compression_8bit(x, codes, prec_t), 20, 50)
             cn.lib().cn_host_absmax_compress_single_launch(0)
+            if n <= (3 << 20):
+                # tensors this small are encoded element by element; the per-call table beside it
+                cn.lib().cn_host_codec_literal_upto(0)
+                replayed["compress_with_table_us"] = time_replayed(
+                    torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50)
+                cn.lib().cn_host_codec_literal_upto(2 ** 64 - 1)
             res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
         if n >= 100000 * 8192:
             # movers that are not this library's: the runtime's device-to-device copy (above) and its fill, the latter a

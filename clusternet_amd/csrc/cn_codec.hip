@@ -146,6 +146,69 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
     }
 }
 
+// ---- the literal procedure for small tensors ---------------------------------------------------------------
+// A workgroup's table costs about 9 000 cycles before the first element is encoded; the literal procedure (division
+// and pivot search, encode_exact) costs about 70 instructions per element and needs only the 126-entry codebook.  A
+// tensor of a few hundred thousand elements spread over the whole chip is a handful of elements per lane, which
+// the literal procedure finishes before a table would exist.  Four elements per lane and step, evaluated level by
+// level so that the search's LDS reads overlap; same bits as the table by construction (the table is made of
+// evaluations of this procedure).
+template <bool kVector, bool kUpdate>
+__global__ __launch_bounds__(kThreads) void compress_literal_kernel(
+    const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr, size_t n,
+    uint8_t *__restrict__ codes, const float *__restrict__ table, float alpha, float *__restrict__ y) {
+    __shared__ float slot[128];
+    __shared__ float dlut[kUpdate ? 256 : 1];
+    const int t = threadIdx.x;
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
+    const size_t nvec = kVector ? n / 4 : 0;
+    const size_t v0 = (size_t)blockIdx.x * kThreads + t;
+    f32x4 first{0.f, 0.f, 0.f, 0.f};
+    if (kVector && v0 < nvec) first = reinterpret_cast<const f32x4 *>(x)[v0];  // beside the codebook's latency
+    if (t < 126) {
+        const float c = table[t];
+        slot[t] = c;
+        if (kUpdate) {
+            const float v = c * precision;
+            dlut[t] = alpha * v;
+            dlut[t + 128] = alpha * (-v);
+        }
+    } else if (t == 126) {
+        slot[126] = 1.0f;
+        slot[127] = 0.0f;
+        if (kUpdate) {
+            dlut[126] = alpha * precision;
+            dlut[127] = alpha * precision;
+            dlut[254] = alpha * precision;
+            dlut[255] = alpha * (-precision);
+        }
+    }
+    __syncthreads();
+    if (kVector) {
+        for (size_t v = v0; v < nvec; v += (size_t)gridDim.x * kThreads) {
+            const f32x4 in = (v == v0) ? first : reinterpret_cast<const f32x4 *>(x)[v];
+            const uint32_t bits[4] = {__float_as_uint(in.x), __float_as_uint(in.y), __float_as_uint(in.z), __float_as_uint(in.w)};
+            uint32_t c[4];
+            encode_exact_many<4>(bits, precision, slot, c);
+            reinterpret_cast<uint32_t *>(codes)[v] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+            if (kUpdate) {
+                f32x4 w = reinterpret_cast<f32x4 *>(y)[v];
+                w.x = w.x + dlut[c[0]];
+                w.y = w.y + dlut[c[1]];
+                w.z = w.z + dlut[c[2]];
+                w.w = w.w + dlut[c[3]];
+                reinterpret_cast<f32x4 *>(y)[v] = w;
+            }
+        }
+    }
+    // without vectors: everything; with them: the n % 4 elements behind the last whole vector
+    for (size_t i = nvec * 4 + (size_t)blockIdx.x * kThreads + t; i < n; i += (size_t)gridDim.x * kThreads) {
+        const uint32_t c = encode_exact(x[i], precision, slot);
+        codes[i] = (uint8_t)c;
+        if (kUpdate) y[i] = y[i] + dlut[c];
+    }
+}
+
 // ---- streaming forms for large tensors ---------------------------------------------------------------------
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 constexpr int kAuxNt = 2;            // cache policy bits of the buffer instructions: nt
@@ -606,6 +669,12 @@ constexpr size_t kStreamFrom = (size_t)1 << 24;
 // Tensors of at least this many elements (256 MiB of fp32) do not fit the 256 MB Infinity Cache.
 constexpr size_t kBeyondCacheFrom = (size_t)1 << 26;
 
+// Tensors of at most this many elements are encoded by the literal procedure, without a table.  Measured, replayed
+// from a graph: 2.9 us against 5.7 us up to 2^18 elements, 4.1 against 5.9 at 2^20, 5.6 against 7.3 at 2^21, 10.7
+// against 9.9 at 5.12 M; the two cross near 4 M.  Tuning hook: cn_host_codec_literal_upto.
+constexpr size_t kLiteralUpto = (size_t)3 << 20;
+static size_t g_literal_upto = kLiteralUpto;
+
 static int stream_grid(const Context *ctx, size_t n, int per_cu) {
     size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
     if (g_workgroups_per_cu > 0) per_cu = g_workgroups_per_cu;
@@ -642,6 +711,18 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
                                    hipFuncAttributeMaxDynamicSharedMemorySize, most));
     }
     const bool vec = aligned(x, 16) && aligned(codes, 4) && (!y || aligned(y, 16));
+    if (n <= g_literal_upto && g_workgroups_per_cu == 0) {
+        const size_t items = vec ? (n + 3) / 4 : n;
+        size_t wgs = (items + kThreads - 1) / kThreads;
+        const size_t cap = (size_t)ctx->num_cu * 8;
+        if (wgs > cap) wgs = cap;
+        auto small = y ? (vec ? compress_literal_kernel<true, true> : compress_literal_kernel<false, true>)
+                       : (vec ? compress_literal_kernel<true, false> : compress_literal_kernel<false, false>);
+        hipLaunchKernelGGL(small, dim3((unsigned)wgs), dim3(kThreads), 0, st, x, precision, precision_dev, n, codes,
+                           ctx->table, alpha, y);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
     if (vec && !y && n >= kStreamFrom && g_workgroups_per_cu == 0) {
         static OncePerDevice stream_configured;
         if (stream_configured.first(ctx->device)) {
@@ -694,6 +775,9 @@ static cn_status decompress_impl(const uint8_t *codes, float precision, const fl
 using namespace cn;
 
 extern "C" {
+
+// Tuning hook: largest element count that compression encodes with the literal procedure instead of a table (0 = never, SIZE_MAX = the library's own threshold).
+void cn_host_codec_literal_upto(size_t n) { g_literal_upto = (n == (size_t)-1) ? kLiteralUpto : n; }
 
 // Tuning hook: workgroups per compute unit for the codec and abs-max kernels, 0 = each kernel's own choice.
 void cn_host_codec_workgroups_per_cu(int per_cu) { g_workgroups_per_cu = per_cu > 0 ? per_cu : 0; }

@@ -36,6 +36,10 @@ void cn_host_gemm_epilogue_in_kernel(int enabled);
 
 /* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
 void cn_host_codec_workgroups_per_cu(int per_cu);
+/* Largest element count that compression (all forms) encodes with the literal procedure, element by element,
+ * instead of building the table first; 0 = always the table, SIZE_MAX = the library's own threshold.
+ * Both give the same bits. */
+void cn_host_codec_literal_upto(size_t n);
 
 /* Nonzero: the single-launch reductions (abs-max, max, sum) put a release fence at device scope between a
  * workgroup's partial result and its arrival count, the form the memory model prescribes, instead of ordering the

@@ -28,3 +28,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(params=["literal_for_small_tensors", "table_always"])
+def codec_form(request):
+    """Compression has two encoders that must give the same bits: the literal procedure per element for small
+    tensors and the per-call table.  Tests that use this fixture run once with the library's own choice and once
+    with the table forced for every size, so the small adversarial inputs exercise both."""
+    from clusternet_amd import _lib as L
+    if request.param == "table_always":
+        L.lib().cn_host_codec_literal_upto(0)
+    yield request.param
+    L.lib().cn_host_codec_literal_upto(2 ** 64 - 1)  # back to the library's own threshold

@@ -78,6 +78,7 @@ def test_decode_tables_follow_the_closed_form():
 
 
 @pytest.mark.gpu
+@pytest.mark.usefixtures("codec_form")
 def test_gpu_codes_equal_the_file():
     import torch
     import clusternet_amd as cn

@@ -5,7 +5,7 @@ import pytest
 import oracle
 from util import cfg2_tensor
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("codec_form")]
 
 
 @pytest.fixture(scope="module")

@@ -6,7 +6,7 @@ import pytest
 
 import oracle
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("codec_form")]
 
 
 @pytest.fixture(scope="module")
