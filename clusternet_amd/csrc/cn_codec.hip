@@ -5,17 +5,20 @@
 // Each lane moves 16-byte vectors laid out so that one wavefront instruction touches one
 // contiguous 1 KiB (fp32 side) / 256 B (code side) span.
 //
-// Large tensors take the *_stream_kernel forms.  What a stream that also writes reaches on this part depends
-// sharply on how many bytes a compute unit keeps in flight: about 48 KB of loads (compression) or 64 KB of stores
-// (decompression) per compute unit, one workgroup each, is the optimum; twice that, or as much again left in
-// flight by not waiting for the stores, costs 10 to 15 %.  So these kernels run one workgroup per compute unit,
-// address memory through a buffer descriptor per tile (a uniform base and a 32-bit lane offset; the descriptor's
-// range replaces the bounds test of the last tile), read with the non-temporal hint and write with it too.
+// What a stream that also writes reaches on this part depends sharply on the window of addresses in flight.
+// Decompression (mostly writes) runs a workgroup per 4096-element tile, as many workgroups as tiles, so that the
+// dispatcher keeps the tiles in flight next to one another: 6.9 TB/s, against 6.1 TB/s for the best persistent grid.
+// Compression cannot start a workgroup per tile (its encoder table costs 9 000 cycles to build); large tensors take
+// compress_stream_kernel, one persistent workgroup per compute unit that draws its tiles in order from a counter, which
+// keeps the same narrow window (6.6 TB/s, against 6.4 TB/s on a grid-stride walk), addressed through a buffer
+// descriptor per tile (a uniform base and a 32-bit lane offset; the descriptor's range replaces the bounds test of
+// the last tile), read and written with the non-temporal hint.
 #include <type_traits>
 
 #include "cn_internal.h"
 #include "cn_xlut.h"
 #include "cn_encode_table.h"
+#include "cn_tile_queue.h"
 
 namespace cn {
 
@@ -219,16 +222,19 @@ __device__ __forceinline__ rsrc_t tile_rsrc(const void *base, uint32_t bytes) {
 }
 
 // Compression of whole float4 groups: a tile is T * U float4, all of its loads are issued at once and awaited
-// together, then encoded and stored; the next tile's loads go out right behind the stores.  Two shapes: 256 x 12
-// (48 KiB of input per tile) with one workgroup per compute unit for tensors that stream from HBM, 512 x 10 with two
-// for tensors that the Infinity Cache can hold, where more bytes in flight pay.
+// together, then encoded and stored; the next tile's loads go out right behind the stores.  Two shapes: 1024 x 12
+// (192 KiB of input per tile), one workgroup per compute unit, tiles drawn in order from a counter (`queue`,
+// cn_tile_queue.h) for tensors that stream from HBM; 512 x 10 with two workgroups per compute unit on a grid-stride
+// walk (`queue` NULL) for tensors that the Infinity Cache can hold.
 template <int T, int U>
 __global__ __launch_bounds__(T) void compress_stream_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr, size_t n,
-    uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table,
+    uint32_t *__restrict__ queue) {
     constexpr uint32_t kVecs = T * U;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    __shared__ uint32_t queue_slots[2];
     const float precision = precision_ptr ? *precision_ptr : precision_value;
     const size_t nvec = n / 4;
     const size_t tiles = (nvec + kVecs - 1) / kVecs;
@@ -240,8 +246,17 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
 #pragma unroll
         for (int j = 0; j < U; ++j) v[j] = __builtin_amdgcn_raw_buffer_load_b128(r, (j * T + tid) * 16u, 0, kAuxNt);
     };
+    // tiles are drawn from a counter (cn_tile_queue.h); without one, a grid-stride walk
+    TileQueue q = tile_queue(queue, (uint32_t)tiles, queue_slots);
     size_t tile = blockIdx.x;
-    if (tile < tiles) load(tile);  // on their way while the table is built
+    if (queue) {
+        q.draw_ahead();
+        tile = q.next();
+    }
+    if (tile < tiles) {
+        load(tile);  // on their way while the table is built
+        if (queue) q.draw_ahead();
+    }
     const bool exact_only = !build_table(sh, steps, step_count, precision, table);
     const uint32_t first = xlut_first(precision);
     // `exact` is a type: the table look-up, or (where no table can be trusted) the literal procedure per element
@@ -262,8 +277,11 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
                 packed[j] = encode(v[j].x) | (encode(v[j].y) << 8) | (encode(v[j].z) << 16) | (encode(v[j].w) << 24);
 #pragma unroll
             for (int j = 0; j < U; ++j) __builtin_amdgcn_raw_buffer_store_b32(packed[j], r, (j * T + tid) * 4u, 0, kAuxNt);
-            tile += gridDim.x;
-            if (tile < tiles) load(tile);
+            tile = queue ? (size_t)q.next() : tile + gridDim.x;
+            if (tile < tiles) {
+                load(tile);
+                if (queue) q.draw_ahead();
+            }
         }
         if (blockIdx.x == 0) {  // ragged tail (n % 4 elements)
             const size_t i = nvec * 4 + tid;
@@ -273,17 +291,29 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
     if (exact_only) run(std::true_type{}); else run(std::false_type{});
 }
 
-// Decompression of whole code words: a tile is kT * kU words (64 KiB of output for 512 x 8); the workgroup waits
-// for its stores before it starts the next tile, which holds the bytes in flight at one tile per compute unit.
-constexpr int kStreamDT = 512, kStreamDU = 8;
-__global__ __launch_bounds__(kStreamDT) void decompress_stream_kernel(
+// Decompression with a workgroup per tile and as many workgroups as tiles, placed by the dispatcher as compute
+// units free up: the workgroups in flight at any moment then cover one narrow, advancing window of addresses, which
+// is what this part's memory rewards in a stream that mostly writes (measured on arithmetic-free kernels: 6.6 TB/s
+// for 1 byte read + 4 written this way, 6.2 TB/s for the best persistent grid).  The price is a decode table per
+// 2048 elements: its inputs are requested together with the tile's codes, so it costs a barrier, not a latency.
+template <int T, int U>
+__global__ __launch_bounds__(T) void decompress_tile_kernel(
     const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr, size_t n,
     float *__restrict__ out, const float *__restrict__ table, const float *__restrict__ given_lut) {
-    constexpr int T = kStreamDT, U = kStreamDU;
+    static_assert(T >= 256, "one lane per table entry");
     constexpr uint32_t kVecs = T * U;
     __shared__ float lut[256];
-    const float precision = precision_ptr ? *precision_ptr : precision_value;
     const uint32_t tid = threadIdx.x;
+    const size_t nvec = n / 4;
+    const size_t first = (size_t)blockIdx.x * kVecs;
+    const size_t left = first < nvec ? nvec - first : 0;
+    const uint32_t vecs = (uint32_t)(left < kVecs ? left : kVecs);
+    const rsrc_t rc = tile_rsrc(codes + first * 4, vecs * 4u);
+    const rsrc_t ro = tile_rsrc(out + first * 4, vecs * 16u);
+    uint32_t w[U];
+#pragma unroll
+    for (int j = 0; j < U; ++j) w[j] = __builtin_amdgcn_raw_buffer_load_b32(rc, (j * T + tid) * 4u, 0, 0);
+    const float precision = precision_ptr ? *precision_ptr : precision_value;
     if (given_lut) {  // the caller's own 256-entry table instead of the codec's
         if (tid < 256) lut[tid] = given_lut[tid];
     } else if (tid < 126) {
@@ -297,36 +327,24 @@ __global__ __launch_bounds__(kStreamDT) void decompress_stream_kernel(
         lut[255] = -precision;
     }
     __syncthreads();
-    const size_t nvec = n / 4;
-    const size_t tiles = (nvec + kVecs - 1) / kVecs;
-    for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-        const size_t left = nvec - tile * kVecs;
-        const uint32_t vecs = (uint32_t)(left < kVecs ? left : kVecs);
-        const rsrc_t rc = tile_rsrc(codes + tile * (size_t)kVecs * 4, vecs * 4u);
-        const rsrc_t ro = tile_rsrc(out + tile * (size_t)kVecs * 4, vecs * 16u);
-        uint32_t w[U];
 #pragma unroll
-        for (int j = 0; j < U; ++j) w[j] = __builtin_amdgcn_raw_buffer_load_b32(rc, (j * T + tid) * 4u, 0, 0);
-#pragma unroll
-        for (int j = 0; j < U; ++j) {
-            u32x4 o;
-            o.x = __float_as_uint(lut[w[j] & 0xffu]);
-            o.y = __float_as_uint(lut[(w[j] >> 8) & 0xffu]);
-            o.z = __float_as_uint(lut[(w[j] >> 16) & 0xffu]);
-            o.w = __float_as_uint(lut[w[j] >> 24]);
-            __builtin_amdgcn_raw_buffer_store_b128(o, ro, (j * T + tid) * 16u, 0, kAuxSc0Sc1Nt);
-        }
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this tile's stores have been acknowledged
+    for (int j = 0; j < U; ++j) {
+        u32x4 o;
+        o.x = __float_as_uint(lut[w[j] & 0xffu]);
+        o.y = __float_as_uint(lut[(w[j] >> 8) & 0xffu]);
+        o.z = __float_as_uint(lut[(w[j] >> 16) & 0xffu]);
+        o.w = __float_as_uint(lut[w[j] >> 24]);
+        __builtin_amdgcn_raw_buffer_store_b128(o, ro, (j * T + tid) * 16u, 0, kAuxSc0Sc1Nt);
     }
-    if (blockIdx.x == 0) {
+    if (blockIdx.x == 0) {  // the n % 4 elements behind the last whole word
         const size_t i = nvec * 4 + tid;
         if (i < n) out[i] = lut[codes[i]];
     }
 }
 
 // Follows kDecompression_8bit (source/clusterKernels.cu:1135-1160): a 256-entry table scaled by
-// the precision, rebuilt once per workgroup, then a pure gather.
-template <bool kVector>
+// the precision, rebuilt once per workgroup, then a pure gather.  Element by element, for buffers that are not
+// aligned to whole words; aligned ones take decompress_tile_kernel.
 __global__ __launch_bounds__(kThreads) void decompress_kernel(
     const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr,
     size_t n, float *__restrict__ out, const float *__restrict__ table, const float *__restrict__ given_lut) {
@@ -345,39 +363,8 @@ __global__ __launch_bounds__(kThreads) void decompress_kernel(
         lut[255] = -precision;
     }
     __syncthreads();
-
-    if (kVector) {
-        const size_t nvec = n / 4;
-        const uint32_t *c4 = reinterpret_cast<const uint32_t *>(codes);
-        f32x4 *o4 = reinterpret_cast<f32x4 *>(out);
-        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
-        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-            const size_t base = tile * kTileVec + threadIdx.x;
-            uint32_t w[kVecPerThread];
-#pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
-                size_t i = base + (size_t)j * kThreads;
-                w[j] = (i < nvec) ? __builtin_nontemporal_load(&c4[i]) : 0u;
-            }
-#pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
-                size_t i = base + (size_t)j * kThreads;
-                f32x4 o;
-                o.x = lut[w[j] & 0xffu];
-                o.y = lut[(w[j] >> 8) & 0xffu];
-                o.z = lut[(w[j] >> 16) & 0xffu];
-                o.w = lut[w[j] >> 24];
-                if (i < nvec) __builtin_nontemporal_store(o, &o4[i]);
-            }
-        }
-        if (blockIdx.x == 0) {
-            size_t i = nvec * 4 + threadIdx.x;
-            if (i < n) out[i] = lut[codes[i]];
-        }
-    } else {
-        for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
-            out[i] = lut[codes[i]];
-    }
+    for (size_t i = (size_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (size_t)gridDim.x * kThreads)
+        out[i] = lut[codes[i]];
 }
 
 // ---- abs-max ------------------------------------------------------------------------------------
@@ -726,17 +713,22 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
     if (vec && !y && n >= kStreamFrom && g_workgroups_per_cu == 0) {
         static OncePerDevice stream_configured;
         if (stream_configured.first(ctx->device)) {
-            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<256, 12>),
+            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<1024, 12>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
             CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<512, 10>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
         }
-        if (n >= kBeyondCacheFrom)
-            hipLaunchKernelGGL((compress_stream_kernel<256, 12>), dim3(ctx->num_cu), dim3(256), sizeof(EncodeShared), st, x,
-                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
+        // Beyond the cache: one workgroup of 1024 lanes per compute unit, tiles of 192 KiB drawn from the counter
+        // (measured on 819.2 M elements: 620 us; 1024 x 8: 626 us, 1024 x 16: 640 us, 512 x 16: 686 us, and 639 us
+        // for 256 x 12 on a grid-stride walk; tiles of 48 KiB would draw tickets faster than one counter hands them out).
+        // Tensors the cache can hold: two workgroups of 512 x 10 per compute unit on a grid-stride walk (26 M elements:
+        // 24.5 us against 32 to 34 us for the drawn forms).
+        if (n >= kBeyondCacheFrom && n < ((size_t)1 << 40))
+            hipLaunchKernelGGL((compress_stream_kernel<1024, 12>), dim3(ctx->num_cu), dim3(1024), sizeof(EncodeShared), st, x,
+                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->tile_queue);
         else
             hipLaunchKernelGGL((compress_stream_kernel<512, 10>), dim3(ctx->num_cu * 2), dim3(512), sizeof(EncodeShared), st, x,
-                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table);
+                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, (uint32_t *)nullptr);
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
@@ -756,15 +748,17 @@ static cn_status decompress_impl(const uint8_t *codes, float precision, const fl
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
-    int grid = stream_grid(ctx, n, 8);
-    if (aligned(codes, 4) && aligned(out, 16) && n >= kStreamFrom && g_workgroups_per_cu == 0)
-        hipLaunchKernelGGL(decompress_stream_kernel, dim3(ctx->num_cu), dim3(kStreamDT), 0, st, codes, precision,
-                           precision_dev, n, out, ctx->table, given_lut);
-    else if (aligned(codes, 4) && aligned(out, 16))
-        hipLaunchKernelGGL(decompress_kernel<true>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
-                           precision_dev, n, out, ctx->table, given_lut);
+    // Tile shape measured on 819.2 M elements (a workgroup per tile each): 512 lanes x 2 words 590 us, 256 x 2 620 us,
+    // 256 x 4 700 us, 512 x 4 760 us, 768 x 2 706 us, 1024 x 2 700 us, one word per lane 830 to 900 us; the
+    // persistent one-workgroup-per-compute-unit form it replaces 672 us.  512 x 2 is also the fastest at 5.12 M
+    // (4.5 us against 5.1 us) and at 26 M elements (16.5 us against 18.5 us).
+    constexpr int kT = 512, kU = 2;
+    const size_t wgs = (n / 4 + (size_t)kT * kU - 1) / ((size_t)kT * kU);
+    if (aligned(codes, 4) && aligned(out, 16) && wgs <= 0x7fffffffu)
+        hipLaunchKernelGGL((decompress_tile_kernel<kT, kU>), dim3((unsigned)(wgs < 1 ? 1 : wgs)), dim3(kT), 0, st, codes,
+                           precision, precision_dev, n, out, ctx->table, given_lut);
     else
-        hipLaunchKernelGGL(decompress_kernel<false>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
+        hipLaunchKernelGGL(decompress_kernel, dim3(stream_grid(ctx, n, 8)), dim3(kThreads), 0, st, codes, precision,
                            precision_dev, n, out, ctx->table, given_lut);
     CN_HIP(hipGetLastError());
     return CN_OK;

@@ -36,8 +36,10 @@ struct Context {
     uint32_t *reduce_scratch = nullptr;  // per-workgroup partial results + ticket counters
     uint32_t *tickets = nullptr;         // running maximum and arrival count of the max reductions (kTicketWords words)
     double *sum_scratch = nullptr;       // per-workgroup partial sums (1024 doubles)
+    uint32_t *tile_queue = nullptr;      // ticket counters of the streaming kernels (kTileQueueWords words, left at 0)
 };
 constexpr int kMaxDevices = 16;
+constexpr int kTileQueueWords = 32;  // one 128-byte line; word 0 is the counter
 constexpr int kReduceSlots = 4096;
 // Max reductions: a running maximum and an arrival count per group of kTicketGroup workgroups and one pair for
 // the groups, every pair on a 128-byte line of its own, all left at 0.

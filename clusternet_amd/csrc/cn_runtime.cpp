@@ -78,6 +78,7 @@ static cn_status init_device(int device) {
             (void)hipFree(c.reduce_scratch);
             (void)hipFree(c.tickets);
             (void)hipFree(c.sum_scratch);
+            (void)hipFree(c.tile_queue);
             c = Context();
             (void)hipSetDevice(previous);
         }
@@ -113,6 +114,8 @@ static cn_status init_device(int device) {
     CN_HIP(hipMalloc((void **)&c.tickets, kTicketWords * sizeof(uint32_t)));
     CN_HIP(hipMemset(c.tickets, 0, kTicketWords * sizeof(uint32_t)));
     CN_HIP(hipMalloc((void **)&c.sum_scratch, 1024 * sizeof(double)));
+    CN_HIP(hipMalloc((void **)&c.tile_queue, kTileQueueWords * sizeof(uint32_t)));
+    CN_HIP(hipMemset(c.tile_queue, 0, kTileQueueWords * sizeof(uint32_t)));
     {
         const cn_status located = gemm_static_setup(device);
         if (located != CN_OK) return located;
@@ -187,6 +190,7 @@ cn_status cn_shutdown(void) {
         CN_HIP(hipFree(c.reduce_scratch));
         CN_HIP(hipFree(c.tickets));
         CN_HIP(hipFree(c.sum_scratch));
+        CN_HIP(hipFree(c.tile_queue));
         c = Context();
     }
     if (have_prev) CN_HIP(hipSetDevice(previous));

@@ -16,6 +16,7 @@ static void add_threads(std::vector<Variant> &v) {
 }
 template <int LAUX, int SAUX>
 static void add_tiles(std::vector<Variant> &v) {
+    if (SWEEP_KIND != R4W1W && SWEEP_KIND != R1W4W) add_threads<LAUX, SAUX, 2>(v);  // the wide byte side needs four vectors
     add_threads<LAUX, SAUX, 4>(v);
     add_threads<LAUX, SAUX, 8>(v);
     add_threads<LAUX, SAUX, 12>(v);

@@ -88,13 +88,21 @@ int main(int argc, char **argv) {
         void *out = to_bytes ? bytes : f32b;
         const uint32_t ib = from_bytes ? (uint32_t)n : (uint32_t)(n * 4), ob = to_bytes ? (uint32_t)n : (uint32_t)(n * 4);
         const double moved = (double)tiles * tile_floats * ((k.kind == R4 || k.kind == W4) ? 4.0 : (k.kind == R4W4 ? 8.0 : 5.0));
+        // One tile per workgroup, as many workgroups as tiles, placed by the dispatcher as compute units free up
+        // (waves_per_cu 0 in the file): the shape of an ordinary element-wise launch.
+        for (int wait = 0; wait < (k.kind == R4 ? 1 : 2); ++wait) {
+            auto t = time_it([&] { k.go(tiles, st, in, out, ib, ob, tiles, 1, 0, wait, sink); });
+            fprintf(f, "%d,%d,%d,%d,%d,%u,%d,%d,%d,%u,%.4f,%.4f,%.1f,%.1f\n", k.kind, k.load_policy, k.store_policy, k.U, k.T, 1u, 0,
+                    wait, 0, tiles, t.first, t.second, moved / t.first / 1e6, moved / t.second / 1e6);
+        }
+        if (k.U < 4) continue;  // the short tiles are there for the launch above only
         for (int waves : {4, 8, 16, 32, 64}) {
             const int per_cu = waves / (k.T / 64);
             if (per_cu < 1) continue;
             const unsigned grid = (unsigned)(cus * per_cu);
             const uint32_t two_mib = std::max(1u, (2u << 20) / (tile_floats * 4));
             const uint32_t full = (tiles + grid - 1) / grid;
-            struct Map { uint32_t chunk; int remap; } maps[] = {{1, 0}, {two_mib, 0}, {two_mib, 1}, {full, 0}, {full, 1}};
+            struct Map { uint32_t chunk; int remap; } maps[] = {{1, 0}, {two_mib, 0}, {two_mib, 1}, {full, 0}, {full, 1}, {1, 2}};
             for (const Map &m : maps)
                 for (int wait = 0; wait < (k.kind == R4 ? 1 : 2); ++wait) {
                     auto t = time_it([&] { k.go(grid, st, in, out, ib, ob, tiles, m.chunk, m.remap, wait, sink); });

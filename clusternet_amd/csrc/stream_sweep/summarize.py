@@ -13,6 +13,10 @@ PEAK = 8000.0
 
 
 def mapping(r):
+    if r["waves_per_cu"] == 0:
+        return "a workgroup per tile"
+    if r["xcd_remap"] == 2:
+        return "tiles drawn from a counter"
     if r["chunk_tiles"] == 1:
         return "grid-stride"
     tiles = N // (r["T"] * r["U"] * 4)

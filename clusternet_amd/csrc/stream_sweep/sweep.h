@@ -31,13 +31,14 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 
 // Workgroup b owns the chunks b, b + G, b + 2G, ... of chunk_tiles consecutive tiles each: chunk_tiles 1 is a
 // grid-stride walk, chunk_tiles = tiles / G one contiguous range per workgroup.  With xcd_remap the workgroups that
-// one XCD receives (block ids congruent mod 8) own neighbouring chunks.
+// one XCD receives (block ids congruent mod 8) own neighbouring chunks; xcd_remap 2 hands the chunks out through a
+// ticket counter (sink[0]) instead, to whichever workgroup is free.
 template <int KIND, int LAUX, int SAUX, int U, int T>
 __global__ __launch_bounds__(T) void stream_kernel(const void *in, void *out, uint32_t in_bytes, uint32_t out_bytes, uint32_t tiles,
                                                    uint32_t chunk_tiles, int xcd_remap, int wait_for_stores, uint32_t *sink) {
     const uint32_t G = gridDim.x;
     uint32_t b = blockIdx.x;
-    if (xcd_remap) {
+    if (xcd_remap == 1) {
         const uint32_t xcd = b & 7u, idx = b >> 3, per = G >> 3, rem = G & 7u;
         b = xcd * per + (xcd < rem ? xcd : rem) + idx;
     }
@@ -46,11 +47,25 @@ __global__ __launch_bounds__(T) void stream_kernel(const void *in, void *out, ui
     uint32_t running = 0;
     constexpr uint32_t kF = (uint32_t)T * U * 16u;  // bytes of a tile on the fp32 side
     constexpr uint32_t kC = (uint32_t)T * U * 4u;   // on the byte side
-    for (uint32_t chunk = b;; chunk += G) {
+    // xcd_remap 2: the persistent workgroups take their tiles from a counter in memory, in the order in which they
+    // become free (the next ticket is drawn before the current tile is processed, so its latency is hidden)
+    __shared__ uint32_t ticket[2];
+    const bool queue = xcd_remap == 2;
+    uint32_t drawn = 0, turn = 0;
+    if (queue) {
+        if (tid == 0) ticket[0] = atomicAdd(sink, 1u);
+        __syncthreads();
+        drawn = ticket[0];
+    }
+    for (uint32_t chunk = queue ? drawn : b;; chunk = queue ? drawn : chunk + G) {
         const uint64_t first = (uint64_t)chunk * chunk_tiles;
         if (first >= tiles) break;
         uint32_t last = (uint32_t)first + chunk_tiles;
         if (last > tiles || last < (uint32_t)first) last = tiles;
+        if (queue) {
+            turn ^= 1u;
+            if (tid == 0) ticket[turn] = atomicAdd(sink, 1u);
+        }
         for (uint32_t t = (uint32_t)first; t < last; ++t) {
             const uint32_t tf = __builtin_amdgcn_readfirstlane(t * kF), tc = __builtin_amdgcn_readfirstlane(t * kC);
             if (KIND == R4 || KIND == R4W1 || KIND == R4W4 || KIND == R4W1W) {
@@ -94,7 +109,7 @@ __global__ __launch_bounds__(T) void stream_kernel(const void *in, void *out, ui
                     __builtin_amdgcn_raw_buffer_store_b128(o, rout, (j * T + tid) * 16u, tf, SAUX);
                 }
             } else if (KIND == R1W4W) {
-                u32x4 w[U / 4];
+                u32x4 w[U >= 4 ? U / 4 : 1];
 #pragma unroll
                 for (int q = 0; q < U / 4; ++q) w[q] = __builtin_amdgcn_raw_buffer_load_b128(rin, (q * T + tid) * 16u, tc, LAUX);
 #pragma unroll
@@ -113,13 +128,19 @@ __global__ __launch_bounds__(T) void stream_kernel(const void *in, void *out, ui
             // closed loop: nothing of the next tile is requested before this tile's stores have been acknowledged
             if (KIND != R4 && wait_for_stores) __builtin_amdgcn_s_waitcnt(0x0f70);
         }
+        if (queue) {
+            __syncthreads();
+            drawn = ticket[turn];
+        }
     }
-    if (KIND == R4) sink[(size_t)blockIdx.x * T + tid] = running;
+    // the maximum must be wanted by something; no input holds this pattern, so nothing is ever stored
+    if (KIND == R4 && running == 0xffffffffu) sink[tid] = running;
 }
 
 template <int KIND, int LAUX, int SAUX, int U, int T>
 static void go(unsigned grid, hipStream_t st, const void *in, void *out, uint32_t ib, uint32_t ob, uint32_t tiles, uint32_t chunk,
                int remap, int wait, uint32_t *sink) {
+    if (remap == 2) (void)hipMemsetAsync(sink, 0, 4, st);  // the ticket counter
     hipLaunchKernelGGL((stream_kernel<KIND, LAUX, SAUX, U, T>), dim3(grid), dim3(T), 0, st, in, out, ib, ob, tiles, chunk, remap,
                        wait, sink);
 }
