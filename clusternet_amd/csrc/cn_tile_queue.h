@@ -45,4 +45,31 @@ __device__ __forceinline__ TileQueue tile_queue(uint32_t *counter, uint32_t tile
     return TileQueue{counter, tiles, two_lds_words, 0};
 }
 
+// Calls tile_body(index of the tile's first 16-byte vector) for every tile of kTileVecs vectors.  kDrawn: a persistent
+// grid draws the tiles from `counter` and waits for a tile's loads and stores before it takes the next (`slots`: two
+// words of LDS); otherwise a grid-stride walk, which with as many workgroups as tiles is a workgroup per tile.
+template <int kTileVecs, bool kDrawn, class F>
+__device__ __forceinline__ void walk_tiles(size_t nvec, uint32_t *counter, uint32_t *slots, F &&tile_body) {
+    const size_t tiles = (nvec + kTileVecs - 1) / kTileVecs;
+    if (kDrawn) {
+        TileQueue q = tile_queue(counter, (uint32_t)tiles, slots);
+        q.draw_ahead();
+        uint32_t tile = q.next();
+        while (tile < tiles) {
+            q.draw_ahead();
+            tile_body((size_t)tile * kTileVecs);
+            __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the tile's stores have been acknowledged
+            tile = q.next();
+        }
+    } else {
+        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) tile_body(tile * kTileVecs);
+    }
+}
+
+// Element counts from which the streaming passes run as a persistent grid that draws its tiles (tensors beyond the
+// 256 MB Infinity Cache); below it a workgroup per tile is faster (33.6 M elements: 64 us against 70 us).
+constexpr size_t kDrawnFrom = (size_t)1 << 26;
+// A drawn tile counts its tiles in 32 bits.
+constexpr size_t kDrawnBelow = (size_t)1 << 40;
+
 }  // namespace cn

@@ -8,18 +8,19 @@
 // Every arithmetic step is a separate fp32 operation in the order the unfused kernels use, so the
 // results equal theirs bit for bit.
 #include "cn_internal.h"
+#include "cn_tile_queue.h"
 
 namespace cn {
 
 namespace {
 
-// A workgroup per tile and as many workgroups as tiles, for arrays of whole 16-byte vectors: the dispatcher then keeps
-// the tiles in flight next to one another in memory, which a stream that also writes needs on this part (the weight
-// update on 819.2 M elements: 1.62 ms this way, 1.79 ms on a persistent grid-stride grid; of the tile shapes 512 lanes
-// x 2 vectors is the fastest, 256 x 4: 1.67 ms, 512 x 4: 1.74 ms, 1024 x 2: 1.75 ms).
+// Arrays of whole 16-byte vectors are walked tile by tile with the tiles handed out in order (cn_tile_queue.h), which a
+// stream that also writes needs on this part: a workgroup per tile of 512 lanes x 2 vectors and as many workgroups as
+// tiles, or, beyond the cache, one persistent workgroup per compute unit that draws tiles of 512 x kDrawnVecs vectors
+// from a counter and waits for a tile's stores before it takes the next.  The weight update on 819.2 M elements: 1.46 ms drawn, 1.62 ms with a workgroup per tile, 1.79 ms
+// on a persistent grid-stride grid.
 constexpr int kThreads = 512;
-constexpr int kVecPerThread = 2;
-constexpr int kTileVec = kThreads * kVecPerThread;  // 16-byte vectors per workgroup tile
+constexpr int kTileVecsSmall = 2;
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -41,29 +42,29 @@ __device__ __forceinline__ void build_lut(float *lut, const float *table, float 
 }
 
 // y[i] = y[i] + alpha * decode(codes[i])
-template <bool kVector>
+template <bool kVector, int kVecs, bool kDrawn>
 __global__ __launch_bounds__(kThreads) void decompress_axpy_kernel(
     const uint8_t *__restrict__ codes, float precision_value, const float *__restrict__ precision_ptr,
-    float alpha, size_t n, float *__restrict__ y, const float *__restrict__ table) {
+    float alpha, size_t n, float *__restrict__ y, const float *__restrict__ table, uint32_t *queue) {
     __shared__ float lut[256];
+    __shared__ uint32_t slots[2];
     build_lut(lut, table, precision_ptr ? *precision_ptr : precision_value, alpha);
     if (kVector) {
         const size_t nvec = n / 4;
         const uint32_t *c4 = reinterpret_cast<const uint32_t *>(codes);
         f32x4 *y4 = reinterpret_cast<f32x4 *>(y);
-        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
-        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-            const size_t base = tile * kTileVec + threadIdx.x;
-            uint32_t w[kVecPerThread];
-            f32x4 v[kVecPerThread];
+        walk_tiles<kThreads * kVecs, kDrawn>(nvec, queue, slots, [&](size_t first) {
+            const size_t base = first + threadIdx.x;
+            uint32_t w[kVecs];
+            f32x4 v[kVecs];
 #pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
+            for (int j = 0; j < kVecs; ++j) {
                 const size_t i = base + (size_t)j * kThreads;
                 w[j] = (i < nvec) ? __builtin_nontemporal_load(&c4[i]) : 0u;
                 v[j] = (i < nvec) ? __builtin_nontemporal_load(&y4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
+            for (int j = 0; j < kVecs; ++j) {
                 const size_t i = base + (size_t)j * kThreads;
                 f32x4 o;
                 o.x = v[j].x + lut[w[j] & 0xffu];
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(kThreads) void decompress_axpy_kernel(
                 o.w = v[j].w + lut[w[j] >> 24];
                 if (i < nvec) __builtin_nontemporal_store(o, &y4[i]);
             }
-        }
+        });
         if (blockIdx.x == 0) {
             const size_t i = nvec * 4 + threadIdx.x;
             if (i < n) y[i] = y[i] + lut[codes[i]];
@@ -92,12 +93,13 @@ __device__ __forceinline__ void rmsprop_one(float g, float &rms, float &w, float
     w = w - step;
 }
 
-template <bool kCoded, bool kVector>
+template <bool kCoded, bool kVector, int kVecs, bool kDrawn>
 __global__ __launch_bounds__(kThreads) void rmsprop_update_kernel(
     float *__restrict__ rms, const float *__restrict__ grad, const uint8_t *__restrict__ codes,
     float precision_value, const float *__restrict__ precision_ptr, float *__restrict__ w, float mult,
-    float rate, size_t n, const float *__restrict__ table) {
+    float rate, size_t n, const float *__restrict__ table, uint32_t *queue) {
     __shared__ float lut[256];
+    __shared__ uint32_t slots[2];
     if (kCoded) build_lut(lut, table, precision_ptr ? *precision_ptr : precision_value, 1.0f);
     const float one_minus = 1.0f - mult;
     if (kVector) {
@@ -106,27 +108,24 @@ __global__ __launch_bounds__(kThreads) void rmsprop_update_kernel(
         const f32x4 *g4 = reinterpret_cast<const f32x4 *>(grad);
         f32x4 *r4 = reinterpret_cast<f32x4 *>(rms);
         f32x4 *w4 = reinterpret_cast<f32x4 *>(w);
-        const size_t tiles = (nvec + kTileVec - 1) / kTileVec;
-        for (size_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-            const size_t base = tile * kTileVec + threadIdx.x;
+        walk_tiles<kThreads * kVecs, kDrawn>(nvec, queue, slots, [&](size_t first) {
+            const size_t base = first + threadIdx.x;
             // all loads of the tile first
-            f32x4 g[kVecPerThread], r[kVecPerThread], ww[kVecPerThread];
+            f32x4 g[kVecs], r[kVecs], ww[kVecs];
+            uint32_t c[kVecs];
 #pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
+            for (int j = 0; j < kVecs; ++j) {
                 const size_t i = base + (size_t)j * kThreads;
                 const bool in = i < nvec;
-                if (kCoded) {
-                    const uint32_t c = in ? __builtin_nontemporal_load(&c4[i]) : 0u;
-                    g[j] = f32x4{lut[c & 0xffu], lut[(c >> 8) & 0xffu], lut[(c >> 16) & 0xffu], lut[c >> 24]};
-                } else {
-                    g[j] = in ? __builtin_nontemporal_load(&g4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
-                }
+                if (kCoded) c[j] = in ? __builtin_nontemporal_load(&c4[i]) : 0u;
+                else g[j] = in ? __builtin_nontemporal_load(&g4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
                 r[j] = in ? __builtin_nontemporal_load(&r4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
                 ww[j] = in ? __builtin_nontemporal_load(&w4[i]) : f32x4{0.f, 0.f, 0.f, 0.f};
             }
 #pragma unroll
-            for (int j = 0; j < kVecPerThread; ++j) {
+            for (int j = 0; j < kVecs; ++j) {
                 const size_t i = base + (size_t)j * kThreads;
+                if (kCoded) g[j] = f32x4{lut[c[j] & 0xffu], lut[(c[j] >> 8) & 0xffu], lut[(c[j] >> 16) & 0xffu], lut[c[j] >> 24]};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float re = r[j][e], we = ww[j][e];
@@ -139,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void rmsprop_update_kernel(
                     __builtin_nontemporal_store(ww[j], &w4[i]);
                 }
             }
-        }
+        });
         if (blockIdx.x == 0) {
             const size_t i = nvec * 4 + threadIdx.x;
             if (i < n) rmsprop_one(kCoded ? lut[codes[i]] : grad[i], rms[i], w[i], mult, one_minus, rate);
@@ -154,11 +153,17 @@ inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_
 
 // Vector form: a workgroup per tile.  Element-by-element form (unaligned arrays): a grid-stride loop on a resident grid.
 int grid_of(const Context *ctx, size_t n, bool vec) {
-    const size_t tiles = vec ? (n / 4 + kTileVec - 1) / kTileVec : (n + kThreads - 1) / kThreads;
+    const size_t per = (size_t)kThreads * kTileVecsSmall;
+    const size_t tiles = vec ? (n / 4 + per - 1) / per : (n + kThreads - 1) / kThreads;
     const size_t cap = vec ? (size_t)0x7fffffffu : (size_t)ctx->num_cu * 4;
     const size_t g = tiles < cap ? tiles : cap;
     return (int)(g < 1 ? 1 : g);
 }
+
+// Vectors per lane of a drawn tile.  Measured on 819.2 M elements, a workgroup per tile / drawn x 4 / drawn x 8:
+// decode+add 1.15 / 1.31 / 1.11 ms, RMSprop 2.82 / 2.58 / 2.61 ms, RMSprop on codes 2.35 / 2.39 / 2.31 ms (tiles of
+// 512 x 4 vectors draw tickets about as fast as one counter hands them out).
+constexpr int kDrawnVecs = 8;
 
 cn_status axpy_impl(const uint8_t *codes, float precision, const float *precision_dev, float alpha, size_t n,
                     float *y, void *stream) {
@@ -170,12 +175,16 @@ cn_status axpy_impl(const uint8_t *codes, float precision, const float *precisio
     hipStream_t st = (hipStream_t)stream;
     const bool vec = aligned(codes, 4) && aligned(y, 16);
     const int grid = grid_of(ctx, n, vec);
-    if (vec)
-        hipLaunchKernelGGL(decompress_axpy_kernel<true>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
-                           precision_dev, alpha, n, y, ctx->table);
+    uint32_t *const none = nullptr;
+    if (vec && n >= kDrawnFrom && n < kDrawnBelow)
+        hipLaunchKernelGGL((decompress_axpy_kernel<true, kDrawnVecs, true>), dim3(ctx->num_cu), dim3(kThreads), 0, st, codes,
+                           precision, precision_dev, alpha, n, y, ctx->table, ctx->tile_queue);
+    else if (vec)
+        hipLaunchKernelGGL((decompress_axpy_kernel<true, kTileVecsSmall, false>), dim3(grid), dim3(kThreads), 0, st, codes,
+                           precision, precision_dev, alpha, n, y, ctx->table, none);
     else
-        hipLaunchKernelGGL(decompress_axpy_kernel<false>, dim3(grid), dim3(kThreads), 0, st, codes, precision,
-                           precision_dev, alpha, n, y, ctx->table);
+        hipLaunchKernelGGL((decompress_axpy_kernel<false, 1, false>), dim3(grid), dim3(kThreads), 0, st, codes, precision,
+                           precision_dev, alpha, n, y, ctx->table, none);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -189,17 +198,21 @@ cn_status rmsprop_impl(float *rms, const float *grad, const uint8_t *codes, floa
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
     const bool vec = aligned(rms, 16) && aligned(w, 16) && (codes ? aligned(codes, 4) : aligned(grad, 16));
-    const int grid = grid_of(ctx, n, vec);
+    const bool drawn = vec && n >= kDrawnFrom && n < kDrawnBelow;
+    const int grid = drawn ? ctx->num_cu : grid_of(ctx, n, vec);
+    uint32_t *const queue = drawn ? ctx->tile_queue : nullptr;
+    auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, st, rms, grad, codes, precision, precision_dev, w, mult, rate, n,
+                           ctx->table, queue);
+    };
     if (codes) {
-        if (vec) hipLaunchKernelGGL((rmsprop_update_kernel<true, true>), dim3(grid), dim3(kThreads), 0, st, rms, grad, codes,
-                                    precision, precision_dev, w, mult, rate, n, ctx->table);
-        else     hipLaunchKernelGGL((rmsprop_update_kernel<true, false>), dim3(grid), dim3(kThreads), 0, st, rms, grad, codes,
-                                    precision, precision_dev, w, mult, rate, n, ctx->table);
+        if (drawn) go(rmsprop_update_kernel<true, true, kDrawnVecs, true>);
+        else if (vec) go(rmsprop_update_kernel<true, true, kTileVecsSmall, false>);
+        else go(rmsprop_update_kernel<true, false, 1, false>);
     } else {
-        if (vec) hipLaunchKernelGGL((rmsprop_update_kernel<false, true>), dim3(grid), dim3(kThreads), 0, st, rms, grad, codes,
-                                    precision, precision_dev, w, mult, rate, n, ctx->table);
-        else     hipLaunchKernelGGL((rmsprop_update_kernel<false, false>), dim3(grid), dim3(kThreads), 0, st, rms, grad, codes,
-                                    precision, precision_dev, w, mult, rate, n, ctx->table);
+        if (drawn) go(rmsprop_update_kernel<false, true, kDrawnVecs, true>);
+        else if (vec) go(rmsprop_update_kernel<false, true, kTileVecsSmall, false>);
+        else go(rmsprop_update_kernel<false, false, 1, false>);
     }
     CN_HIP(hipGetLastError());
     return CN_OK;

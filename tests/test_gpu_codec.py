@@ -331,3 +331,30 @@ def test_absmax_and_compression_in_one_call(dev):
     finally:
         L.lib().cn_host_absmax_compress_spin_limit(-1)
         L.lib().cn_host_absmax_compress_single_launch(0)
+
+
+def test_compression_beyond_the_cache_draws_its_tiles(dev, codec_form):
+    """From 2^26 elements on compression runs one workgroup per compute unit that draws 49152-element tiles from a
+    counter: sizes round a tile boundary, n % 4 tails and a start that is 16 bytes in, against the CPU checker, each
+    size twice in a row (the second call finds the counter as the first one left it)."""
+    if codec_form != "literal_for_small_tensors":
+        pytest.skip("the table is used at this size either way")
+    import torch
+    import clusternet_amd as cn
+    rng = np.random.default_rng(77)
+    tile = 1024 * 12 * 4
+    base_n = (1 << 26) + 2 * tile + 16
+    mag = np.exp(rng.uniform(np.log(1e-7), np.log(1.3), base_n)).astype(np.float32)
+    base = (mag * rng.choice(np.array([-1.0, 1.0], np.float32), base_n)).astype(np.float32)
+    want_all = oracle.port_compress(base, 0.77)
+    bt, ct = _t(base, dev), _t(want_all, dev)
+    for n in (1 << 26, (1 << 26) + 1, (1 << 26) + 3, (1 << 26) + tile - 4, (1 << 26) + tile, (1 << 26) + 2 * tile + 7):
+        for off in (0, 4):
+            for _ in range(2):
+                canary = torch.full((n + 64,), 0xAB, dtype=torch.uint8, device=dev)
+                cn.compression_8bit(bt[off:off + n], 0.77, out=canary[32:32 + n])
+                assert torch.equal(canary[32:32 + n], ct[off:off + n]), (n, off)
+                assert int(canary[:32].min()) == 0xAB and int(canary[32 + n:].min()) == 0xAB
+    # a smaller tensor in between takes the other kernels and must not be disturbed by the counter
+    got = cn.compression_8bit(bt[:1 << 20], 0.77)
+    assert torch.equal(got, ct[:1 << 20])

@@ -157,3 +157,52 @@ def test_null_and_size_errors(dev):
     assert L.cn_decompress_8bit_axpy(None, 1.0, 1.0, 4, None, None) == 1
     assert L.cn_rmsprop_update_f32(None, None, None, 0.9, 0.1, 4, None) == 1
     assert L.cn_decompress_8bit_axpy(None, 1.0, 1.0, 0, None, None) == 0
+
+
+def test_tensors_beyond_the_cache_take_drawn_tiles_and_give_the_same_bits(dev, codec_form):
+    """From 2^26 elements on the update passes run as a persistent grid that draws its tiles from a counter.  Each is
+    held to the same call made on pieces below that size (the workgroup-per-tile form, which the tests above hold to
+    the CPU checker), on a size that ends in a partial tile and an n % 4 tail, twice in a row: the second call
+    finds the counter as the first one left it."""
+    if codec_form != "literal_for_small_tensors":
+        pytest.skip("no compression in this test; one run is enough")
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(5)
+    n = (1 << 26) + 3 * 4096 + 7
+    cut = (1 << 25) + 4 * 1000  # pieces: 16-byte aligned starts, both below 2^26
+    g = torch.randn(n, device=dev, generator=gen) * 0.02
+    w0 = torch.randn(n, device=dev, generator=gen)
+    r0 = torch.rand(n, device=dev, generator=gen)
+    codes = torch.randint(0, 256, (n,), dtype=torch.uint8, device=dev, generator=gen)
+
+    def pieces(fn, *arrays):
+        for lo, hi in ((0, cut), (cut, n)):
+            fn(*[a[lo:hi] for a in arrays])
+
+    def same(a, b):
+        return torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+    for _ in range(2):
+        # flat passes
+        w, ref = w0.clone(), w0.clone()
+        L.sgd_update(w, g, 0.0125)
+        pieces(lambda a, b: L.sgd_update(a, b, 0.0125), ref, g)
+        assert same(w, ref)
+        assert same(w, w0 - 0.0125 * g)
+        out, ref = torch.empty_like(g), torch.empty_like(g)
+        L.sub(w0, g, out)
+        assert same(out, w0 - g)
+        # decode + add
+        w, ref = w0.clone(), w0.clone()
+        cn.decompression_8bit_axpy(codes, 0.37, -0.5, w)
+        pieces(lambda c, y: cn.decompression_8bit_axpy(c, 0.37, -0.5, y), codes, ref)
+        assert same(w, ref)
+        # RMSprop on a fp32 gradient and on codes
+        for grad, prec in ((g, None), (codes, 0.37)):
+            w, r, wref, rref = w0.clone(), r0.clone(), w0.clone(), r0.clone()
+            cn.rmsprop_update(r, grad, w, 0.9, 0.001, precision=prec)
+            pieces(lambda rr, gg, ww: cn.rmsprop_update(rr, gg, ww, 0.9, 0.001, precision=prec), rref, grad, wref)
+            assert same(w, wref) and same(r, rref)
