@@ -65,12 +65,13 @@ def test_decompress_axpy_equals_the_unfused_kernels_and_takes_device_precision(d
     assert torch.equal(w2[1:].view(torch.int32), w_ref[1:].view(torch.int32)) and w2[0] == w[0]
 
 
-@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 1023, 4096, 4097, 1_000_003, 8_388_608 + 6])
+@pytest.mark.parametrize("n", [0, 1, 3, 4, 5, 1023, 4096, 4097, 1_000_003, 8_388_608 + 6, (1 << 26) + 2 * 16384 + 7])
 @pytest.mark.parametrize("prec", [0.0371, 1e-30, 0.0])
 def test_compress_axpy_is_compress_then_decompress_axpy(dev, n, prec):
     """Codes and updated array of the one-pass kernel against the two kernels it replaces and, for the
     sizes the checker finishes quickly, against the checker.  A precision of 1e-30 or 0 takes the
-    encoder's search instead of its table."""
+    encoder's search instead of its table.  The largest size is beyond the cache and takes the form that draws
+    its tiles from a counter."""
     import torch
     import clusternet_amd as cn
     rng = np.random.default_rng(n + 3)
