@@ -768,10 +768,10 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
         // tile kernel on a resident grid-stride grid: 1.96 ms).
         if (y)
             hipLaunchKernelGGL((compress_stream_kernel<1024, 4, true>), dim3(ctx->num_cu), dim3(1024), lds, st, x, precision,
-                               precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->tile_queue, alpha, y);
+                               precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->next_tile_counter(), alpha, y);
         else if (n >= kBeyondCacheFrom && n < ((size_t)1 << 40))
             hipLaunchKernelGGL((compress_stream_kernel<1024, 12, false>), dim3(ctx->num_cu), dim3(1024), sizeof(EncodeShared), st, x,
-                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->tile_queue,
+                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->next_tile_counter(),
                                0.0f, (float *)nullptr);
         else
             hipLaunchKernelGGL((compress_stream_kernel<512, 10, false>), dim3(ctx->num_cu * 2), dim3(512), sizeof(EncodeShared), st, x,

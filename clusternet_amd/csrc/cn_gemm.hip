@@ -921,6 +921,7 @@ static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, 
 
 static int g_force_tile_n = 0;
 static bool g_wide_store = true;
+static bool g_w8_rows = true;  // test hook: false keeps the tiled kernel for every product on 8-bit weights
 static bool g_epilogue_in_kernel = true;  // test hook: false sends every fused product through the workspace
 
 // What follows the product instead of its delivery: bias and maxout (the forward pass of a maxout layer; `bias`
@@ -983,6 +984,16 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         CN_HIP(hipGetLastError());
         if (then) return finish_from(C);
         return CN_OK;
+    }
+    if (w8 && !then && g_w8_rows && g_force_tile_n == 0) {
+        // a handful of rows: the kernel that decodes straight into the matrix instruction's registers
+        const int chunks = gemm_w8_rows_splits(M, N, K, A, lda, (const uint8_t *)B, ldb, scale, C, ldc, ctx->num_cu, ctx->workspace_bytes);
+        if (chunks > 1 || (chunks == 1 && !amax)) {
+            s = gemm_w8_rows(chunks, M, N, K, A, lda, (const uint8_t *)B, ldb, scale, C, ldc, ctx->table, ctx->workspace, ctx->device, st);
+            if (s != CN_OK) return s;
+            if (chunks > 1) return add_chunk_planes(ctx->workspace, ctx->num_cu, chunks, M, N, C, ldc, amax, st);
+            return CN_OK;
+        }
     }
     GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->plan_bytes, g_force_tile_n);
     // K not split, whole 128-row tiles and pools of 1, 2 or 4: bias + maxout, or the expansion, happen in the
@@ -1105,6 +1116,7 @@ extern "C" {
 void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
 
 // Test hook: 0 = bias + maxout and the maxout expansion never run inside the product's write-out.
+void cn_host_gemm_w8_rows(int enabled) { g_w8_rows = enabled != 0; }
 void cn_host_gemm_epilogue_in_kernel(int enabled) { g_epilogue_in_kernel = enabled != 0; }
 
 // Test and tuning hook: 0 = let the planner choose the tile, 128 / 256 = force that width of the 128-row

@@ -24,6 +24,8 @@ cn_status hip_fail(hipError_t e, const char *what, const char *file, int line);
 void host_table(float out[126]);
 
 // ---- per-device state ------------------------------------------------------------------------
+constexpr int kTileQueues = 32;  // ticket counters of the streaming kernels, each on a 128-byte line of its own
+constexpr int kTileQueueWords = kTileQueues * 32;
 struct Context {
     bool ready = false;
     int device = -1;
@@ -37,9 +39,12 @@ struct Context {
     uint32_t *tickets = nullptr;         // running maximum and arrival count of the max reductions (kTicketWords words)
     double *sum_scratch = nullptr;       // per-workgroup partial sums (1024 doubles)
     uint32_t *tile_queue = nullptr;      // ticket counters of the streaming kernels (kTileQueueWords words, left at 0)
+    unsigned tile_queue_turn = 0;        // which of the counters the next launch takes
+    // A counter for one launch of a kernel that draws its tiles.  The launches take the kTileQueues counters in turn, so
+    // that kernels which overlap (on different streams) do not draw from the same one unless that many are in flight.
+    uint32_t *next_tile_counter() { return tile_queue + (size_t)(tile_queue_turn++ % (unsigned)kTileQueues) * 32u; }
 };
 constexpr int kMaxDevices = 16;
-constexpr int kTileQueueWords = 32;  // one 128-byte line; word 0 is the counter
 constexpr int kReduceSlots = 4096;
 // Max reductions: a running maximum and an arrival count per group of kTicketGroup workgroups and one pair for
 // the groups, every pair on a 128-byte line of its own, all left at 0.
@@ -97,6 +102,13 @@ struct GemmPlan {
 // C = sum of `splits` M x N planes held at the start of the workspace (ascending order); optional max |C|.
 cn_status add_chunk_planes(const void *planes, int num_cu, int splits, int64_t M, int64_t N, float *C, int64_t ldc,
                            uint32_t *amax, hipStream_t st);
+
+// The product on 8-bit weights for at most 64 rows (cn_gemm_w8_rows.hip): number of K chunks if it applies, else 0;
+// with more than one chunk the planes land at the start of `workspace` for add_chunk_planes.
+int gemm_w8_rows_splits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W, int64_t ldw,
+                        float scale, const float *C, int64_t ldc, int num_cu, size_t workspace_bytes);
+cn_status gemm_w8_rows(int splits, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W, int64_t ldw,
+                       float scale, float *C, int64_t ldc, const float *table, void *workspace, int device, hipStream_t st);
 
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 

@@ -98,7 +98,7 @@ static cn_status launch_flat(Context *ctx, hipStream_t st, const float *a, const
         // beyond the cache: one workgroup per compute unit, tiles of 512 lanes x 8 vectors drawn from the counter (the
         // weight update on 819.2 M elements: 1.46 ms; 1024 x 4: 1.48, 256 x 16: 1.50, 512 x 4: 1.49, 1024 x 8: 1.58)
         hipLaunchKernelGGL((flat_kernel<Op, kTwo, true, kFT, 8, true>), dim3(ctx->num_cu), dim3(kFT), 0, st, a, b, n, out, f,
-                           ctx->tile_queue);
+                           ctx->next_tile_counter());
     } else if (vec) {
         // a workgroup per tile of 512 lanes x 2 vectors, as many workgroups as tiles
         int64_t grid = (n / 4 + kFT * 2 - 1) / (kFT * 2);

@@ -11,7 +11,7 @@
 // The counter must be 0 when the kernel starts and is left at 0: every workgroup draws until its ticket is past the
 // last tile, so exactly gridDim.x tickets fail, and the workgroup that draws the last of them (ticket tiles +
 // gridDim.x - 1) knows that nobody will draw again and clears the counter.  Kernels that share a counter must not
-// overlap (the library's calls are issued on one stream at a time).
+// overlap: the library keeps several and gives them to its launches in turn (Context::next_tile_counter).
 #pragma once
 
 #include "cn_internal.h"

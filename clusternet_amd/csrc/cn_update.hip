@@ -178,7 +178,7 @@ cn_status axpy_impl(const uint8_t *codes, float precision, const float *precisio
     uint32_t *const none = nullptr;
     if (vec && n >= kDrawnFrom && n < kDrawnBelow)
         hipLaunchKernelGGL((decompress_axpy_kernel<true, kDrawnVecs, true>), dim3(ctx->num_cu), dim3(kThreads), 0, st, codes,
-                           precision, precision_dev, alpha, n, y, ctx->table, ctx->tile_queue);
+                           precision, precision_dev, alpha, n, y, ctx->table, ctx->next_tile_counter());
     else if (vec)
         hipLaunchKernelGGL((decompress_axpy_kernel<true, kTileVecsSmall, false>), dim3(grid), dim3(kThreads), 0, st, codes,
                            precision, precision_dev, alpha, n, y, ctx->table, none);
@@ -200,7 +200,7 @@ cn_status rmsprop_impl(float *rms, const float *grad, const uint8_t *codes, floa
     const bool vec = aligned(rms, 16) && aligned(w, 16) && (codes ? aligned(codes, 4) : aligned(grad, 16));
     const bool drawn = vec && n >= kDrawnFrom && n < kDrawnBelow;
     const int grid = drawn ? ctx->num_cu : grid_of(ctx, n, vec);
-    uint32_t *const queue = drawn ? ctx->tile_queue : nullptr;
+    uint32_t *const queue = drawn ? ctx->next_tile_counter() : nullptr;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, st, rms, grad, codes, precision, precision_dev, w, mult, rate, n,
                            ctx->table, queue);

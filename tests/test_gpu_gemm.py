@@ -299,6 +299,49 @@ def test_fused_w8_ragged(dev, shape):
     assert e1 <= 1e-4 and e2 <= 1e-4, (e1, e2)
 
 
+@pytest.mark.parametrize("shape", [(1, 128, 64), (8, 132, 72), (31, 1000, 512), (32, 4096, 1024), (33, 260, 1024),
+                                   (64, 4100, 264), (64, 8192, 4096)])
+def test_fused_w8_few_rows(dev, shape):
+    """Products of at most 64 rows on 8-bit weights take a kernel of their own (codes decoded straight into the
+    matrix instruction's registers, K dealt to the eight wavefronts of a workgroup and to chunks).  Against the CPU
+    checker, against the tiled kernel it replaces there (the hook keeps it), with operands that sit inside wider
+    arrays, and with one-hot rows, for which every output must be the decoded weight itself, bit for bit."""
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    A = rng.normal(0, 1, (M, K)).astype(np.float32)
+    W = rng.integers(0, 256, (K, N), dtype=np.uint8)
+    Cref, Cabs = oracle.gemm_with_abs(A, oracle.decompress(W, 0.25))
+    At, Wt = _t(A, dev), _t(W, dev)
+    got = cn.gemm_w8(At, Wt, 0.25).cpu().numpy()
+    e1, e2 = gemm_errors(got, Cref, Cabs)
+    assert e1 <= 1e-4 and e2 <= 1e-4, (e1, e2)
+    try:
+        L.lib().cn_host_gemm_w8_rows(0)
+        tiled = cn.gemm_w8(At, Wt, 0.25).cpu().numpy()
+    finally:
+        L.lib().cn_host_gemm_w8_rows(1)
+    assert np.abs(tiled - got).max() / np.abs(Cref).max() <= 1e-4
+    # operands inside wider arrays (leading dimensions larger than the rows), output into a wider array too
+    Aw = torch.zeros((M, K + 8), device=dev)
+    Aw[:, 4:4 + K] = At
+    Ww = torch.full((K, N + 12), 77, dtype=torch.uint8, device=dev)
+    Ww[:, 8:8 + N] = Wt
+    Cw = torch.full((M, N + 4), 7.0, device=dev)
+    cn.gemm_w8(Aw[:, 4:4 + K], Ww[:, 8:8 + N], 0.25, out=Cw[:, :N])
+    assert np.array_equal(Cw[:, :N].cpu().numpy().view(np.uint32), got.view(np.uint32))
+    assert float(Cw[:, N:].min()) == 7.0 and float(Cw[:, N:].max()) == 7.0
+    # one-hot rows: the product is a row of decoded weights
+    ks = rng.integers(0, K, M)
+    onehot = np.zeros((M, K), np.float32)
+    onehot[np.arange(M), ks] = 1.0
+    rows = cn.gemm_w8(_t(onehot, dev), Wt, 0.0371).cpu().numpy()
+    want = oracle.decompress(W[ks], 0.0371)
+    assert np.array_equal(rows.view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("shape,ta,tb", [((128, 300, 64), False, False), ((1000, 257, 128), True, False),
                                           ((37, 1029, 515), False, True), ((128, 512, 8192), False, False),
                                           ((3, 5, 7), True, True), ((64, 64, 1), False, False)])
