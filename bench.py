@@ -232,11 +232,10 @@ def bench_fused(torch, cn, dev):
         res["batch%d" % b] = {"fused_us": t_f * 1e3, "decompress_plus_dot_us": t_u * 1e3,
                               "dot_fp32_only_us": t_g * 1e3, "speedup": t_u / t_f,
                               "fused_TFLOPs": 2.0 * b * 4096 * 4096 / t_f / 1e9}
-        if b <= 64:
-            # a handful of rows takes a kernel of its own; the tiled kernel it replaces there, for comparison
-            cn.lib().cn_host_gemm_w8_rows(0)
-            res["batch%d" % b]["fused_tiled_kernel_us"] = time_region(torch, lambda: cn.gemm_w8(A, codes, scale, C), 200, 5) * 1e3
-            cn.lib().cn_host_gemm_w8_rows(1)
+        # these batches take the kernel that decodes into registers; the tiled kernel it replaces there, for comparison
+        cn.lib().cn_host_gemm_w8_rows(0)
+        res["batch%d" % b]["fused_tiled_kernel_us"] = time_region(torch, lambda: cn.gemm_w8(A, codes, scale, C), 200, 5) * 1e3
+        cn.lib().cn_host_gemm_w8_rows(1)
     return res
 
 

@@ -986,7 +986,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         return CN_OK;
     }
     if (w8 && !then && g_w8_rows && g_force_tile_n == 0) {
-        // a handful of rows: the kernel that decodes straight into the matrix instruction's registers
+        // up to 1024 rows: the kernel that decodes straight into the matrix instruction's registers
         const int chunks = gemm_w8_rows_splits(M, N, K, A, lda, (const uint8_t *)B, ldb, scale, C, ldc, ctx->num_cu, ctx->workspace_bytes);
         if (chunks > 1 || (chunks == 1 && !amax)) {
             s = gemm_w8_rows(chunks, M, N, K, A, lda, (const uint8_t *)B, ldb, scale, C, ldc, ctx->table, ctx->workspace, ctx->device, st);

@@ -1,12 +1,12 @@
-// C = A . decode(W8) for products of a handful of rows (at most 64), gfx950.
+// C = A . decode(W8) for products of up to 1024 rows, gfx950.
 //
-// With so few rows the product is one pass over the codes: 16.8 MB for a 4096 x 4096 layer, against 67 MB for
+// With few rows the product is one pass over the codes: 16.8 MB for a 4096 x 4096 layer, against 67 MB for
 // fp32 weights.  The tiled kernel (cn_gemm.hip) decodes a stage of codes into LDS, waits at a barrier and reads
 // the values back as matrix fragments: three LDS operations per weight and a barrier between decode and use,
 // which left it slower than the fp32 product it should beat (24 us against 20 us at 32 x 4096 x 4096).
 //
 // Here a wavefront decodes straight into the registers the matrix instruction reads:
-//   * a workgroup of eight wavefronts owns 128 columns of the result and one chunk of K; each wavefront takes a
+//   * a workgroup of eight wavefronts owns 128 columns of 32 or 64 rows of the result and one chunk of K; each wavefront takes a
 //     contiguous eighth of the chunk and all 128 columns, so no weight is shared between wavefronts and nothing
 //     of B passes through LDS except the 1 KB decode table;
 //   * lane (h, i) of a wavefront loads, for a group of 8 k, the four code words W[k0 + 4h + j][n0 + 4i .. 4i + 3],
@@ -29,10 +29,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
-constexpr int kWaves = 8;
-constexpr int kLanes = kWaves * 64;
 constexpr int kCols = 128;     // columns of a workgroup
-constexpr size_t kLdsBytes = (size_t)(kWaves * 32 * kCols + 256) * sizeof(float);
+constexpr size_t lds_bytes(int waves) { return (size_t)(waves * 32 * kCols + 256) * sizeof(float); }
 
 struct RowsArgs {
     const float *A;
@@ -43,7 +41,7 @@ struct RowsArgs {
     int64_t M, N;
     int64_t groups;        // K / 8
     float scale;
-    int splits, tiles_n;
+    int splits, tiles_n, tiles_m;
 };
 
 __device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
@@ -51,8 +49,11 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
 }
 
-template <int FM, int kAhead>  // blocks of 32 rows (1 or 2); groups of 8 k whose loads are in flight
-__global__ __launch_bounds__(kLanes) void gemm_w8_rows_kernel(RowsArgs g) {
+// FM blocks of 32 rows per workgroup (row tiles of 32 FM rows), kAhead groups of 8 k whose loads are in flight, kWaves
+// wavefronts that share the workgroup's chunk of K.
+template <int FM, int kAhead, int kWaves>
+__global__ __launch_bounds__(kWaves * 64) void gemm_w8_rows_kernel(RowsArgs g) {
+    constexpr int kLanes = kWaves * 64;
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float *lut = smem + kWaves * 32 * kCols;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5, l32 = lane & 31;
@@ -67,9 +68,12 @@ __global__ __launch_bounds__(kLanes) void gemm_w8_rows_kernel(RowsArgs g) {
         lut[254] = g.scale;
         lut[255] = -g.scale;
     }
-    const int split = __builtin_amdgcn_readfirstlane((int)(blockIdx.x / (unsigned)g.tiles_n));
-    const int tn = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % (unsigned)g.tiles_n));
-    const int64_t n0 = (int64_t)tn * kCols;
+    // row tiles of one column tile and chunk are neighbours: they read the same codes at the same time
+    const unsigned column_unit = blockIdx.x / (unsigned)g.tiles_m;
+    const int tm = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % (unsigned)g.tiles_m));
+    const int split = __builtin_amdgcn_readfirstlane((int)(column_unit / (unsigned)g.tiles_n));
+    const int tn = __builtin_amdgcn_readfirstlane((int)(column_unit % (unsigned)g.tiles_n));
+    const int64_t n0 = (int64_t)tn * kCols, m0 = (int64_t)tm * 32 * FM;
     // the groups of 8 k are dealt to the wavefronts of all chunks in contiguous, nearly equal runs
     const int64_t parts = (int64_t)g.splits * kWaves, part = (int64_t)split * kWaves + wave;
     const int64_t g0 = __builtin_amdgcn_readfirstlane((int)(g.groups * part / parts));
@@ -81,7 +85,7 @@ __global__ __launch_bounds__(kLanes) void gemm_w8_rows_kernel(RowsArgs g) {
     const rsrc_t ra = make_rsrc(g.A, (uint32_t)(((g.M - 1) * g.lda + g.groups * 8) * (int64_t)sizeof(float)));
     const int64_t cols_here = g.N - n0 < kCols ? g.N - n0 : kCols;
     const rsrc_t rw = make_rsrc(g.W + g0 * 8 * g.ldw + n0, count > 0 ? (uint32_t)((count * 8 - 1) * g.ldw + cols_here) : 0u);
-    const uint32_t a_lane = (uint32_t)(l32 * g.lda * (int64_t)sizeof(float)) + 16u * half;
+    const uint32_t a_lane = (uint32_t)((m0 + l32) * g.lda * (int64_t)sizeof(float)) + 16u * half;
     const uint32_t a_block = (uint32_t)(32 * g.lda * (int64_t)sizeof(float));
     const uint32_t w_lane = (uint32_t)(4 * half * g.ldw) + 4u * l32;
     const uint32_t w_row = (uint32_t)g.ldw;
@@ -138,7 +142,7 @@ __global__ __launch_bounds__(kLanes) void gemm_w8_rows_kernel(RowsArgs g) {
         }
     }
 
-    // The eight partial tiles of the workgroup: through LDS, summed in wavefront order.  Accumulator r of a lane holds
+    // The partial tiles of the workgroup's wavefronts: through LDS, summed in wavefront order.  Accumulator r of a lane holds
     // row 8 (r / 4) + 4 half + (r % 4) of its block; its four blocks are four consecutive columns, 4 l32 .. 4 l32 + 3.
     float *mine = smem + wave * 32 * kCols;
     float *dst = g.out + (g.splits > 1 ? (int64_t)split * g.plane : 0);
@@ -158,7 +162,7 @@ __global__ __launch_bounds__(kLanes) void gemm_w8_rows_kernel(RowsArgs g) {
             f32x4 s = *reinterpret_cast<const f32x4 *>(smem + row * kCols + col);
 #pragma unroll
             for (int w = 1; w < kWaves; ++w) s = s + *reinterpret_cast<const f32x4 *>(smem + w * 32 * kCols + row * kCols + col);
-            const int64_t m = mi * 32 + row, n = n0 + col;
+            const int64_t m = m0 + mi * 32 + row, n = n0 + col;
             if (m < g.M && n < g.N) *reinterpret_cast<f32x4 *>(dst + m * g.out_ld + n) = s;
         }
     }
@@ -166,24 +170,33 @@ __global__ __launch_bounds__(kLanes) void gemm_w8_rows_kernel(RowsArgs g) {
 
 }  // namespace
 
-// Whether the product takes this kernel, and if so how many K chunks (0 = no): few rows, whole 16-byte and 4-byte
-// accesses, a finite scale (rows and groups outside a wavefront's run are multiplied by zero), offsets that fit
-// 32 bits.
+// Products of more rows than this stay with the tiled kernel of cn_gemm.hip: every 64-row tile decodes the codes it
+// needs by itself, and from about 2000 rows on that costs more than a tile's barriers (4096 x 4096 weights: 42.6 us
+// against 50.1 us at 128 rows, 134.5 against 142.6 at 512, 267 against 272 at 1024, 530 against 519 at 2048).
+constexpr int64_t kRowsUpto = 1024;
+
+// Whether the product takes this kernel, and if so how many K chunks (0 = no): whole 16-byte and 4-byte accesses, a
+// finite scale (rows and groups outside a wavefront's run are multiplied by zero), offsets that fit 32 bits.
+// Row tiles of 32 rows for up to 32 rows, of 64 rows beyond (tiles of 128 rows would need 256 accumulator registers
+// per lane; the compiler spills them); eight wavefronts per workgroup.
+static int rows_per_tile(int64_t M) { return M <= 32 ? 32 : 64; }
+static int waves_for(int64_t) { return 8; }
+
 int gemm_w8_rows_splits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W, int64_t ldw,
                         float scale, const float *C, int64_t ldc, int num_cu, size_t workspace_bytes) {
     auto aligned_to = [](const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; };
-    if (M < 1 || M > 64 || N < 4 || K < 64 || N % 4 != 0 || K % 8 != 0) return 0;
+    if (M < 1 || M > kRowsUpto || N < 4 || K < 64 || N % 4 != 0 || K % 8 != 0) return 0;
     if (!aligned_to(A, 16) || lda % 4 != 0 || !aligned_to(W, 4) || ldw % 4 != 0) return 0;
     if (!(scale == scale) || scale - scale != 0.0f) return 0;  // NaN or infinite
     if ((uint64_t)K * (uint64_t)ldw >= (1ull << 31) || (uint64_t)M * (uint64_t)lda * 4 >= (1ull << 31)) return 0;
-    const int64_t tiles_n = (N + kCols - 1) / kCols, groups = K / 8;
+    const int64_t tiles_n = (N + kCols - 1) / kCols, tiles_m = (M + rows_per_tile(M) - 1) / rows_per_tile(M), groups = K / 8;
     // one workgroup per compute unit; a wavefront wants at least four groups
-    int64_t splits = (num_cu + tiles_n - 1) / tiles_n;
-    if (splits > groups / (kWaves * 4)) splits = groups / (kWaves * 4);
+    int64_t splits = (num_cu + tiles_n * tiles_m - 1) / (tiles_n * tiles_m);
+    if (splits > groups / (waves_for(M) * 4)) splits = groups / (waves_for(M) * 4);
     if (splits < 1) splits = 1;
     while (splits > 1 && (size_t)splits * (size_t)M * (size_t)N * sizeof(float) > workspace_bytes) --splits;
     if (splits == 1 && (!aligned_to(C, 16) || ldc % 4 != 0)) return 0;
-    if (tiles_n * splits > 0x7fffffffLL) return 0;
+    if (tiles_n * tiles_m * splits > 0x7fffffffLL) return 0;
     return (int)splits;
 }
 
@@ -194,18 +207,19 @@ cn_status gemm_w8_rows(int splits, int64_t M, int64_t N, int64_t K, const float 
     g.lda = lda; g.ldw = ldw;
     g.M = M; g.N = N; g.groups = K / 8; g.scale = scale;
     g.splits = splits; g.tiles_n = (int)((N + kCols - 1) / kCols);
+    g.tiles_m = (int)((M + rows_per_tile(M) - 1) / rows_per_tile(M));
     if (splits > 1) { g.out = (float *)workspace; g.out_ld = N; g.plane = M * N; }
     else            { g.out = C; g.out_ld = ldc; g.plane = 0; }
     static OncePerDevice configured;
     if (configured.first(device)) {
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8_rows_kernel<1, 4>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes));
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8_rows_kernel<2, 4>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8_rows_kernel<1, 4, 8>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(8)));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_w8_rows_kernel<2, 4, 8>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes(8)));
     }
-    const dim3 grid((unsigned)(g.tiles_n * splits));
-    if (M <= 32) hipLaunchKernelGGL((gemm_w8_rows_kernel<1, 4>), grid, dim3(kLanes), kLdsBytes, st, g);
-    else         hipLaunchKernelGGL((gemm_w8_rows_kernel<2, 4>), grid, dim3(kLanes), kLdsBytes, st, g);
+    const dim3 grid((unsigned)(g.tiles_n * g.tiles_m * splits));
+    if (M <= 32)      hipLaunchKernelGGL((gemm_w8_rows_kernel<1, 4, 8>), grid, dim3(512), lds_bytes(8), st, g);
+    else              hipLaunchKernelGGL((gemm_w8_rows_kernel<2, 4, 8>), grid, dim3(512), lds_bytes(8), st, g);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }

@@ -103,7 +103,7 @@ struct GemmPlan {
 cn_status add_chunk_planes(const void *planes, int num_cu, int splits, int64_t M, int64_t N, float *C, int64_t ldc,
                            uint32_t *amax, hipStream_t st);
 
-// The product on 8-bit weights for at most 64 rows (cn_gemm_w8_rows.hip): number of K chunks if it applies, else 0;
+// The product on 8-bit weights for up to 1024 rows (cn_gemm_w8_rows.hip): number of K chunks if it applies, else 0;
 // with more than one chunk the planes land at the start of `workspace` for add_chunk_planes.
 int gemm_w8_rows_splits(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W, int64_t ldw,
                         float scale, const float *C, int64_t ldc, int num_cu, size_t workspace_bytes);

@@ -32,7 +32,7 @@ void cn_host_gemm_wide_store(int enabled);
 /* 0 = cn_gemm_f32_bias_maxout / cn_gemm_f32_expand_maxout_grad never take the kernel that applies them in the
  * product's own write-out (K not split, whole tiles): they then pass through the workspace, which the tests compare
  * against. */
-/* 0 keeps the tiled kernel for every product on 8-bit weights; 1 (default) lets products of at most 64 rows take the
+/* 0 keeps the tiled kernel for every product on 8-bit weights; 1 (default) lets products of up to 1024 rows take the
  * kernel that decodes straight into registers. */
 void cn_host_gemm_w8_rows(int enabled);
 void cn_host_gemm_epilogue_in_kernel(int enabled);

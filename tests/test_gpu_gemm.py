@@ -300,9 +300,9 @@ def test_fused_w8_ragged(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(1, 128, 64), (8, 132, 72), (31, 1000, 512), (32, 4096, 1024), (33, 260, 1024),
-                                   (64, 4100, 264), (64, 8192, 4096)])
+                                   (64, 4100, 264), (64, 8192, 4096), (65, 128, 4096), (200, 300, 512), (1024, 1024, 256)])
 def test_fused_w8_few_rows(dev, shape):
-    """Products of at most 64 rows on 8-bit weights take a kernel of their own (codes decoded straight into the
+    """Products of up to 1024 rows on 8-bit weights take a kernel of their own (codes decoded straight into the
     matrix instruction's registers, K dealt to the eight wavefronts of a workgroup and to chunks).  Against the CPU
     checker, against the tiled kernel it replaces there (the hook keeps it), with operands that sit inside wider
     arrays, and with one-hot rows, for which every output must be the decoded weight itself, bit for bit."""
