@@ -358,3 +358,45 @@ def test_compression_beyond_the_cache_draws_its_tiles(dev, codec_form):
     # a smaller tensor in between takes the other kernels and must not be disturbed by the counter
     got = cn.compression_8bit(bt[:1 << 20], 0.77)
     assert torch.equal(got, ct[:1 << 20])
+
+
+def test_kernels_that_draw_tiles_replay_from_a_graph(dev, codec_form):
+    """The kernels that draw their tiles leave their counter at zero, so a captured graph of them can be replayed:
+    compression and the weight update beyond the cache, captured once, replayed three times with eager calls of the
+    same kernels in between, every replay against the eager result."""
+    if codec_form != "literal_for_small_tensors":
+        pytest.skip("one run is enough")
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(21)
+    n = (1 << 26) + 5 * 4096 + 3
+    x = torch.randn(n, device=dev, generator=gen) * 0.02
+    w0 = torch.randn(n, device=dev, generator=gen)
+    want_codes = cn.compression_8bit(x, 0.11)
+    want_w = w0.clone()
+    L.sgd_update(want_w, x, 0.5)
+    codes = torch.zeros(n, dtype=torch.uint8, device=dev)
+    w = w0.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # warm-up on the capturing stream, as the capture API asks
+        cn.compression_8bit(x, 0.11, out=codes)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cn.compression_8bit(x, 0.11, out=codes)
+        L.sgd_update(w, x, 0.5)
+    for _ in range(3):
+        codes.zero_()
+        w.copy_(w0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(codes, want_codes)
+        assert torch.equal(w.view(torch.int32), want_w.view(torch.int32))
+        # eager calls of the same kernels between the replays
+        assert torch.equal(cn.compression_8bit(x, 0.11), want_codes)
+        again = w0.clone()
+        L.sgd_update(again, x, 0.5)
+        assert torch.equal(again.view(torch.int32), want_w.view(torch.int32))
