@@ -89,6 +89,8 @@ def lib():
     L.cn_host_codec_literal_upto.restype = None
     L.cn_host_gemm_w8_rows.argtypes = [C.c_int]
     L.cn_host_gemm_w8_rows.restype = None
+    L.cn_host_tile_counters_in_use.argtypes = []
+    L.cn_host_tile_counters_in_use.restype = C.c_int
     L.cn_host_reduction_fences.argtypes = [C.c_int]
     L.cn_host_reduction_fences.restype = None
     L.cn_host_csr_strip_kernel.argtypes = [C.c_int]

@@ -170,6 +170,19 @@ const char *cn_last_error(void) { return g_error; }
 
 void cn_host_reduction_fences(int enabled) { g_reduction_fences = enabled != 0; }
 
+// Test hook: after a device synchronisation, the number of ticket counters of the current device that are not zero
+// (kernels that draw their tiles leave theirs at zero), or -1 if the device is not initialised.
+int cn_host_tile_counters_in_use(void) {
+    Context *c;
+    if (current_context(&c) != CN_OK) return -1;
+    uint32_t words[kTileQueueWords];
+    if (hipDeviceSynchronize() != hipSuccess) return -1;
+    if (hipMemcpy(words, c->tile_queue, sizeof(words), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    int busy = 0;
+    for (int q = 0; q < kTileQueues; ++q) busy += words[q * 32] != 0u;
+    return busy;
+}
+
 cn_status cn_init(int device) {
     std::lock_guard<std::mutex> lock(g_mutex);
     return init_device(device);

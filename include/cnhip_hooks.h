@@ -49,6 +49,10 @@ void cn_host_codec_literal_upto(size_t n);
  * two by a data dependence; the last workgroup acquires either way.  Same results; for tests of that equality. */
 void cn_host_reduction_fences(int enabled);
 
+/* Synchronises the current device and returns how many of its ticket counters (the ones the streaming kernels draw
+ * their tiles from) are not zero: 0 whenever no kernel is running; -1 if the device is not initialised. */
+int cn_host_tile_counters_in_use(void);
+
 /* Nonzero: cn_absmax_compress_8bit runs as one launch (abs-max, a wait across the resident grid, compression) for
  * aligned tensors below 2^26 elements instead of as two kernels.  Same bits. */
 void cn_host_absmax_compress_single_launch(int enabled);

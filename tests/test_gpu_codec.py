@@ -358,6 +358,8 @@ def test_compression_beyond_the_cache_draws_its_tiles(dev, codec_form):
     # a smaller tensor in between takes the other kernels and must not be disturbed by the counter
     got = cn.compression_8bit(bt[:1 << 20], 0.77)
     assert torch.equal(got, ct[:1 << 20])
+    from clusternet_amd import _lib as L
+    assert L.lib().cn_host_tile_counters_in_use() == 0  # every kernel that drew tiles left its counter at zero
 
 
 def test_kernels_that_draw_tiles_replay_from_a_graph(dev, codec_form):

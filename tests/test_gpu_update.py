@@ -207,3 +207,4 @@ def test_tensors_beyond_the_cache_take_drawn_tiles_and_give_the_same_bits(dev, c
             cn.rmsprop_update(r, grad, w, 0.9, 0.001, precision=prec)
             pieces(lambda rr, gg, ww: cn.rmsprop_update(rr, gg, ww, 0.9, 0.001, precision=prec), rref, grad, wref)
             assert same(w, wref) and same(r, rref)
+    assert L.lib().cn_host_tile_counters_in_use() == 0  # every kernel that drew tiles left its counter at zero
