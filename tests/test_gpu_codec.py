@@ -226,8 +226,8 @@ def test_large_tensor_by_tiling(dev):
 
 
 def test_streaming_forms_ragged_sizes_offsets_and_fallback(dev):
-    """Tensors of 2^24 elements and more take the one-workgroup-per-compute-unit streaming kernels, whose last tile
-    is bounded by a buffer descriptor instead of a per-element test: sizes round a tile boundary, tails of 1 to 3
+    """Compression of 2^24 elements and more takes the streaming kernel, and decompression a workgroup per tile; in both
+    the last tile is bounded by a buffer descriptor instead of a per-element test: sizes round a tile boundary, tails of 1 to 3
     elements, starts that are not 16-byte aligned (which fall back to the element-wise kernel), and a precision for
     which no table can be built (the literal procedure per element), all against the CPU checker."""
     import torch
@@ -268,8 +268,8 @@ def test_streaming_forms_ragged_sizes_offsets_and_fallback(dev):
 
 
 def test_decode_through_a_given_table(dev):
-    """cn_decode_8bit_lut: out[i] = lut[codes[i]] for any 256-entry table, on both kernels (tile and streaming),
-    ragged sizes and unaligned starts."""
+    """cn_decode_8bit_lut: out[i] = lut[codes[i]] for any 256-entry table, on both kernels (a workgroup per tile, and
+    element by element), ragged sizes and unaligned starts."""
     import torch
     from clusternet_amd import _lib as L
     rng = np.random.default_rng(8)
