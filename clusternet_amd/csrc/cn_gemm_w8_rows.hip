@@ -92,7 +92,8 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_w8_rows_kernel(RowsArgs g) {
 
     uint32_t c[kAhead][4];
     f32x4 a[kAhead][FM];
-    auto request = [&](int slot, int i) {  // group g0 + i; beyond the run the code words read zero and are not used
+    auto request = [&](int slot, int i) {  // group g0 + i; a request beyond the run reads the last group again (unused)
+        i = i < count ? i : (count > 0 ? count - 1 : 0);
         const uint32_t w_base = __builtin_amdgcn_readfirstlane((int)((uint32_t)i * 8u * w_row));
         const uint32_t a_base = __builtin_amdgcn_readfirstlane((int)((uint32_t)((g0 + i) * 8 * (int64_t)sizeof(float))));
 #pragma unroll

@@ -17,6 +17,8 @@
 // With X the 128 x 100000 batch:  X W = CSR(X) W and X^T E = CSR(X^T) E.
 // Sums run over the nonzeros in ascending order with a rounded product and a rounded addition per
 // term, so the results are reproducible to the bit.
+#include <type_traits>
+
 #include "cn_internal.h"
 #include "cn_encode_table.h"
 
@@ -325,6 +327,20 @@ constexpr int kBAhead = 1;     // B values are requested this many rows ahead
 constexpr int kBRing = 2 * kBAhead;
 constexpr int kFixed = 4;      // B rows requested ahead per row
 
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kRowAuxNt = 2;  // cache policy bit of the buffer instructions: nt
+__device__ __forceinline__ rsrc_t row_rsrc(const void *base, uint32_t bytes) {
+    // 0x00020000: 32-bit untyped data; accesses at or beyond `bytes` read zero and write nothing
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+__device__ __forceinline__ f32x4 as_f32x4(u32x4 v) {
+    return f32x4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+}
+__device__ __forceinline__ u32x4 as_u32x4(f32x4 v) {
+    return u32x4{__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+}
+
 struct RowBlockMeta {
     int rp;    // lane l: row_ptr[first row + l], l <= 16
     int c;     // lane l: column index of the block's nonzero l
@@ -336,7 +352,8 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
     int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
     const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks, uint32_t *amax_out,
     const float *__restrict__ precision_ptr, uint8_t *__restrict__ codes, float *__restrict__ w, int64_t ldw, float alpha,
-    float *__restrict__ rms, float rate, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table) {
+    float *__restrict__ rms, float rate, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table,
+    uint32_t b_bytes) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
     float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // decode table times alpha
@@ -390,15 +407,19 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
     const int64_t unit_first = (int64_t)blockIdx.x * (row_threads<kMode>() / 64) + (t >> 6);
     const uint32_t b_row_bytes = (uint32_t)(ldb * (int64_t)sizeof(float));  // B spans less than 4 GiB on this path
     const char *Bbytes = reinterpret_cast<const char *>(B);
+    // Everything a row touches is addressed through buffer descriptors: the part of an address that is the same for all
+    // lanes (the row) travels in a scalar register, the lane's part is computed once per unit, and no row spends vector
+    // instructions on 64-bit pointer arithmetic.
+    const rsrc_t rb = row_rsrc(B, b_bytes);
+    const uint32_t w_row_bytes = (uint32_t)(ldw * (int64_t)sizeof(float));
     // Where a unit lives: computed once per unit, the rows then only add multiples of the leading dimensions.
     struct UnitPos {
         int64_t row0;
         int rows;           // rows of the block inside the matrix (1 .. 16)
         bool live;          // the lane's four columns exist
         uint32_t lane_off;  // byte offset of the lane's columns inside a row of B (column 0 for idle lanes)
-        float *wp;          // weights of row0 at the lane's columns
-        float *rp2;         // running mean squares of row0 at the lane's columns (RMSprop)
-        uint8_t *cp;        // codes of row0 at the lane's columns
+        rsrc_t rw, rr, rc;  // the unit's 16 x 256 patch of the weights, the running mean squares (RMSprop) and the codes
+        uint32_t w_lane;    // byte offset of the lane's columns inside a row of those patches (column 0 for idle lanes)
     };
     auto locate = [&](int64_t unit) -> UnitPos {
         UnitPos p;
@@ -410,9 +431,11 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
         p.live = n < N;
         const int64_t nc = p.live ? n : 0;
         p.lane_off = (uint32_t)(nc * (int64_t)sizeof(float));
-        p.wp = kMode >= 3 ? w + p.row0 * ldw + nc : nullptr;
-        p.rp2 = kMode == 4 ? rms + p.row0 * ldw + nc : nullptr;
-        p.cp = kMode >= 2 ? codes + p.row0 * N + nc : nullptr;
+        const int64_t c0 = (int64_t)cb * 256, cols_here = N - c0 < 256 ? N - c0 : 256;
+        p.w_lane = p.live ? (uint32_t)(4 * lane) : 0u;
+        if (kMode >= 3) p.rw = row_rsrc(w + p.row0 * ldw + c0, (uint32_t)(((p.rows - 1) * ldw + cols_here) * (int64_t)sizeof(float)));
+        if (kMode == 4) p.rr = row_rsrc(rms + p.row0 * ldw + c0, (uint32_t)(((p.rows - 1) * ldw + cols_here) * (int64_t)sizeof(float)));
+        if (kMode >= 2) p.rc = row_rsrc(codes + p.row0 * N + c0, (uint32_t)((p.rows - 1) * N + cols_here));
         return p;
     };
     struct Ready {  // block metadata with what every request needs precomputed
@@ -437,14 +460,15 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
             // a request beyond the row's nonzeros (or the cached 64) is still issued, so that the number of
             // loads per row is fixed, but all lanes then read the first 16 bytes of B: one cache line
             const bool real = q0 + s2 < qend;
-            const uint32_t off = real ? (uint32_t)__builtin_amdgcn_readlane((int)m.row_off, (q0 + s2) & 63) + lane_off : 0u;
-            dst[s2] = *reinterpret_cast<const f32x4 *>(Bbytes + off);
+            const uint32_t row = (uint32_t)__builtin_amdgcn_readlane((int)m.row_off, (q0 + s2) & 63);
+            dst[s2] = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(rb, real ? lane_off : 0u, real ? row : 0u, 0));
         }
     };
     auto request_w = [&](const UnitPos &p, int u, f32x4 &dst, f32x4 &dst2) {
         const int uu = u < p.rows ? u : p.rows - 1;
-        dst = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.wp + (int64_t)uu * ldw));
-        if (kMode == 4) dst2 = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.rp2 + (int64_t)uu * ldw));
+        const uint32_t row = (uint32_t)uu * w_row_bytes;
+        dst = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(p.rw, 4u * p.w_lane, row, kRowAuxNt));
+        if (kMode == 4) dst2 = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(p.rr, 4u * p.w_lane, row, kRowAuxNt));
     };
 
     f32x4 b[kBRing][kFixed];
@@ -517,8 +541,8 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
                 } else {
                     const uint32_t c0 = encode(acc.x), c1 = encode(acc.y), c2 = encode(acc.z), c3 = encode(acc.w);
                     if (pos.live)
-                        __builtin_nontemporal_store(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24),
-                                                    reinterpret_cast<uint32_t *>(pos.cp + (int64_t)u * N));
+                        __builtin_amdgcn_raw_buffer_store_b32(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24), pos.rc, pos.w_lane,
+                                                              (uint32_t)u * (uint32_t)N, kRowAuxNt);
                     if (kMode == 4) {  // kRMSprop_with_weight_update on the decoded gradient, operation by operation
                         f32x4 wv = wr[u % kWRing], rv = rr[u % kWRing];
                         const float g[4] = {dlut[c0], dlut[c1], dlut[c2], dlut[c3]};
@@ -530,8 +554,8 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
                             wv[e] = wv[e] - step;
                         }
                         if (pos.live) {
-                            __builtin_nontemporal_store(rv, reinterpret_cast<f32x4 *>(pos.rp2 + (int64_t)u * ldw));
-                            __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(pos.wp + (int64_t)u * ldw));
+                            __builtin_amdgcn_raw_buffer_store_b128(as_u32x4(rv), pos.rr, 4u * pos.w_lane, (uint32_t)u * w_row_bytes, kRowAuxNt);
+                            __builtin_amdgcn_raw_buffer_store_b128(as_u32x4(wv), pos.rw, 4u * pos.w_lane, (uint32_t)u * w_row_bytes, kRowAuxNt);
                         }
                     }
                     if (kMode == 3) {
@@ -540,7 +564,8 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
                         wv.y = wv.y + dlut[c1];
                         wv.z = wv.z + dlut[c2];
                         wv.w = wv.w + dlut[c3];
-                        if (pos.live) __builtin_nontemporal_store(wv, reinterpret_cast<f32x4 *>(pos.wp + (int64_t)u * ldw));
+                        if (pos.live)
+                            __builtin_amdgcn_raw_buffer_store_b128(as_u32x4(wv), pos.rw, 4u * pos.w_lane, (uint32_t)u * w_row_bytes, kRowAuxNt);
                     }
                 }
             }
@@ -1042,7 +1067,8 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
         if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
         hipLaunchKernelGGL(csr_rows_kernel<1>, dim3((unsigned)grid), dim3(kRowThreads), 0, st, R, N, row_ptr, col_idx, vals, B, ldb,
                            cblocks, amax, (const float *)nullptr, (uint8_t *)nullptr, (float *)nullptr, (int64_t)0, 0.0f,
-                           (float *)nullptr, 0.0f, (const XStep *)nullptr, 0, (const float *)nullptr);
+                           (float *)nullptr, 0.0f, (const XStep *)nullptr, 0, (const float *)nullptr,
+                           (uint32_t)(((Cc - 1) * ldb + N) * (int64_t)sizeof(float)));
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
@@ -1165,7 +1191,7 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
         auto kernel = rms ? csr_rows_kernel<4> : (w ? csr_rows_kernel<3> : csr_rows_kernel<2>);
         hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), lds, st, R, N, row_ptr, col_idx, vals, B, ldb, col_blocks,
                            (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, rms, rate, ctx->xsteps, ctx->xstep_count,
-                           ctx->table);
+                           ctx->table, (uint32_t)(((Cc - 1) * ldb + N) * (int64_t)sizeof(float)));
     } else {
         const int64_t col_blocks = (N + 1023) / 1024;
         int64_t row_groups = ((int64_t)ctx->num_cu * 3 + col_blocks - 1) / col_blocks;
