@@ -402,3 +402,33 @@ def test_kernels_that_draw_tiles_replay_from_a_graph(dev, codec_form):
         again = w0.clone()
         L.sgd_update(again, x, 0.5)
         assert torch.equal(again.view(torch.int32), want_w.view(torch.int32))
+
+
+def test_kernels_that_draw_tiles_may_overlap_on_two_streams(dev, codec_form):
+    """Launches take the library's ticket counters in turn, so two compressions beyond the cache issued on two streams
+    (default priority) may run at the same time without drawing each other's tiles: both must give the codes of a
+    compression that ran alone, over several rounds."""
+    if codec_form != "literal_for_small_tensors":
+        pytest.skip("one run is enough")
+    import torch
+    import clusternet_amd as cn
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(33)
+    n = (1 << 26) + 12345 * 4
+    xs = [torch.randn(n, device=dev, generator=gen) * 0.02 for _ in range(2)]
+    want = [cn.compression_8bit(x, 0.09) for x in xs]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [torch.zeros(n, dtype=torch.uint8, device=dev) for _ in range(2)]
+    torch.cuda.synchronize()
+    for _ in range(4):
+        for o in outs:
+            o.zero_()
+        torch.cuda.synchronize()
+        for s, x, o in zip(streams, xs, outs):
+            with torch.cuda.stream(s):
+                cn.compression_8bit(x, 0.09, out=o)
+        torch.cuda.synchronize()
+        for o, w in zip(outs, want):
+            assert torch.equal(o, w)
+    assert L.lib().cn_host_tile_counters_in_use() == 0
