@@ -623,6 +623,16 @@ def softmax(A, out=None):
     return out
 
 
+def fill(t, value):
+    """t[:] = value on a contiguous fp32 device tensor (the reference's zeros / ones / fill)."""
+    import torch
+    _need(t, torch.float32, "t")
+    if not t.is_contiguous():
+        raise ValueError("t must be contiguous")
+    check(lib().cn_fill_f32(t.data_ptr(), float(value), t.numel(), _stream()))
+    return t
+
+
 def sub(a, b, out=None):
     import torch
     L = _declare_layers(lib())

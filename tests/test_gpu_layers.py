@@ -407,3 +407,20 @@ def test_maxout_training_step_full_size_properties(dev):
     rel = ((dec - g1).abs() / pv)[keep]
     assert float(rel.max()) <= 0.0172 + 1e-6
     assert torch.equal(torch.sign(dec[keep]), torch.sign(g1[keep]))
+
+
+def test_fill_on_every_path(dev):
+    """cn_fill_f32 (zeros / ones of the reference): the element loop, a workgroup per tile and the form that draws its
+    tiles; sizes round the tile borders, n % 4 tails, a start that is not 16-byte aligned, nothing written outside."""
+    import torch
+    from clusternet_amd import _lib as L
+    for n in (1, 3, 5, 4097, (1 << 20) + 7, (1 << 22) + 32768 + 3, (1 << 26) + 5 * 32768 + 2):
+        for off in (0, 1, 4):
+            buf = torch.full((n + 16,), 7.0, device=dev)
+            L.fill(buf[4 + off:4 + off + n], -0.375)
+            assert float(buf[:4 + off].min()) == 7.0 and float(buf[:4 + off].max()) == 7.0, (n, off)
+            assert float(buf[4 + off + n:].min()) == 7.0 and float(buf[4 + off + n:].max()) == 7.0, (n, off)
+            got = buf[4 + off:4 + off + n]
+            assert float(got.min()) == -0.375 and float(got.max()) == -0.375, (n, off)
+            del buf
+    assert L.lib().cn_host_tile_counters_in_use() == 0
