@@ -10,12 +10,58 @@
 namespace cn {
 
 constexpr int kT = 256;
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 static inline int grid_for(const Context *ctx, int64_t work_items, int per_cu = 8) {
     int64_t blocks = (work_items + kT - 1) / kT;
     int64_t cap = (int64_t)ctx->num_cu * per_cu;
     if (blocks > cap) blocks = cap;
     return (int)(blocks < 1 ? 1 : blocks);
+}
+
+// out[c][r] = in[r][c] on 64 x 64 tiles through LDS, a workgroup per tile.  Whole tiles of 16-byte aligned matrices move as
+// 16-byte vectors on both sides (256 contiguous bytes per tile row); the tiles are numbered down the columns of `in`, so
+// that workgroups started one after the other write neighbouring pieces of the same 64 rows of `out`: the stream that
+// writes is the one that needs its window narrow.  4.3 TB/s became 5.3 TB/s on a 100000 x 8192 matrix and 4.2 became
+// 5.7 on 20000 x 40000.
+template <bool kVector>
+__global__ __launch_bounds__(kT) void transpose64_kernel(const float *__restrict__ in, int64_t rows, int64_t cols,
+                                                         float *__restrict__ out, int64_t tiles_r) {
+    __shared__ float tile[64][65];
+    const int64_t tc = blockIdx.x / tiles_r, tr = blockIdx.x % tiles_r;
+    const int64_t r0 = tr * 64, c0 = tc * 64;
+    if (kVector && r0 + 64 <= rows && c0 + 64 <= cols) {
+        const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;  // 16 vectors across, 16 rows down, four passes
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = ty + 16 * j;
+            const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(in + (r0 + r) * cols + c0 + 4 * tx));
+            tile[r][4 * tx + 0] = v.x;
+            tile[r][4 * tx + 1] = v.y;
+            tile[r][4 * tx + 2] = v.z;
+            tile[r][4 * tx + 3] = v.w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = ty + 16 * j;
+            const f32x4_t o = {tile[4 * tx + 0][c], tile[4 * tx + 1][c], tile[4 * tx + 2][c], tile[4 * tx + 3][c]};
+            __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t *>(out + (c0 + c) * rows + r0 + 4 * tx));
+        }
+    } else {
+        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 across, 4 down, sixteen passes
+#pragma unroll 4
+        for (int j = 0; j < 64; j += 4) {
+            const int64_t r = r0 + ty + j, c = c0 + tx;
+            if (r < rows && c < cols) tile[ty + j][tx] = in[r * cols + c];
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int j = 0; j < 64; j += 4) {
+            const int64_t c = c0 + ty + j, r = r0 + tx;
+            if (r < rows && c < cols) out[c * rows + r] = tile[tx][ty + j];
+        }
+    }
 }
 
 // out[c][r] = in[r][c]; 32 x 32 tiles through LDS (33-float pitch), both sides coalesced.
@@ -47,7 +93,6 @@ __global__ __launch_bounds__(kT) void transpose_kernel(const float *__restrict__
 // draws its tiles from a counter (the weight update on 819.2 M elements: 6.7 TB/s drawn, 6.1 TB/s with a workgroup per
 // tile, 5.5 TB/s on a persistent grid-stride grid).  Otherwise, and for the last n % 4 elements, element by element.
 // Each f is the single fp32 expression of its reference routine.
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
 struct AffineOp { float mul, add; __device__ float operator()(float x, float) const { return x * mul + add; } };
 struct AbsOp { __device__ float operator()(float x, float) const { return fabsf(x); } };
 struct SubOp { __device__ float operator()(float a, float b) const { return a - b; } };
@@ -288,6 +333,16 @@ cn_status cn_transpose_f32(const float *in, int64_t rows, int64_t cols, float *o
     CN_REQUIRE(in && out, CN_ERR_NULL, "transpose_f32: NULL pointer");
     CN_REQUIRE(in != out, CN_ERR_ARG, "transpose_f32: in-place transpose is not supported");
     CN_ENTER();
+    const int64_t tiles_r = (rows + 63) / 64, tiles64 = tiles_r * ((cols + 63) / 64);
+    auto ok16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    if (tiles64 <= 0x7fffffffLL && rows * cols >= (1 << 16)) {
+        if (ok16(in) && ok16(out) && rows % 4 == 0 && cols % 4 == 0)
+            hipLaunchKernelGGL(transpose64_kernel<true>, dim3((unsigned)tiles64), dim3(kT), 0, st, in, rows, cols, out, tiles_r);
+        else
+            hipLaunchKernelGGL(transpose64_kernel<false>, dim3((unsigned)tiles64), dim3(kT), 0, st, in, rows, cols, out, tiles_r);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    }
     int64_t tiles = ((rows + 31) / 32) * ((cols + 31) / 32);
     int64_t cap = (int64_t)ctx->num_cu * 8;
     hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(kT), 0, st, in, rows, cols, out);

@@ -424,3 +424,22 @@ def test_fill_on_every_path(dev):
             assert float(got.min()) == -0.375 and float(got.max()) == -0.375, (n, off)
             del buf
     assert L.lib().cn_host_tile_counters_in_use() == 0
+
+
+def test_transpose_on_every_path(dev):
+    """cn_transpose_f32: small matrices (32 x 32 tiles), whole and ragged 64 x 64 tiles, dimensions that are not
+    multiples of four and starts that are not 16-byte aligned (element-wise tiles), against torch's transposition."""
+    import torch
+    from clusternet_amd import _lib as L
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(17)
+    for r, c in ((1, 1), (3, 5), (63, 65), (64, 64), (128, 784), (1000, 1003), (260, 516), (4096, 4100), (516, 260),
+                 (1024, 4096), (8192, 384)):
+        for off in (0, 1, 4):
+            buf = torch.randn(r * c + 8, device=dev, generator=gen)
+            A = buf[off:off + r * c].view(r, c)
+            obuf = torch.full((r * c + 8,), 7.0, device=dev)
+            out = obuf[off:off + r * c].view(c, r)
+            L.transpose(A, out)
+            assert torch.equal(out, A.t()), (r, c, off)
+            assert float(obuf[:off].sum()) == 7.0 * off and float(obuf[off + r * c:].min()) == 7.0, (r, c, off)
