@@ -169,16 +169,18 @@ def bench_codec(torch, cn, dev):
                             torch, lambda: (cn.absmax(x, prec_t), cn.compression_8bit(x, prec_t, codes)), 20, 50),
                         "absmax_compress_one_call_us": time_replayed(
                             torch, lambda: cn.absmax_compression_8bit(x, codes, prec_t), 20, 50)}
-            cn.lib().cn_host_absmax_compress_single_launch(1)
-            replayed["absmax_compress_single_launch_us"] = time_replayed(
-                torch, lambda: cn.absmax_compression_8bit(x, codes, prec_t), 20, 50)
-            cn.lib().cn_host_absmax_compress_single_launch(0)
-            if n <= (3 << 20):
-                # tensors this small are encoded element by element; the per-call table beside it
-                cn.lib().cn_host_codec_literal_upto(0)
-                replayed["compress_with_table_us"] = time_replayed(
-                    torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50)
-                cn.lib().cn_host_codec_literal_upto(2 ** 64 - 1)
+            # the one call pinned to each of its two forms (it picks by size)
+            for label, mode in (("absmax_compress_two_kernels_us", 0), ("absmax_compress_single_launch_us", 1)):
+                cn.lib().cn_host_absmax_compress_single_launch(mode)
+                replayed[label] = time_replayed(torch, lambda: cn.absmax_compression_8bit(x, codes, prec_t), 20, 50)
+            cn.lib().cn_host_absmax_compress_single_launch(-1)
+            # the other encoders beside the one the library picks for this size (same bits)
+            for label, which in (("compress_literal_us", 1), ("compress_table_on_quotient_us", 2), ("compress_own_table_us", 3)):
+                if which == 1 and n > (8 << 20):
+                    continue
+                cn.lib().cn_host_codec_encoder(which)
+                replayed[label] = time_replayed(torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50)
+                cn.lib().cn_host_codec_encoder(0)
             res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
         if n >= 100000 * 8192:
             # movers that are not this library's: the runtime's device-to-device copy (above) and its fill, the latter a

@@ -85,8 +85,10 @@ def lib():
     L.cn_host_gemm_epilogue_in_kernel.restype = None
     L.cn_host_gemm_wide_store.argtypes = [C.c_int]
     L.cn_host_gemm_wide_store.restype = None
-    L.cn_host_codec_literal_upto.argtypes = [C.c_size_t]
-    L.cn_host_codec_literal_upto.restype = None
+    L.cn_host_codec_encoder.argtypes = [C.c_int]
+    L.cn_host_codec_encoder.restype = None
+    L.cn_host_quotient_mismatches.argtypes = [C.c_float, C.c_uint32, C.c_ulonglong]
+    L.cn_host_quotient_mismatches.restype = C.c_longlong
     L.cn_host_gemm_w8_rows.argtypes = [C.c_int]
     L.cn_host_gemm_w8_rows.restype = None
     L.cn_host_tile_counters_in_use.argtypes = []

@@ -8,11 +8,15 @@
 // What a stream that also writes reaches on this part depends sharply on the window of addresses in flight.
 // Decompression (mostly writes) runs a workgroup per 4096-element tile, as many workgroups as tiles, so that the
 // dispatcher keeps the tiles in flight next to one another: 6.9 TB/s, against 6.1 TB/s for the best persistent grid.
-// Compression cannot start a workgroup per tile (its encoder table costs 9 000 cycles to build); large tensors take
-// compress_stream_kernel, one persistent workgroup per compute unit that draws its tiles in order from a counter, which
-// keeps the same narrow window (6.6 TB/s, against 6.4 TB/s on a grid-stride walk), addressed through a buffer
-// descriptor per tile (a uniform base and a 32-bit lane offset; the descriptor's range replaces the bounds test of
-// the last tile), read and written with the non-temporal hint.
+// Compression cannot start a workgroup per tile (a workgroup first needs its encoder table in LDS: 40 KB copied, or
+// built in 9 000 cycles); large tensors take compress_stream_kernel, one persistent workgroup per compute unit that
+// draws its tiles in order from a counter, which keeps the same narrow window (6.6 TB/s, against 6.4 TB/s on a
+// grid-stride walk), addressed through a buffer descriptor per tile (a uniform base and a 32-bit lane offset; the
+// descriptor's range replaces the bounds test of the last tile), read and written with the non-temporal hint.
+//
+// Three encoders give the same codes (compress_impl picks by size): the literal procedure element by element, the
+// fixed table on the quotient x / precision (cn_xlut.h, cn_encode_table.h) and the table built per call for the
+// call's precision (cn_encode_table.h).
 #include <type_traits>
 
 #include "cn_internal.h"
@@ -31,11 +35,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // kUpdate: besides the codes, y += alpha * (decoded value of each code), as decompress_axpy would add it
 // afterwards: the gradient's codes for the exchange and the own weight update in one pass over both arrays.
-template <bool kVector, bool kUpdate>
+template <bool kVector, bool kUpdate, bool kQuotient = false>
 __global__ __launch_bounds__(kThreads) void compress_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr,
     size_t n, uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count,
-    const float *__restrict__ table, float alpha, float *__restrict__ y) {
+    const float *__restrict__ table, float alpha, float *__restrict__ y, const XEntry *__restrict__ quotient_table = nullptr) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
     float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // kUpdate: decode table times alpha
@@ -62,9 +66,19 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
     auto load = [&](size_t tile, f32x4 (&v)[kVecPerThread], f32x4 (&w)[kUpdate ? kVecPerThread : 1]) {
         load_tile(tile, v, reinterpret_cast<f32x4 (&)[kVecPerThread]>(w));
     };
+    QuotientTableCopy<kThreads> copy;
+    if (kQuotient) copy.request(quotient_table);  // ahead of the tile: loads return in order
     if (kVector && blockIdx.x < tiles) load(blockIdx.x, va, wa);
 
-    const bool exact_only = !build_table(sh, steps, step_count, precision, table);
+    bool exact_only = false;
+    if (kQuotient) {
+        copy.store(sh.lut);
+        if (!kUpdate) __syncthreads();
+    } else {
+        exact_only = !build_table(sh, steps, step_count, precision, table);
+    }
+    const double scale = quotient_scale(precision);
+    const uint32_t first_of_one = xlut_first(1.0f);
     if (kUpdate) {
         const int t = threadIdx.x;
         if (t < 126) {
@@ -82,6 +96,7 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
     const uint32_t first = xlut_first(precision);
     auto encode = [&](float v) -> uint32_t {
         const uint32_t bits = __float_as_uint(v);
+        if (kQuotient) return encode_by_quotient(bits, scale, sh.lut, first_of_one);
         return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
     };
 
@@ -150,12 +165,12 @@ __global__ __launch_bounds__(kThreads) void compress_kernel(
 }
 
 // ---- the literal procedure for small tensors ---------------------------------------------------------------
-// A workgroup's table costs about 9 000 cycles before the first element is encoded; the literal procedure (division
-// and pivot search, encode_exact) costs about 70 instructions per element and needs only the 126-entry codebook.  A
-// tensor of a few hundred thousand elements spread over the whole chip is a handful of elements per lane, which
-// the literal procedure finishes before a table would exist.  Four elements per lane and step, evaluated level by
-// level so that the search's LDS reads overlap; same bits as the table by construction (the table is made of
-// evaluations of this procedure).
+// A workgroup's table is 40 KB to copy, or about 9 000 cycles to build, before the first element is encoded; the
+// literal procedure (division and pivot search, encode_exact) costs about 70 instructions per element and needs only
+// the 126-entry codebook.  A tensor of up to a few hundred thousand elements spread over the whole chip is a handful
+// of elements per lane, which the literal procedure finishes before a table would be there.  Four elements per lane
+// and step, evaluated level by level so that the search's LDS reads overlap; same bits as the tables by construction
+// (they are made of evaluations of this procedure).
 template <bool kVector, bool kUpdate>
 __global__ __launch_bounds__(kThreads) void compress_literal_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr, size_t n,
@@ -225,12 +240,13 @@ __device__ __forceinline__ rsrc_t tile_rsrc(const void *base, uint32_t bytes) {
 // together, then encoded and stored; the next tile's loads go out right behind the stores.  Two shapes: 1024 x 12
 // (192 KiB of input per tile), one workgroup per compute unit, tiles drawn in order from a counter (`queue`,
 // cn_tile_queue.h) for tensors that stream from HBM; 512 x 10 with two workgroups per compute unit on a grid-stride
-// walk (`queue` NULL) for tensors that the Infinity Cache can hold.
-template <int T, int U, bool kUpdate>
+// walk (`queue` NULL) below that.  kQuotient: the table on the quotient, copied from `quotient_table`, instead of a
+// table built for the precision.
+template <int T, int U, bool kUpdate, bool kQuotient = false>
 __global__ __launch_bounds__(T) void compress_stream_kernel(
     const float *__restrict__ x, float precision_value, const float *__restrict__ precision_ptr, size_t n,
     uint8_t *__restrict__ codes, const XStep *__restrict__ steps, int step_count, const float *__restrict__ table,
-    uint32_t *__restrict__ queue, float alpha, float *__restrict__ y) {
+    uint32_t *__restrict__ queue, float alpha, float *__restrict__ y, const XEntry *__restrict__ quotient_table = nullptr) {
     constexpr uint32_t kVecs = T * U;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
@@ -256,6 +272,8 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
     // tiles are drawn from a counter (cn_tile_queue.h); without one, a grid-stride walk
     TileQueue q = tile_queue(queue, (uint32_t)tiles, queue_slots);
     size_t tile = blockIdx.x;
+    QuotientTableCopy<T> copy;
+    if (kQuotient) copy.request(quotient_table);  // ahead of the tile: loads return in order
     if (queue) {
         q.draw_ahead();
         tile = q.next();
@@ -264,7 +282,15 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
         load(tile);  // on their way while the table is built
         if (queue) q.draw_ahead();
     }
-    const bool exact_only = !build_table(sh, steps, step_count, precision, table);
+    bool exact_only = false;
+    if (kQuotient) {
+        copy.store(sh.lut);
+        if (!kUpdate) __syncthreads();
+    } else {
+        exact_only = !build_table(sh, steps, step_count, precision, table);
+    }
+    const double scale = quotient_scale(precision);
+    const uint32_t first_of_one = xlut_first(1.0f);
     if (kUpdate) {
         if (tid < 126) {
             const float d = table[tid] * precision;
@@ -282,6 +308,7 @@ __global__ __launch_bounds__(T) void compress_stream_kernel(
     // `exact` is a type: the table look-up, or (where no table can be trusted) the literal procedure per element
     auto run = [&](auto exact) {
         auto encode = [&](uint32_t bits) -> uint32_t {
+            if (kQuotient) return encode_by_quotient(bits, scale, sh.lut, first_of_one);
             if (decltype(exact)::value) return encode_exact(__uint_as_float(bits), precision, sh.slot);
             return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
         };
@@ -439,6 +466,28 @@ __device__ __forceinline__ float max_unkey(uint32_t key) {
     return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
 }
 
+// One arrival at a ticket line: the 64-bit word at `line` holds the running maximum in its low half and the number of
+// arrivals in its high half.  The maximum is folded in with a 32-bit atomicMax on the low half, the arrival counted
+// with a 64-bit atomicAdd of 1 << 32 on the whole word, which leaves the low half as it is and returns both halves as
+// they were: whoever finds members - 1 earlier arrivals holds, in the low half of what its own count returned, the
+// maximum over all members (each member's fold comes before its count in the order of operations on that word, and
+// all the counts came before this one), without a further read.  Both atomics return a value and the count's
+// operand is made to depend on what the fold returned, so the fold has been performed before the count is issued;
+// `fenced` puts a release fence between the two and an acquire fence behind the count, the memory model's own form
+// for a pair of locations.  Returns true for the last arrival, with *all = the maximum; it then puts the word back to 0.
+__device__ __forceinline__ bool ticket_arrive(uint32_t *line, uint32_t value, uint32_t members, int fenced, uint32_t *all) {
+    const uint32_t before = atomicMax(line, value);
+    unsigned long long one = 1ull << 32;
+    asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
+    if (fenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    const unsigned long long seen = atomicAdd(reinterpret_cast<unsigned long long *>(line), one);
+    if ((uint32_t)(seen >> 32) != members - 1) return false;
+    if (fenced) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(line), 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *all = (uint32_t)seen;  // includes `value`: this lane's fold was performed before its count
+    return true;
+}
+
 template <bool kVector, bool kAbs>
 __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restrict__ x, size_t n,
                                                           float *__restrict__ out,
@@ -477,45 +526,24 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
             m = max(m, max_key<kAbs>(__float_as_uint(x[i])));
     }
     m = block_max(m, smem);
-    // Two-level ticket.  The workgroup folds its maximum into the running maximum of its group of eight with a
-    // device-scope atomicMax and counts itself in with an atomicAdd; the last of a group to arrive carries the
-    // group's maximum to the second level in the same way, and the last group there writes the result.  Every
-    // word is put back to 0 by whoever arrived last at it.  Both atomics return a value and the count is made
-    // to depend on what the fold returned, so the fold has been performed before the count is issued:
-    // ordering by data dependence instead of by fences, which cost far more here (a release fence per
-    // workgroup writes the L2 back; nothing in this kernel needs that).  Atomics on one word are performed one
-    // after the other, about 12 ns each, hence the groups: their words lie on lines of their own.
-    // The writer side therefore rests on a property of this part (a returning atomic has been performed at the
-    // device's coherence point before an instruction that consumes its result issues), not on the memory model;
-    // the reader side is model-correct: whoever arrives last issues an acquire fence at agent scope before it
-    // reads.  `fenced` (cn_host_reduction_fences) switches the writer to the model's own form, a release fence
-    // between the fold and the count; the tests hold the two forms to the same bits.
+    // Two-level ticket (ticket_arrive): the workgroup arrives at the line of its group of eight; the last of a group
+    // carries the group's maximum to the line of the groups, and the last group writes the result.  Atomics on one
+    // word are performed one after the other, about 12 ns each, hence the groups: their words lie on lines of their
+    // own.  Ordering by data dependence instead of by fences costs far less here (a release fence per workgroup
+    // writes the L2 back; nothing in this kernel needs that) and rests on a property of this part: a returning
+    // atomic has been performed at the device's coherence point before an instruction that consumes its result
+    // issues.  `fenced` (cn_host_reduction_fences) switches to the memory model's own form; the tests hold the two
+    // forms to the same bits.  A grid of one workgroup, or of one group, skips what it does not need.
     if (threadIdx.x == 0) {
         const uint32_t groups = (gridDim.x + kTicketGroup - 1) / kTicketGroup;
         const uint32_t group = blockIdx.x / kTicketGroup;
         const uint32_t left = gridDim.x - group * kTicketGroup;
         const uint32_t members = left < (uint32_t)kTicketGroup ? left : (uint32_t)kTicketGroup;
-        uint32_t *first = tickets + (1 + group) * kTicketStride, *second = tickets;
-        auto fold_and_count = [fenced](uint32_t *line, uint32_t value) -> uint32_t {
-            const uint32_t before = atomicMax(line, value);
-            uint32_t one = 1u;
-            asm volatile("" : "+v"(one) : "v"(before));  // `one` is not available before `before` is
-            if (fenced) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            return atomicAdd(line + 1, one);
-        };
-        auto take = [](uint32_t *line, uint32_t ticket) -> uint32_t {
-            asm volatile("" : "+v"(line) : "v"(ticket));  // the read is not issued before the ticket is known
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-            const uint32_t v = __hip_atomic_load(line, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(line, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(line + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            return v;
-        };
-        const uint32_t ticket = fold_and_count(first, m);
-        if (ticket == members - 1) {
-            const uint32_t of_group = take(first, ticket);
-            const uint32_t ticket2 = fold_and_count(second, of_group);
-            if (ticket2 == groups - 1) out[0] = max_unkey<kAbs>(take(second, ticket2));
+        uint32_t all = m;
+        if (gridDim.x == 1) {
+            out[0] = max_unkey<kAbs>(all);
+        } else if (ticket_arrive(tickets + (1 + group) * kTicketStride, m, members, fenced, &all)) {
+            if (groups == 1 || ticket_arrive(tickets, all, groups, fenced, &all)) out[0] = max_unkey<kAbs>(all);
         }
     }
 }
@@ -524,8 +552,9 @@ __global__ __launch_bounds__(kThreads) void absmax_kernel(const float *__restric
 // Phase 1: every workgroup folds the maximum of its tiles into the two-level ticket of absmax_kernel (same words,
 // same ordering; kernels of one stream do not overlap).  Whoever arrives last of all holds the maximum and
 // publishes it, together with the number of this call, in a word of every group's line; every workgroup waits
-// for that word on its own group's line (eight readers per line) and goes on to phase 2: the table for that
-// maximum and the codes of the same tiles, whose second read comes from the caches for tensors they can hold.
+// for that word on its own group's line (eight readers per line) and goes on to phase 2: the codes of the same
+// tiles under that maximum (the encoder's table is the one on the quotient, which does not depend on the precision
+// and is copied into LDS before the first phase), whose second read comes from the caches for tensors they can hold.
 // The grid is sized to be resident as a whole, so the wait ends; it is bounded all the same: a workgroup that
 // gives up (part of the grid not resident because another kernel holds compute units) takes the maximum over the
 // whole tensor by itself, slow and still exact, and every workgroup ends either way.
@@ -536,10 +565,11 @@ constexpr int kResultWord = 8;  // in a group's line (64-bit): call number << 32
 
 __global__ __launch_bounds__(kThreads) void absmax_compress_kernel(
     const float *__restrict__ x, size_t n, uint8_t *__restrict__ codes, float *__restrict__ precision_out,
-    const XStep *__restrict__ steps, int step_count, const float *__restrict__ table, uint32_t *__restrict__ tickets,
-    uint32_t spin_limit) {
+    uint32_t *__restrict__ tickets, uint32_t spin_limit, const XEntry *__restrict__ quotient_table) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
+    XEntry *lut = reinterpret_cast<XEntry *>(smem_raw);  // kXEntries entries
+    QuotientTableCopy<kThreads> copy;
+    copy.request(quotient_table);  // ahead of the tiles: loads return in order
     __shared__ uint32_t red[kThreads / 64];
     __shared__ uint32_t s_key, s_complete;
     const size_t nvec = n / 4;
@@ -579,10 +609,10 @@ __global__ __launch_bounds__(kThreads) void absmax_compress_kernel(
     u32x4 kept[kKeep][kVecPerThread];
     uint32_t own = 0;
 #pragma unroll
-    for (int k = 0; k < kKeep; ++k) {
-        load_tile(blockIdx.x + (size_t)k * gridDim.x, kept[k]);
-        own = fold(own, kept[k]);
-    }
+    for (int k = 0; k < kKeep; ++k) load_tile(blockIdx.x + (size_t)k * gridDim.x, kept[k]);
+    copy.store(lut);  // published by the barriers of the first phase
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) own = fold(own, kept[k]);
     own = max(own, tile_max(blockIdx.x + (size_t)kKeep * gridDim.x, gridDim.x));
     if (blockIdx.x == 0) {
         const size_t i = nvec * 4 + threadIdx.x;
@@ -593,34 +623,17 @@ __global__ __launch_bounds__(kThreads) void absmax_compress_kernel(
         const uint32_t left = gridDim.x - group * kTicketGroup;
         const uint32_t members = left < (uint32_t)kTicketGroup ? left : (uint32_t)kTicketGroup;
         uint32_t *first = tickets + (1 + group) * kTicketStride, *second = tickets;
-        auto fold_and_count = [](uint32_t *line, uint32_t value) -> uint32_t {
-            const uint32_t before = atomicMax(line, value);
-            uint32_t one = 1u;
-            asm volatile("" : "+v"(one) : "v"(before));  // the count is not issued before the fold has been performed
-            return atomicAdd(line + 1, one);
-        };
-        auto take = [](uint32_t *line, uint32_t ticket) -> uint32_t {
-            asm volatile("" : "+v"(line) : "v"(ticket));
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-            const uint32_t v = __hip_atomic_load(line, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(line, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(line + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            return v;
-        };
-        const uint32_t ticket = fold_and_count(first, m);
-        if (ticket == members - 1) {
-            const uint32_t of_group = take(first, ticket);
-            const uint32_t ticket2 = fold_and_count(second, of_group);
-            if (ticket2 == groups - 1) {
-                // everyone has arrived, hence read the call number: publish, then advance it
-                const uint32_t key = take(second, ticket2);
-                const unsigned long long word = ((unsigned long long)call << 32) | key;
-                for (uint32_t g = 0; g < groups; ++g)
-                    __hip_atomic_store(reinterpret_cast<unsigned long long *>(tickets + (1 + g) * kTicketStride + kResultWord), word,
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(&tickets[kCallWord], call, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                precision_out[0] = __uint_as_float(key);
-            }
+        uint32_t key = m;
+        // a grid of one workgroup still publishes: the wait below is the same for every grid
+        if ((gridDim.x == 1 || ticket_arrive(first, m, members, 0, &key)) &&
+            (groups == 1 || ticket_arrive(second, key, groups, 0, &key))) {
+            // everyone has arrived, hence read the call number: publish, then advance it
+            const unsigned long long word = ((unsigned long long)call << 32) | key;
+            for (uint32_t g = 0; g < groups; ++g)
+                __hip_atomic_store(reinterpret_cast<unsigned long long *>(tickets + (1 + g) * kTicketStride + kResultWord), word,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&tickets[kCallWord], call, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            precision_out[0] = __uint_as_float(key);
         }
         const unsigned long long *mine = reinterpret_cast<const unsigned long long *>(first + kResultWord);
         unsigned long long seen = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -646,12 +659,9 @@ __global__ __launch_bounds__(kThreads) void absmax_compress_kernel(
         key = s_key;
     }
     const float precision = __uint_as_float(key);
-    const bool exact_only = !build_table(sh, steps, step_count, precision, table);
-    const uint32_t first = xlut_first(precision);
-    auto encode = [&](uint32_t bits) -> uint32_t {
-        if (exact_only) return encode_exact(__uint_as_float(bits), precision, sh.slot);
-        return xlut_code(bits, sh.lut[xlut_index(bits & 0x7fffffffu, first)]);
-    };
+    const double scale = quotient_scale(precision);
+    const uint32_t first_of_one = xlut_first(1.0f);
+    auto encode = [&](uint32_t bits) -> uint32_t { return encode_by_quotient(bits, scale, lut, first_of_one); };
     uint32_t *c4 = reinterpret_cast<uint32_t *>(codes);
     auto encode_tile = [&](size_t tile, const u32x4 (&v)[kVecPerThread]) {
         const size_t base = tile * kTileVec + threadIdx.x;
@@ -705,20 +715,48 @@ __global__ __launch_bounds__(kLanes) void fill_tiles_kernel(float *__restrict__ 
     }
 }
 
+// Test kernel: over `count` consecutive bit patterns of x from `first`, how often the quotient the table encoder forms
+// ((float)((double)x * (1.0 / (double)p)), cn_encode_table.h) differs from the division x / p.  Two NaNs count as equal, and
+// so do two results below the normal range (every such quotient has the code 254).
+__global__ __launch_bounds__(256) void quotient_check_kernel(uint32_t first, unsigned long long count, float p,
+                                                             unsigned long long *__restrict__ mismatches) {
+    const double scale = quotient_scale(p);
+    unsigned long long bad = 0;
+    for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < count;
+         i += (unsigned long long)gridDim.x * blockDim.x) {
+        const float x = __uint_as_float(first + (uint32_t)i);
+        const uint32_t by_division = __float_as_uint(x / p);
+        const uint32_t by_product = __float_as_uint((float)((double)x * scale));
+        const uint32_t ma = by_division & 0x7fffffffu, mb = by_product & 0x7fffffffu;
+        const bool both_nan = ma > 0x7f800000u && mb > 0x7f800000u;
+        const bool both_tiny = ma < 0x00800000u && mb < 0x00800000u;
+        if (by_division != by_product && !both_nan && !both_tiny) ++bad;
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
 static inline bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
 static int g_workgroups_per_cu = 0;  // tuning hook: nonzero overrides every kernel's own figure (and keeps the tile kernels)
-// Tensors of at least this many elements take the streaming forms: enough tiles for every compute unit to have
-// several, so that the uneven last round does not show.
-constexpr size_t kStreamFrom = (size_t)1 << 24;
-// Tensors of at least this many elements (256 MiB of fp32) do not fit the 256 MB Infinity Cache.
-constexpr size_t kBeyondCacheFrom = (size_t)1 << 26;
 
-// Tensors of at most this many elements are encoded by the literal procedure, without a table.  Measured, replayed
-// from a graph: 2.9 us against 5.7 us up to 2^18 elements, 4.1 against 5.9 at 2^20, 5.6 against 7.3 at 2^21, 10.7
-// against 9.9 at 5.12 M; the two cross near 4 M.  Tuning hook: cn_host_codec_literal_upto.
-constexpr size_t kLiteralUpto = (size_t)3 << 20;
-static size_t g_literal_upto = kLiteralUpto;
+// Which encoder a compression takes.  Three give the same bits:
+//  - the literal procedure, element by element (compress_literal_kernel): nothing to prepare, about 70 instructions and
+//    nine LDS reads per element; tensors of at most kLiteralUpto elements, which are a handful of elements per lane;
+//  - the table on the quotient (cn_encode_table.h): a 40 KB copy per workgroup, three more instructions per element;
+//  - the table for the call's precision (build_table): about 9 000 cycles per workgroup before the first element, the
+//    fewest instructions per element; tensors from kOwnTableFrom elements on, where those instructions show (819.2 M
+//    elements: 622 us against 638 us) and the build does not.
+// Measured, replayed from a graph, literal / quotient / own table: 2^18 elements 3.0 / 3.1 / 5.7 us; 2^20: 4.1 / 3.4 /
+// 5.9; 5.12 M: 10.7 / 6.2-7.0 / 9.1-9.7; 2^23: - / 8.2 / 12.4; 26.2 M: - / 21.7-23.0 / 22.5-24.4; 2^27: - / 117 / 117.
+constexpr size_t kLiteralUpto = (size_t)1 << 18;
+constexpr size_t kOwnTableFrom = (size_t)1 << 27;
+// Whole float4 groups from this many elements on take compress_stream_kernel (2^24 elements: 15.1 us on the tile
+// kernel, 17.0 us streamed; 26.2 M: 24.5 against 23.0), and tensors with their own table draw their tiles.
+constexpr size_t kStreamFrom = (size_t)20 << 20;
+// With the update the streamed form exists for tensors beyond the 256 MB Infinity Cache only (2^26 elements of fp32).
+constexpr size_t kBeyondCacheFrom = (size_t)1 << 26;
+enum Encoder { kBySize = 0, kLiteral = 1, kQuotientTable = 2, kOwnTable = 3 };
+static int g_encoder = kBySize;  // test hook (cn_host_codec_encoder): one encoder for every size
 
 static int stream_grid(const Context *ctx, size_t n, int per_cu) {
     size_t tiles = (n / 4 + kTileVec - 1) / kTileVec;
@@ -729,6 +767,12 @@ static int stream_grid(const Context *ctx, size_t n, int per_cu) {
     return (int)(g < 1 ? 1 : g);
 }
 
+template <typename Kernel>
+static cn_status with_table_space(Kernel kernel, int bytes) {
+    CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    return CN_OK;
+}
+
 static cn_status compress_impl(const char *who, const float *x, float precision, const float *precision_dev, size_t n,
                                uint8_t *codes, float alpha, float *y, void *stream) {
     if (n == 0) return CN_OK;
@@ -737,26 +781,32 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
-    // Three workgroups per CU, which is what the encode table's 43 KB of LDS lets a CU hold: the whole grid
-    // is resident at once.  Measured on 819.2 M elements: 677 us against 720 us with two and 802 us with
-    // four (a second, quarter-full round); mixed read/write streams run fastest on this part with few
-    // wavefronts in flight, and the kernel keeps its own next tile in flight to stay busy at that occupancy.
-    int grid = stream_grid(ctx, n, 3);
+    const int lds_all = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);  // with the update's decode table
     const int lds = (int)sizeof(EncodeShared) + (y ? 256 * (int)sizeof(float) : 0);
     static OncePerDevice configured;
     if (configured.first(ctx->device)) {
-        const int most = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<true, false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<false, false>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<true, true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
-        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_kernel<false, true>),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, most));
+        cn_status c = CN_OK;
+        if (c == CN_OK) c = with_table_space(&compress_kernel<true, false, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<false, false, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<true, true, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<false, true, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<true, false, true>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<false, false, true>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<true, true, true>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_kernel<false, true, true>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_stream_kernel<1024, 12, false, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_stream_kernel<1024, 12, false, true>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_stream_kernel<512, 10, false, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_stream_kernel<512, 10, false, true>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_stream_kernel<1024, 4, true, false>, lds_all);
+        if (c == CN_OK) c = with_table_space(&compress_stream_kernel<1024, 4, true, true>, lds_all);
+        if (c != CN_OK) return c;
     }
     const bool vec = aligned(x, 16) && aligned(codes, 4) && (!y || aligned(y, 16));
-    if (n <= g_literal_upto && g_workgroups_per_cu == 0) {
+    const bool tuned = g_workgroups_per_cu != 0;  // the tuning hook keeps the tile kernel and its grid
+    int encoder = g_encoder;
+    if (encoder == kBySize) encoder = (n <= kLiteralUpto && !tuned) ? kLiteral : n < kOwnTableFrom ? kQuotientTable : kOwnTable;
+    if (encoder == kLiteral) {
         const size_t items = vec ? (n + 3) / 4 : n;
         size_t wgs = (items + kThreads - 1) / kThreads;
         const size_t cap = (size_t)ctx->num_cu * 8;
@@ -768,43 +818,44 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
-    if (vec && n >= kStreamFrom && g_workgroups_per_cu == 0 && (!y || (n >= kBeyondCacheFrom && n < ((size_t)1 << 40)))) {
-        static OncePerDevice stream_configured;
-        if (stream_configured.first(ctx->device)) {
-            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<1024, 12, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
-            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<512, 10, false>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
-            const int with_decode_table = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
-            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&compress_stream_kernel<1024, 4, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, with_decode_table));
+    const bool q = encoder == kQuotientTable;
+    const bool beyond_cache = n >= kBeyondCacheFrom && n < ((size_t)1 << 40);
+    if (vec && n >= kStreamFrom && !tuned && (!y || beyond_cache)) {
+        // One workgroup of 1024 lanes per compute unit and tiles of 192 KiB drawn from the counter for tensors that
+        // stream from HBM (819.2 M elements: 620 us; 1024 x 8: 626 us, 1024 x 16: 640 us, 512 x 16: 686 us, and 639 us for
+        // 256 x 12 on a grid-stride walk; tiles of 48 KiB would draw tickets faster than one counter hands them out);
+        // two workgroups of 512 x 10 per compute unit on a grid-stride walk below that (2^27 elements: 117 us either
+        // way; 2^26: 59 us against 66 us drawn; 2^28: 239 us against 217 us drawn).
+        // With the update (x and y read, codes and y written): tiles of 1024 x 4 vectors of each array, drawn, 1.60 ms
+        // on 819.2 M elements (512 x 4: 1.59 to 1.61, 512 x 6: 1.63, 512 x 8: 1.65, 512 x 12: 1.69; the tile kernel on
+        // a resident grid-stride grid: 1.96 ms).
+        const bool drawn = n >= kOwnTableFrom && n < ((size_t)1 << 40);
+        auto launch = [&](auto kernel, int wgs, int lanes, uint32_t *queue) {
+            hipLaunchKernelGGL(kernel, dim3(wgs), dim3(lanes), lds, st, x, precision, precision_dev, n, codes, ctx->xsteps,
+                               ctx->xstep_count, ctx->table, queue, alpha, y, ctx->quotient_table);
+        };
+        if (y) {
+            if (q) launch(&compress_stream_kernel<1024, 4, true, true>, ctx->num_cu, 1024, ctx->next_tile_counter());
+            else   launch(&compress_stream_kernel<1024, 4, true, false>, ctx->num_cu, 1024, ctx->next_tile_counter());
+        } else if (drawn) {
+            if (q) launch(&compress_stream_kernel<1024, 12, false, true>, ctx->num_cu, 1024, ctx->next_tile_counter());
+            else   launch(&compress_stream_kernel<1024, 12, false, false>, ctx->num_cu, 1024, ctx->next_tile_counter());
+        } else {
+            if (q) launch(&compress_stream_kernel<512, 10, false, true>, ctx->num_cu * 2, 512, nullptr);
+            else   launch(&compress_stream_kernel<512, 10, false, false>, ctx->num_cu * 2, 512, nullptr);
         }
-        // Beyond the cache: one workgroup of 1024 lanes per compute unit, tiles of 192 KiB drawn from the counter
-        // (measured on 819.2 M elements: 620 us; 1024 x 8: 626 us, 1024 x 16: 640 us, 512 x 16: 686 us, and 639 us
-        // for 256 x 12 on a grid-stride walk; tiles of 48 KiB would draw tickets faster than one counter hands them out).
-        // Tensors the cache can hold: two workgroups of 512 x 10 per compute unit on a grid-stride walk (26 M elements:
-        // 24.5 us against 32 to 34 us for the drawn forms).
-        // With the update (x and y read, codes and y written; beyond the cache only): tiles of 1024 x 4 vectors of each
-        // array, 1.60 ms on 819.2 M elements (512 x 4: 1.59 to 1.61, 512 x 6: 1.63, 512 x 8: 1.65, 512 x 12: 1.69; the
-        // tile kernel on a resident grid-stride grid: 1.96 ms).
-        if (y)
-            hipLaunchKernelGGL((compress_stream_kernel<1024, 4, true>), dim3(ctx->num_cu), dim3(1024), lds, st, x, precision,
-                               precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->next_tile_counter(), alpha, y);
-        else if (n >= kBeyondCacheFrom && n < ((size_t)1 << 40))
-            hipLaunchKernelGGL((compress_stream_kernel<1024, 12, false>), dim3(ctx->num_cu), dim3(1024), sizeof(EncodeShared), st, x,
-                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->next_tile_counter(),
-                               0.0f, (float *)nullptr);
-        else
-            hipLaunchKernelGGL((compress_stream_kernel<512, 10, false>), dim3(ctx->num_cu * 2), dim3(512), sizeof(EncodeShared), st, x,
-                               precision, precision_dev, n, codes, ctx->xsteps, ctx->xstep_count, ctx->table, (uint32_t *)nullptr,
-                               0.0f, (float *)nullptr);
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
-    auto kernel = y ? (vec ? compress_kernel<true, true> : compress_kernel<false, true>)
-                    : (vec ? compress_kernel<true, false> : compress_kernel<false, false>);
+    // Three workgroups per compute unit, which is what the table's LDS lets a compute unit hold: the whole grid is
+    // resident at once, and the kernel keeps its own next tile in flight to stay busy at that occupancy.
+    const int grid = stream_grid(ctx, n, 3);
+    auto kernel = q ? (y ? (vec ? compress_kernel<true, true, true> : compress_kernel<false, true, true>)
+                         : (vec ? compress_kernel<true, false, true> : compress_kernel<false, false, true>))
+                    : (y ? (vec ? compress_kernel<true, true, false> : compress_kernel<false, true, false>)
+                         : (vec ? compress_kernel<true, false, false> : compress_kernel<false, false, false>));
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, st, x, precision, precision_dev, n, codes, ctx->xsteps,
-                       ctx->xstep_count, ctx->table, alpha, y);
+                       ctx->xstep_count, ctx->table, alpha, y, ctx->quotient_table);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -840,7 +891,17 @@ using namespace cn;
 extern "C" {
 
 // Tuning hook: largest element count that compression encodes with the literal procedure instead of a table (0 = never, SIZE_MAX = the library's own threshold).
-void cn_host_codec_literal_upto(size_t n) { g_literal_upto = (n == (size_t)-1) ? kLiteralUpto : n; }
+long long cn_host_quotient_mismatches(float precision, uint32_t first_pattern, unsigned long long patterns) {
+    Context *ctx;
+    if (current_context(&ctx) != CN_OK) return -1;
+    unsigned long long *count = reinterpret_cast<unsigned long long *>(ctx->sum_scratch);  // 8 KB of scratch, idle here
+    if (hipMemset(count, 0, sizeof(*count)) != hipSuccess) return -1;
+    hipLaunchKernelGGL(quotient_check_kernel, dim3(ctx->num_cu * 8), dim3(256), 0, (hipStream_t)0, first_pattern, patterns, precision, count);
+    unsigned long long host = 0;
+    if (hipMemcpy(&host, count, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess) return -1;
+    return (long long)host;
+}
+void cn_host_codec_encoder(int which) { g_encoder = (which >= kBySize && which <= kOwnTable) ? which : kBySize; }
 
 // Tuning hook: workgroups per compute unit for the codec and abs-max kernels, 0 = each kernel's own choice.
 void cn_host_codec_workgroups_per_cu(int per_cu) { g_workgroups_per_cu = per_cu > 0 ? per_cu : 0; }
@@ -904,12 +965,17 @@ cn_status cn_absmax_f32(const float *x, size_t n, float *out, void *stream) {
     return CN_OK;
 }
 
-static uint32_t g_absmax_compress_spins = 1u << 16;  // test hook: 0 makes every workgroup that has to wait give up at once
-// Measured on this part, the two stream-ordered kernels are faster than the single launch at every size (5.12 M
-// elements: 16.3 us against 17.1 us replayed from a graph; 40 960: 10.7 against 12.0; 26 M: 42 against 53): back to
-// back, a second launch costs next to nothing, while the wait inside the kernel is a chain of round trips to the
-// device's coherence point.  So the single launch is there, tested, and off unless asked for.
-static bool g_absmax_compress_single_launch = false;
+constexpr uint32_t kSpinLimit = 1u << 14;
+static uint32_t g_absmax_compress_spins = kSpinLimit;  // test hook: 0 makes every workgroup that has to wait give up at once
+// The single launch against the two stream-ordered kernels, replayed from a graph: 4 096 elements 4.3 us against 5.2;
+// 0.8 M: 7.6 against 7.7; 5.12 M: 10.8 against 12.3; 2^23: 14.6 against 16.1; 2^24: 31 against 26; 26 M: 45 against 40.
+// Up to 2^23 elements a workgroup's tiles stay in registers between the phases and the tensor is read once; beyond
+// that the second read and the wait across the grid (a chain of round trips to the device's coherence point) cost
+// more than a second launch, which is nearly free back to back.  (With a table that had to be built for the maximum
+// found, the single launch was slower at every size; its table now does not depend on the precision and is
+// in LDS before the wait.)
+constexpr size_t kSingleLaunchUpto = (size_t)1 << 23;
+static int g_absmax_compress_single_launch = -1;  // test hook: 0 never, 1 wherever it can run, -1 by size
 
 cn_status cn_absmax_compress_8bit(const float *x, size_t n, uint8_t *codes, float *precision_out, void *stream) {
     if (!precision_out) { set_error("absmax_compress_8bit: NULL output for the precision"); return CN_ERR_NULL; }
@@ -918,21 +984,23 @@ cn_status cn_absmax_compress_8bit(const float *x, size_t n, uint8_t *codes, floa
     cn_status s = current_context(&ctx);
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
-    // Unless the single launch is asked for (see above), and for inputs that are empty, too large for the caches to
-    // serve the second read or not aligned for 16-byte loads: the two kernels, one behind the other on the stream.
-    if (!g_absmax_compress_single_launch || n == 0 || n >= kBeyondCacheFrom || !aligned(x, 16) || !aligned(codes, 4)) {
+    // Inputs that are empty, not aligned for 16-byte loads or too large (see above; when asked for, up to what the
+    // caches can serve on the second read) take the two kernels, one behind the other on the stream.
+    const bool single = g_absmax_compress_single_launch < 0 ? n <= kSingleLaunchUpto : g_absmax_compress_single_launch != 0;
+    if (!single || n == 0 || n >= kBeyondCacheFrom || !aligned(x, 16) || !aligned(codes, 4)) {
         s = cn_absmax_f32(x, n, precision_out, stream);
         if (s != CN_OK || n == 0) return s;
         return cn_compress_8bit_dp(x, precision_out, n, codes, stream);
     }
+    constexpr int kTableBytes = kXEntries * (int)sizeof(XEntry);
     static int resident_per_cu[kMaxDevices] = {};
     int &per_cu = resident_per_cu[ctx->device];
     if (per_cu == 0) {
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&absmax_compress_kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(EncodeShared)));
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, kTableBytes));
         int blocks = 0;
         CN_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void *>(&absmax_compress_kernel),
-                                                            kThreads, sizeof(EncodeShared)));
+                                                            kThreads, kTableBytes));
         if (blocks < 1) { set_error("absmax_compress_8bit: the kernel does not fit a compute unit"); return CN_ERR_HIP; }
         per_cu = blocks > 2 ? 2 : blocks;
     }
@@ -940,15 +1008,15 @@ cn_status cn_absmax_compress_8bit(const float *x, size_t n, uint8_t *codes, floa
     size_t grid = (size_t)ctx->num_cu * per_cu;  // resident as a whole: the wait inside the kernel relies on it
     if (grid > tiles) grid = tiles;
     if (grid < 1) grid = 1;
-    hipLaunchKernelGGL(absmax_compress_kernel, dim3((unsigned)grid), dim3(kThreads), sizeof(EncodeShared), st, x, n, codes,
-                       precision_out, ctx->xsteps, ctx->xstep_count, ctx->table, ctx->tickets, g_absmax_compress_spins);
+    hipLaunchKernelGGL(absmax_compress_kernel, dim3((unsigned)grid), dim3(kThreads), kTableBytes, st, x, n, codes,
+                       precision_out, ctx->tickets, g_absmax_compress_spins, ctx->quotient_table);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
 
-void cn_host_absmax_compress_single_launch(int enabled) { g_absmax_compress_single_launch = enabled != 0; }
+void cn_host_absmax_compress_single_launch(int mode) { g_absmax_compress_single_launch = mode < 0 ? -1 : mode != 0; }
 
-void cn_host_absmax_compress_spin_limit(int spins) { g_absmax_compress_spins = spins < 0 ? (1u << 16) : (uint32_t)spins; }
+void cn_host_absmax_compress_spin_limit(int spins) { g_absmax_compress_spins = spins < 0 ? kSpinLimit : (uint32_t)spins; }
 
 cn_status cn_max_f32(const float *x, size_t n, float *out, void *stream) {
     if (!out) { set_error("max_f32: NULL output"); return CN_ERR_NULL; }

@@ -74,6 +74,24 @@ int cn_host_xlut_encode_many(float precision, const float *x, size_t n, uint8_t 
     return unusable ? 0 : 1;
 }
 
+// The encoder on the quotient as the device runs it: the table for precision 1 and the quotient formed as a
+// product in double precision.  Returns 1, or 0 if the table for precision 1 cannot be built.
+int cn_host_quotient_encode_many(float precision, const float *x, size_t n, uint8_t *codes) {
+    static std::vector<cn::XEntry> of_one;
+    static int usable = -1;
+    if (usable < 0) {
+        of_one.resize(cn::kXEntries);
+        uint32_t first = 0;
+        usable = cn_host_xlut_build(1.0f, of_one.data(), &first) == 0 ? 1 : 0;
+    }
+    if (!usable) return 0;
+    const uint32_t first_of_one = cn::xlut_first(1.0f);
+    const double scale = cn::xlut_quotient_scale(precision);
+    for (size_t i = 0; i < n; ++i)
+        codes[i] = (uint8_t)cn::xlut_code_by_quotient(cn::x_to_bits(x[i]), scale, of_one.data(), first_of_one);
+    return 1;
+}
+
 int cn_host_encode_exact(float x, float precision) {
     float slot[128];
     host_slot(slot);

@@ -150,4 +150,44 @@ __device__ __forceinline__ bool build_table(EncodeShared &sh, const XStep *__res
     return true;
 }
 
+// ---- the encoder on the quotient ---------------------------------------------------------------------
+// The table of cn_xlut.h for precision 1 is the code as a function of the quotient x / precision (see there); it is
+// built and verified once on the host at initialisation and kept in device memory.  A workgroup copies it into LDS
+// (kXEntries entries of 8 bytes) instead of building a table for the call's precision, and pays three instructions
+// per element for the quotient (conversion, fp64 product, conversion).
+constexpr int kQuotientTableVecs = kXEntries * (int)sizeof(XEntry) / 16;
+static_assert(kXEntries * sizeof(XEntry) % 16 == 0, "whole 16-byte vectors");
+
+typedef uint32_t qt_u32x4 __attribute__((ext_vector_type(4)));
+
+// Requests this thread's share of the table; `store_quotient_table` puts it into LDS.  Split so that the caller can issue
+// other loads in between; a barrier must follow the store.
+template <int kThreadsOfGroup>
+struct QuotientTableCopy {
+    static constexpr int kEach = (kQuotientTableVecs + kThreadsOfGroup - 1) / kThreadsOfGroup;
+    qt_u32x4 part[kEach];
+    __device__ __forceinline__ void request(const XEntry *__restrict__ table_in_memory) {
+        const qt_u32x4 *src = reinterpret_cast<const qt_u32x4 *>(table_in_memory);
+#pragma unroll
+        for (int j = 0; j < kEach; ++j) {
+            const int at = j * kThreadsOfGroup + (int)threadIdx.x;
+            part[j] = src[at < kQuotientTableVecs ? at : kQuotientTableVecs - 1];
+        }
+    }
+    __device__ __forceinline__ void store(XEntry *lut) {
+        qt_u32x4 *dst = reinterpret_cast<qt_u32x4 *>(lut);
+#pragma unroll
+        for (int j = 0; j < kEach; ++j) {
+            const int at = j * kThreadsOfGroup + (int)threadIdx.x;
+            if (at < kQuotientTableVecs) dst[at] = part[j];
+        }
+    }
+};
+
+__device__ __forceinline__ double quotient_scale(float precision) { return xlut_quotient_scale(precision); }
+
+__device__ __forceinline__ uint32_t encode_by_quotient(uint32_t x_bits, double scale, const XEntry *lut, uint32_t first_of_one) {
+    return xlut_code_by_quotient(x_bits, scale, lut, first_of_one);
+}
+
 }  // namespace cn

@@ -33,6 +33,7 @@ struct Context {
     float *table = nullptr;          // 126 floats
     struct XStep *xsteps = nullptr;  // the steps of the code function (cn_xlut.h), found once at init
     int xstep_count = 0;
+    struct XEntry *quotient_table = nullptr;  // the encoder's table for precision 1 (cn_encode_table.h), built once at init
     void *workspace = nullptr;       // split-K partial sums
     size_t workspace_bytes = 0;
     uint32_t *reduce_scratch = nullptr;  // per-workgroup partial results + ticket counters

@@ -74,6 +74,7 @@ static cn_status init_device(int device) {
             if (!armed) return;
             (void)hipFree(c.table);
             (void)hipFree(c.xsteps);
+            (void)hipFree(c.quotient_table);
             (void)hipFree(c.workspace);
             (void)hipFree(c.reduce_scratch);
             (void)hipFree(c.tickets);
@@ -104,6 +105,14 @@ static cn_status init_device(int device) {
         c.xstep_count = count;
         CN_HIP(hipMalloc((void **)&c.xsteps, sizeof(steps)));
         CN_HIP(hipMemcpy(c.xsteps, steps, sizeof(steps), hipMemcpyHostToDevice));
+        // the table for precision 1, where the quotient is the operand itself: the code as a function of the quotient
+        static XEntry of_quotient[kXEntries];
+        if (!xlut_build_from_steps(steps, count, 1.0f, slot, of_quotient)) {
+            set_error("init: the encoder's table on the quotient could not be built");
+            return CN_ERR_ARG;
+        }
+        CN_HIP(hipMalloc((void **)&c.quotient_table, sizeof(of_quotient)));
+        CN_HIP(hipMemcpy(c.quotient_table, of_quotient, sizeof(of_quotient), hipMemcpyHostToDevice));
     }
 
     c.workspace_bytes = default_workspace_bytes();
@@ -199,6 +208,7 @@ cn_status cn_shutdown(void) {
         CN_HIP(hipDeviceSynchronize());
         CN_HIP(hipFree(c.table));
         CN_HIP(hipFree(c.xsteps));
+        CN_HIP(hipFree(c.quotient_table));
         CN_HIP(hipFree(c.workspace));
         CN_HIP(hipFree(c.reduce_scratch));
         CN_HIP(hipFree(c.tickets));

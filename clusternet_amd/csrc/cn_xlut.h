@@ -290,4 +290,22 @@ CN_HD uint32_t xlut_code(uint32_t bits, XEntry e) {
     return (e.codes >> sel) & 0xffu;
 }
 
+// ---- the table on the quotient -------------------------------------------------------------------
+// The literal procedure looks at x only through a = fl(x / precision), so its code is one fixed step function of
+// the bit pattern of a, whatever the precision: the table above for precision 1 (where a = x) is that function.
+// An encoder can therefore keep that one table and pay for the quotient per element instead of building a table
+// per precision.  The quotient is formed as (float)((double)x * (1.0 / (double)precision)), which rounds the way
+// x / precision does for every pair of fp32 operands whose quotient lies in the normal range: the product carries
+// a relative error below 2^-51, and a quotient of two 24-bit significands is either representable or at least
+// 2^-49 (relative) away from the nearest rounding boundary of the format, so the conversion falls on the same side;
+// zeros, infinities and NaNs come out as the division's own (0 * inf = NaN = 0 / 0 and so on; a NaN's sign and
+// payload do not matter to the code); no intermediate leaves the range of a double.  Below the normal range the
+// two may differ in the last place, where every quotient has the code 254.
+CN_HD double xlut_quotient_scale(float precision) { return 1.0 / (double)precision; }
+
+CN_HD uint32_t xlut_code_by_quotient(uint32_t x_bits, double scale, const XEntry *table_of_one, uint32_t first_of_one) {
+    const uint32_t a = x_to_bits((float)((double)x_from_bits(x_bits) * scale));
+    return xlut_code(a, table_of_one[xlut_index(a & 0x7fffffffu, first_of_one)]);
+}
+
 }  // namespace cn

@@ -133,9 +133,9 @@ cn_status cn_compress_8bit_dp(const float *x_device, const float *precision_devi
 /* *precision_out_device = max_i |x_i| and codes = the codes of x under that precision, in one call and without a
  * round trip to the host: the same bits as cn_absmax_f32 followed by cn_compress_8bit_dp.  The pair of calls in front
  * of every exchange of a gradient, max(abs(grad)) then compression_8bit (source/DeepNeuralNetwork.cpp:334-339,
- * source/test.cu:2108-2111).  It runs as those two kernels, one behind the other on the stream; a form that does both
- * phases in one launch (a wait across the grid between them) exists and measures slower on this part, see
- * cn_host_absmax_compress_single_launch. */
+ * source/test.cu:2108-2111).  Aligned tensors of up to 2^23 elements take one launch that does both phases (a bounded
+ * wait across the resident grid between them, the tensor read once); everything else runs as those two kernels, one
+ * behind the other on the stream.  cn_host_absmax_compress_single_launch pins either form. */
 cn_status cn_absmax_compress_8bit(const float *x_device, size_t n, uint8_t *codes_device,
                                   float *precision_out_device, void *stream);
 

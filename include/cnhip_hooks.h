@@ -39,10 +39,14 @@ void cn_host_gemm_epilogue_in_kernel(int enabled);
 
 /* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
 void cn_host_codec_workgroups_per_cu(int per_cu);
-/* Largest element count that compression (all forms) encodes with the literal procedure, element by element,
- * instead of building the table first; 0 = always the table, SIZE_MAX = the library's own threshold.
- * Both give the same bits. */
-void cn_host_codec_literal_upto(size_t n);
+/* Which encoder compression (all forms) takes: 0 = the library's choice by size, 1 = the literal procedure element by
+ * element, 2 = the table on the quotient x / precision, 3 = the table built for the call's precision.  All give the
+ * same bits; for tests of that equality and for measurements. */
+void cn_host_codec_encoder(int which);
+/* Over `patterns` consecutive fp32 bit patterns of x starting at `first_pattern`: how often the quotient that the
+ * table encoder forms, (float)((double)x * (1.0 / (double)precision)), differs in its bits from x / precision on the
+ * device (two NaNs and two results below the normal range count as equal).  Synchronises; -1 on a HIP error. */
+long long cn_host_quotient_mismatches(float precision, uint32_t first_pattern, unsigned long long patterns);
 
 /* Nonzero: the single-launch reductions (abs-max, max, sum) put a release fence at device scope between a
  * workgroup's partial result and its arrival count, the form the memory model prescribes, instead of ordering the
@@ -53,9 +57,10 @@ void cn_host_reduction_fences(int enabled);
  * their tiles from) are not zero: 0 whenever no kernel is running; -1 if the device is not initialised. */
 int cn_host_tile_counters_in_use(void);
 
-/* Nonzero: cn_absmax_compress_8bit runs as one launch (abs-max, a wait across the resident grid, compression) for
- * aligned tensors below 2^26 elements instead of as two kernels.  Same bits. */
-void cn_host_absmax_compress_single_launch(int enabled);
+/* cn_absmax_compress_8bit as one launch (abs-max, a wait across the resident grid, compression) instead of as two
+ * kernels: 1 = wherever the single launch can run (aligned tensors below 2^26 elements), 0 = never, negative = the
+ * library's own choice by size.  Same bits. */
+void cn_host_absmax_compress_single_launch(int mode);
 
 /* How often a workgroup of the single-launch cn_absmax_compress_8bit looks for the rest of the grid before it takes the maximum
  * by itself; negative = the library's figure.  0 lets the tests reach that path: every workgroup then gives up at once. */
@@ -80,6 +85,9 @@ int cn_host_xlut_step_count(void);
 int cn_host_xlut_build(float precision, void *entries, uint32_t *first);
 int cn_host_xlut_encode_many(float precision, const float *x, size_t n, uint8_t *codes);
 int cn_host_encode_exact(float x, float precision);
+/* The encoder on the quotient, evaluated on the CPU as a workgroup evaluates it: the table for precision 1 looked
+ * up at (float)((double)x * (1.0 / (double)precision)).  Returns 1, or 0 if that table cannot be built. */
+int cn_host_quotient_encode_many(float precision, const float *x, size_t n, uint8_t *codes);
 
 #ifdef __cplusplus
 }

@@ -30,13 +30,13 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
-@pytest.fixture(params=["literal_for_small_tensors", "table_always"])
+@pytest.fixture(params=["literal_for_small_tensors", "table_on_the_quotient", "table_always"])
 def codec_form(request):
-    """Compression has two encoders that must give the same bits: the literal procedure per element for small
-    tensors and the per-call table.  Tests that use this fixture run once with the library's own choice and once
-    with the table forced for every size, so the small adversarial inputs exercise both."""
+    """Compression has three encoders that must give the same bits: the literal procedure per element for small
+    tensors, the fixed table on the quotient x / precision for mid-size ones and the table built for the call's
+    precision for the largest.  Tests that use this fixture run once with the library's own choice by size and once
+    with each table forced for every size, so the small adversarial inputs exercise all three."""
     from clusternet_amd import _lib as L
-    if request.param == "table_always":
-        L.lib().cn_host_codec_literal_upto(0)
+    L.lib().cn_host_codec_encoder({"literal_for_small_tensors": 0, "table_on_the_quotient": 2, "table_always": 3}[request.param])
     yield request.param
-    L.lib().cn_host_codec_literal_upto(2 ** 64 - 1)  # back to the library's own threshold
+    L.lib().cn_host_codec_encoder(0)  # back to the library's own choice

@@ -287,7 +287,7 @@ def test_decode_through_a_given_table(dev):
 
 def test_absmax_and_compression_in_one_call(dev):
     """cn_absmax_compress_8bit against cn_absmax_f32 followed by cn_compress_8bit_dp and against the CPU checker, as
-    the two kernels it runs by default and as the single launch behind cn_host_absmax_compress_single_launch: sizes on
+    the library picks by size, as the two kernels and as the single launch (cn_host_absmax_compress_single_launch): sizes on
     both sides of every dispatch boundary, unaligned starts, all-zero and NaN-bearing data, calls in a row, and with
     the single launch's wait for the rest of the grid cut to nothing, so that every workgroup that would have
     waited takes the maximum by itself."""
@@ -300,7 +300,7 @@ def test_absmax_and_compression_in_one_call(dev):
     base[::101] *= 20
     bt = _t(base, dev)
     try:
-        for single, spins in ((0, -1), (1, -1), (1, 0), (1, -1)):
+        for single, spins in ((-1, -1), (0, -1), (1, -1), (1, 0), (1, -1)):
             L.lib().cn_host_absmax_compress_single_launch(single)
             L.lib().cn_host_absmax_compress_spin_limit(spins)
             for n, off in ((1, 0), (3, 0), (5, 4), (4096, 0), (4097, 0), (70_001, 0), (128 * 40000, 0), (128 * 40000, 1),
@@ -330,25 +330,27 @@ def test_absmax_and_compression_in_one_call(dev):
             assert float(prec.cpu()[0]) == -1.0 and codes.numel() == 0
     finally:
         L.lib().cn_host_absmax_compress_spin_limit(-1)
-        L.lib().cn_host_absmax_compress_single_launch(0)
+        L.lib().cn_host_absmax_compress_single_launch(-1)
 
 
 def test_compression_beyond_the_cache_draws_its_tiles(dev, codec_form):
-    """From 2^26 elements on compression runs one workgroup per compute unit that draws 49152-element tiles from a
+    """From 2^27 elements on compression runs one workgroup per compute unit that draws 49152-element tiles from a
     counter: sizes round a tile boundary, n % 4 tails and a start that is 16 bytes in, against the CPU checker, each
-    size twice in a row (the second call finds the counter as the first one left it)."""
-    if codec_form != "literal_for_small_tensors":
-        pytest.skip("the table is used at this size either way")
+    size twice in a row (the second call finds the counter as the first one left it).  Once with the encoder the
+    library takes at this size (the table built for the call's precision) and once with the table on the quotient."""
+    if codec_form == "table_always":
+        pytest.skip("the library's own choice at this size")
     import torch
     import clusternet_amd as cn
     rng = np.random.default_rng(77)
     tile = 1024 * 12 * 4
-    base_n = (1 << 26) + 2 * tile + 16
+    first = 1 << 27
+    base_n = first + 2 * tile + 16
     mag = np.exp(rng.uniform(np.log(1e-7), np.log(1.3), base_n)).astype(np.float32)
     base = (mag * rng.choice(np.array([-1.0, 1.0], np.float32), base_n)).astype(np.float32)
     want_all = oracle.port_compress(base, 0.77)
     bt, ct = _t(base, dev), _t(want_all, dev)
-    for n in (1 << 26, (1 << 26) + 1, (1 << 26) + 3, (1 << 26) + tile - 4, (1 << 26) + tile, (1 << 26) + 2 * tile + 7):
+    for n in (first, first + 1, first + 3, first + tile - 4, first + tile, first + 2 * tile + 7):
         for off in (0, 4):
             for _ in range(2):
                 canary = torch.full((n + 64,), 0xAB, dtype=torch.uint8, device=dev)
@@ -373,7 +375,7 @@ def test_kernels_that_draw_tiles_replay_from_a_graph(dev, codec_form):
     from clusternet_amd import _lib as L
     gen = torch.Generator(device=dev)
     gen.manual_seed(21)
-    n = (1 << 26) + 5 * 4096 + 3
+    n = (1 << 27) + 5 * 4096 + 3
     x = torch.randn(n, device=dev, generator=gen) * 0.02
     w0 = torch.randn(n, device=dev, generator=gen)
     want_codes = cn.compression_8bit(x, 0.11)
@@ -405,7 +407,7 @@ def test_kernels_that_draw_tiles_replay_from_a_graph(dev, codec_form):
 
 
 def test_kernels_that_draw_tiles_may_overlap_on_two_streams(dev, codec_form):
-    """Launches take the library's ticket counters in turn, so two compressions beyond the cache issued on two streams
+    """Launches take the library's ticket counters in turn, so two compressions of 2^27 elements and more issued on two streams
     (default priority) may run at the same time without drawing each other's tiles: both must give the codes of a
     compression that ran alone, over several rounds."""
     if codec_form != "literal_for_small_tensors":
@@ -415,7 +417,7 @@ def test_kernels_that_draw_tiles_may_overlap_on_two_streams(dev, codec_form):
     from clusternet_amd import _lib as L
     gen = torch.Generator(device=dev)
     gen.manual_seed(33)
-    n = (1 << 26) + 12345 * 4
+    n = (1 << 27) + 12345 * 4
     xs = [torch.randn(n, device=dev, generator=gen) * 0.02 for _ in range(2)]
     want = [cn.compression_8bit(x, 0.09) for x in xs]
     streams = [torch.cuda.Stream(), torch.cuda.Stream()]
@@ -432,3 +434,23 @@ def test_kernels_that_draw_tiles_may_overlap_on_two_streams(dev, codec_form):
         for o, w in zip(outs, want):
             assert torch.equal(o, w)
     assert L.lib().cn_host_tile_counters_in_use() == 0
+
+
+def test_the_quotient_formed_in_double_precision_is_the_division(dev, codec_form):
+    """The table on the quotient looks up (float)((double)x * (1.0 / (double)p)) where the literal procedure looks at x / p.
+    On the device, over all 2^32 bit patterns of x, the two must agree in every bit (NaNs aside, and results below the
+    normal range, which all have the code 254) for precisions of every kind: ordinary, negative, powers of two,
+    significands of all ones or one above a power of two (the reciprocal's worst cases), tiny, huge, denormal, zero,
+    infinite and NaN."""
+    if codec_form != "table_on_the_quotient":
+        pytest.skip("one run is enough")
+    from clusternet_amd import _lib as L
+    rng = np.random.default_rng(2024)
+    bits = lambda b: float(np.array([b], np.uint32).view(np.float32)[0])
+    precisions = [1.0, 0.1, 3.0, -0.37, 0.0234375, 2.0 ** -60, 2.0 ** 60, 1e-30, 1e30, 3e38, 1.2e-38, 1e-42, 1.4e-45,
+                  bits(0x3fffffff), bits(0x3f800001), bits(0x3f7fffff), bits(0x40400001), bits(0x007fffff), bits(0x7f7fffff),
+                  0.0, -0.0, float("inf"), float("nan")]
+    precisions += [float(v) for v in np.exp(rng.uniform(np.log(1e-36), np.log(1e36), 40))]
+    precisions += [float(v) for v in rng.uniform(1e-3, 2.0, 40).astype(np.float32)]
+    for p in precisions:
+        assert L.lib().cn_host_quotient_mismatches(p, 0, 1 << 32) == 0, p

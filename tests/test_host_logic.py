@@ -121,6 +121,51 @@ def test_encoder_table_over_precisions_and_step_neighbourhoods():
     assert trusted_precisions >= 18
 
 
+def _encode_by_quotient_host(x, precision):
+    L = cn.lib()
+    x = np.ascontiguousarray(x, np.float32)
+    codes = np.empty(x.size, np.uint8)
+    L.cn_host_quotient_encode_many.argtypes = [C.c_float, C.c_void_p, C.c_size_t, C.c_void_p]
+    assert L.cn_host_quotient_encode_many(float(precision), x.ctypes.data, x.size, codes.ctypes.data) == 1
+    return codes
+
+
+def test_encoder_on_the_quotient_equals_the_literal_procedure():
+    """The table for precision 1 looked up at (float)((double)x * (1 / (double)p)) against the literal procedure (the CPU
+    checker), for every kind of precision, with no exception: there is no precision for which this encoder steps
+    aside.  Inputs: random values over the whole coded range, every pattern within 40 ulps of p times every step of
+    the code function (where a quotient rounded the wrong way would change the code), a strided sweep over all
+    bit patterns.  The precisions include ones whose significand is all ones or one above a power of two (the
+    reciprocal's worst cases), denormal ones and the degenerate ones (0, inf, NaN)."""
+    rng = np.random.default_rng(321)
+    t = oracle.table()
+    edges = np.concatenate([t, (t[:-1] + t[1:]) / 2, [1.5e-6, 0.995703, 1.0]]).astype(np.float32)
+    bits = lambda b: float(np.array([b], np.uint32).view(np.float32)[0])
+    with np.errstate(all="ignore"):
+        sweep = np.arange(0, 1 << 32, 16411, dtype=np.uint64).astype(np.uint32).view(np.float32)
+        precisions = [1.0, 0.1, 0.0234375, 3.0, 1e-5, 7.7e4, -1.0, -0.37, 2.0 ** -60, 2.0 ** 60, 1e-30, 1e30,
+                      3e38, 1.2e-38, 1e-42, 1.4e-45, 0.0, -0.0, float("inf"), float("-inf"), float("nan"),
+                      bits(0x3fffffff), bits(0x3f800001), bits(0x3f7fffff), bits(0x40400001), bits(0x007fffff), bits(0x7f7fffff)]
+        precisions += list(np.exp(rng.uniform(np.log(1e-36), np.log(1e36), 30)))
+        for p in precisions:
+            p32 = np.float32(p)
+            scale = p32 if np.isfinite(p32) and p32 != 0 else np.float32(1.0)
+            near = (np.repeat(edges, 81).view(np.uint32).astype(np.int64)
+                    + np.tile(np.arange(-40, 41), edges.size)).astype(np.uint32).view(np.float32)
+            scaled = (near.astype(np.float64) * float(scale)).astype(np.float32)
+            around = (np.repeat(scaled, 9).view(np.uint32).astype(np.int64) + np.tile(np.arange(-4, 5), scaled.size))
+            around = np.clip(around, 0, 0x7f800000).astype(np.uint32).view(np.float32)
+            x = np.concatenate([
+                np.exp(rng.uniform(np.log(1e-7), np.log(1.5), 200_000)).astype(np.float32) * scale,
+                -np.exp(rng.uniform(np.log(1e-7), np.log(1.5), 50_000)).astype(np.float32) * scale,
+                around, -around, sweep,
+            ]).astype(np.float32)
+            codes = _encode_by_quotient_host(x, p)
+            want = oracle.compress(x, float(p), 0)
+            bad = np.nonzero(codes != want)[0]
+            assert bad.size == 0, (p, x[bad[:4]], codes[bad[:4]], want[bad[:4]])
+
+
 def test_encoder_table_shape():
     L = cn.lib()
     n = L.cn_host_xlut_entries()
