@@ -91,6 +91,8 @@ def lib():
     L.cn_host_quotient_mismatches.restype = C.c_longlong
     L.cn_host_gemm_w8_rows.argtypes = [C.c_int]
     L.cn_host_gemm_w8_rows.restype = None
+    L.cn_host_gemm_small.argtypes = [C.c_int]
+    L.cn_host_gemm_small.restype = None
     L.cn_host_tile_counters_in_use.argtypes = []
     L.cn_host_tile_counters_in_use.restype = C.c_int
     L.cn_host_reduction_fences.argtypes = [C.c_int]

@@ -922,6 +922,7 @@ static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, 
 static int g_force_tile_n = 0;
 static bool g_wide_store = true;
 static bool g_w8_rows = true;  // test hook: false keeps the tiled kernel for every product on 8-bit weights
+static bool g_small = true;    // test hook: false keeps the tiled kernel for small products too
 static bool g_epilogue_in_kernel = true;  // test hook: false sends every fused product through the workspace
 
 // What follows the product instead of its delivery: bias and maxout (the forward pass of a maxout layer; `bias`
@@ -994,6 +995,18 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
             if (chunks > 1) return add_chunk_planes(ctx->workspace, ctx->num_cu, chunks, M, N, C, ldc, amax, st);
             return CN_OK;
         }
+    }
+    if (!w8 && g_small && g_force_tile_n == 0 && gemm_small_applies(ta, tb, M, N, K, A, lda, (const float *)B, ldb)) {
+        // too small to fill the chip with tiles: one launch, and for every entry point the same one, so that the
+        // calls that fuse something behind the product keep giving the bits of the separate calls
+        if (then) {
+            if ((size_t)M * (size_t)N * sizeof(float) > ctx->workspace_bytes) { set_error("%s: product does not fit the workspace", who); return CN_ERR_WORKSPACE; }
+            C = (float *)ctx->workspace;
+            ldc = N;
+        }
+        s = gemm_small(ta, tb, M, N, K, A, lda, (const float *)B, ldb, C, ldc, amax, st);
+        if (s != CN_OK) return s;
+        return then ? finish_from(C) : CN_OK;
     }
     GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->plan_bytes, g_force_tile_n);
     // K not split, whole 128-row tiles and pools of 1, 2 or 4: bias + maxout, or the expansion, happen in the
@@ -1117,6 +1130,7 @@ void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
 
 // Test hook: 0 = bias + maxout and the maxout expansion never run inside the product's write-out.
 void cn_host_gemm_w8_rows(int enabled) { g_w8_rows = enabled != 0; }
+void cn_host_gemm_small(int enabled) { g_small = enabled != 0; }
 void cn_host_gemm_epilogue_in_kernel(int enabled) { g_epilogue_in_kernel = enabled != 0; }
 
 // Test and tuning hook: 0 = let the planner choose the tile, 128 / 256 = force that width of the 128-row

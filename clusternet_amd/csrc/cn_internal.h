@@ -111,6 +111,16 @@ int gemm_w8_rows_splits(int64_t M, int64_t N, int64_t K, const float *A, int64_t
 cn_status gemm_w8_rows(int splits, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const uint8_t *W, int64_t ldw,
                        float scale, float *C, int64_t ldc, const float *table, void *workspace, int device, hipStream_t st);
 
+// The product in one launch for shapes too small to fill the chip with tiles (cn_gemm_small.hip): a workgroup per
+// 32 x 32 block of the result, K split among its wavefronts.
+constexpr int64_t kSmallMaxBlocks = 512;           // of 32 x 32 results
+constexpr int64_t kSmallMaxWork = (int64_t)1 << 28;  // M * N * K; half of it where the blocks are 16 x 16
+bool gemm_small_applies(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
+                        int64_t ldb);
+// amax: NULL, or a word that starts at 0 and receives the bit pattern of max |C|.
+cn_status gemm_small(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
+                     int64_t ldb, float *C, int64_t ldc, uint32_t *amax, hipStream_t st);
+
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
 
 constexpr int kTileM = 128;

@@ -35,6 +35,9 @@ void cn_host_gemm_wide_store(int enabled);
 /* 0 keeps the tiled kernel for every product on 8-bit weights; 1 (default) lets products of up to 1024 rows take the
  * kernel that decodes straight into registers. */
 void cn_host_gemm_w8_rows(int enabled);
+/* 0 keeps the tiled kernel (and its chunk sum) for every plain product; 1 (default) lets products too small to fill the
+ * chip with tiles take the kernel that finishes them in one launch. */
+void cn_host_gemm_small(int enabled);
 void cn_host_gemm_epilogue_in_kernel(int enabled);
 
 /* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
