@@ -454,3 +454,45 @@ def test_the_quotient_formed_in_double_precision_is_the_division(dev, codec_form
     precisions += [float(v) for v in rng.uniform(1e-3, 2.0, 40).astype(np.float32)]
     for p in precisions:
         assert L.lib().cn_host_quotient_mismatches(p, 0, 1 << 32) == 0, p
+
+
+def test_more_than_2_to_the_32_elements(dev, codec_form):
+    """Element counts are size_t throughout: a tensor of 2^32 + 12293 elements (17 GB of fp32; the reference's int sizes
+    stop at 2^31) through abs-max, compression and decompression.  Abs-max finds a value planted in the last element;
+    the codes and the decoded values of the whole tensor equal, window by window (the start, both sides of element
+    2^32, the end with its n % 4 tail), those of the windows processed on their own, which the other tests hold to
+    the CPU checker."""
+    if codec_form != "literal_for_small_tensors":
+        pytest.skip("one run is enough")
+    import torch
+    import clusternet_amd as cn
+    n = (1 << 32) + 3 * 4096 + 5
+    free, _ = torch.cuda.mem_get_info()
+    if free < 48 * (1 << 30):
+        pytest.skip("needs 48 GB of device memory")
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(99)
+    x = torch.empty(n, device=dev)
+    piece = 1 << 28
+    for lo in range(0, n, piece):  # filled piece by piece: the generator's own limits are not under test
+        hi = min(lo + piece, n)
+        x[lo:hi].normal_(0.0, 0.02, generator=gen)
+    x[n - 1] = 7.25
+    prec = cn.absmax(x)
+    assert float(prec.cpu()[0]) == 7.25
+    x[n - 1] = 0.01
+    x[(1 << 32) + 1] = -0.3
+    assert float(cn.absmax(x).cpu()[0]) == float(torch.maximum(x[:1 << 31].abs().max(), x[1 << 31:].abs().max()).cpu())
+    p = 0.11
+    codes = cn.compression_8bit(x, p)
+    windows = [(0, 1 << 20), ((1 << 32) - (1 << 20), (1 << 32) + 4096 + 8), (n - (1 << 20) - 3, n)]
+    for lo, hi in windows:
+        lo -= lo % 4  # windows start 16-byte aligned, as the whole tensor does
+        assert torch.equal(codes[lo:hi], cn.compression_8bit(x[lo:hi], p)), (lo, hi)
+    del x
+    back = cn.decompression_8bit(codes, p)
+    for lo, hi in windows:
+        lo -= lo % 4
+        assert torch.equal(back[lo:hi].view(torch.int32), cn.decompression_8bit(codes[lo:hi], p).view(torch.int32)), (lo, hi)
+    from clusternet_amd import _lib as L
+    assert L.lib().cn_host_tile_counters_in_use() == 0
