@@ -496,3 +496,39 @@ def test_more_than_2_to_the_32_elements(dev, codec_form):
         assert torch.equal(back[lo:hi].view(torch.int32), cn.decompression_8bit(codes[lo:hi], p).view(torch.int32)), (lo, hi)
     from clusternet_amd import _lib as L
     assert L.lib().cn_host_tile_counters_in_use() == 0
+
+
+def test_one_launch_abs_max_and_compression_beside_a_product_on_another_stream(dev, codec_form):
+    """The single launch waits inside the kernel for the rest of its grid.  With products that fill the chip running on
+    another stream (default priority) part of that grid may not be resident when the first workgroups arrive: the
+    wait is bounded, whoever gives up takes the maximum by itself, and the result is the one of a call that ran
+    alone.  Products and codec share no scratch memory (the products' chunk planes against the codec's ticket lines)."""
+    if codec_form != "literal_for_small_tensors":
+        pytest.skip("one run is enough")
+    import torch
+    import clusternet_amd as cn
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(8)
+    n = 128 * 40000
+    x = torch.randn(n, device=dev, generator=gen) * 0.02
+    want_codes, want_prec = cn.absmax_compression_8bit(x)
+    A = torch.randn((4096, 4096), device=dev, generator=gen)
+    B = torch.randn((4096, 4096), device=dev, generator=gen)
+    C = torch.empty((4096, 4096), device=dev)
+    want_C = cn.dot(A, B)
+    side, main = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        codes = torch.zeros(n, dtype=torch.uint8, device=dev)
+        prec = torch.zeros(1, device=dev)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            for _ in range(4):
+                cn.dot(A, B, out=C)
+        with torch.cuda.stream(main):
+            for _ in range(8):
+                cn.absmax_compression_8bit(x, out=codes, precision_out=prec)
+        torch.cuda.synchronize()
+        assert torch.equal(prec.view(torch.int32), want_prec.view(torch.int32))
+        assert torch.equal(codes, want_codes)
+        assert torch.equal(C.view(torch.int32), want_C.view(torch.int32))
