@@ -212,6 +212,28 @@ def bench_cfg1(torch, cn, dev):
     return out
 
 
+def bench_layout(torch, cn, dev):
+    """The passes either side of the products: transposition (the reference's T / to_col_major, source/basicOps.cu:14-127)
+    and fill (zeros / ones / fill), on the 100000 x 8192 weights; torch's own beside them as movers that are not this
+    library's."""
+    from clusternet_amd import _lib as L
+    rows, cols = 100000, 8192
+    n = rows * cols
+    A = torch.empty((rows, cols), device=dev).normal_(0.0, 1.0)
+    out = torch.empty((cols, rows), device=dev)
+    res = {}
+    t = time_region(torch, lambda: L.transpose(A, out), 20, 3)
+    res["transpose_GBps"] = 8.0 * n / t / 1e6
+    res["transpose_ms"] = t
+    t = time_region(torch, lambda: out.copy_(A.t()), 10, 2)
+    res["torch_transpose_GBps"] = 8.0 * n / t / 1e6
+    t = time_region(torch, lambda: L.fill(out, 1.0), 20, 3)
+    res["fill_GBps"] = 4.0 * n / t / 1e6
+    t = time_region(torch, lambda: out.fill_(1.0), 20, 3)
+    res["torch_fill_GBps"] = 4.0 * n / t / 1e6
+    return res
+
+
 def bench_fused(torch, cn, dev):
     """C = A . decode(W8) for A {32,128,512} x 4096, W 4096 x 4096: fused kernel against
     decompression_8bit followed by dot."""
@@ -457,6 +479,9 @@ def main():
         torch.cuda.empty_cache()
         if not args.no_cpu and args.only is None and "error" not in extra["codec"]:
             extra["codec"]["cpu_port"] = cpu_codec_baseline()
+    if args.only in (None, "codec"):
+        section("layout_100000x8192", lambda: bench_layout(torch, cn, dev))
+        torch.cuda.empty_cache()
     if args.only in (None, "fused"):
         section("fused_w8_gemm_4096x4096", lambda: bench_fused(torch, cn, dev))
     if args.only in (None, "step"):
