@@ -19,48 +19,118 @@ static inline int grid_for(const Context *ctx, int64_t work_items, int per_cu = 
     return (int)(blocks < 1 ? 1 : blocks);
 }
 
-// out[c][r] = in[r][c] on 64 x 64 tiles through LDS, a workgroup per tile.  Whole tiles of 16-byte aligned matrices move as
-// 16-byte vectors on both sides (256 contiguous bytes per tile row); the tiles are numbered down the columns of `in`, so
-// that workgroups started one after the other write neighbouring pieces of the same 64 rows of `out`: the stream that
-// writes is the one that needs its window narrow.  4.3 TB/s became 5.3 TB/s on a 100000 x 8192 matrix and 4.2 became
-// 5.7 on 20000 x 40000.
-template <bool kVector>
-__global__ __launch_bounds__(kT) void transpose64_kernel(const float *__restrict__ in, int64_t rows, int64_t cols,
-                                                         float *__restrict__ out, int64_t tiles_r) {
-    __shared__ float tile[64][65];
+// out[c][r] = in[r][c] on square tiles of kEdge = 64 or 128 through LDS, a workgroup of kEdge^2 / 16 lanes per tile.  Whole
+// tiles of 16-byte aligned matrices move as 16-byte vectors on both sides (256 or 512 contiguous bytes per tile row); the
+// tiles are numbered down the columns of `in`, so that workgroups started one after the other write neighbouring
+// pieces of the same kEdge rows of `out`: the stream that writes is the one that needs its window narrow.  On 64 x 64
+// tiles 4.3 TB/s (32 x 32 tiles of single floats) became 4.9 to 5.3 TB/s on a 100000 x 8192 matrix and 4.2 became 5.5 to
+// 5.7 on 20000 x 40000; 128 x 128 tiles (twice the contiguous bytes per row on either side, 66 KB of LDS) give 5.5 and 5.7
+// there and 6.1 instead of 5.5 on 8192 x 100096 (128 x 64 tiles: 5.3 / 5.5 / 6.1; 64 x 128: 5.0 / 5.5 / 5.6; 32 x 256 and
+// 256 x 32 in between), so matrices with a thousand and more of them take those.
+template <int kEdge, bool kVector>
+__global__ __launch_bounds__(kEdge * kEdge / 16) void transpose_tile_kernel(const float *__restrict__ in, int64_t rows, int64_t cols,
+                                                                            float *__restrict__ out, int64_t tiles_r) {
+    extern __shared__ float tile[];  // kEdge rows of kEdge + 1 floats
+    constexpr int kPitch = kEdge + 1, kLanes = kEdge * kEdge / 16;
     const int64_t tc = blockIdx.x / tiles_r, tr = blockIdx.x % tiles_r;
-    const int64_t r0 = tr * 64, c0 = tc * 64;
-    if (kVector && r0 + 64 <= rows && c0 + 64 <= cols) {
-        const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;  // 16 vectors across, 16 rows down, four passes
+    const int64_t r0 = tr * kEdge, c0 = tc * kEdge;
+    if (kVector && r0 + kEdge <= rows && c0 + kEdge <= cols) {
+        constexpr int kAcross = kEdge / 4, kDown = kLanes / kAcross;  // vectors across, rows down, four passes
+        const int tx = threadIdx.x % kAcross, ty = threadIdx.x / kAcross;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int r = ty + 16 * j;
+        for (int j = 0; j < kEdge / kDown; ++j) {
+            const int r = ty + kDown * j;
             const f32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(in + (r0 + r) * cols + c0 + 4 * tx));
-            tile[r][4 * tx + 0] = v.x;
-            tile[r][4 * tx + 1] = v.y;
-            tile[r][4 * tx + 2] = v.z;
-            tile[r][4 * tx + 3] = v.w;
+            tile[r * kPitch + 4 * tx + 0] = v.x;
+            tile[r * kPitch + 4 * tx + 1] = v.y;
+            tile[r * kPitch + 4 * tx + 2] = v.z;
+            tile[r * kPitch + 4 * tx + 3] = v.w;
         }
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = ty + 16 * j;
-            const f32x4_t o = {tile[4 * tx + 0][c], tile[4 * tx + 1][c], tile[4 * tx + 2][c], tile[4 * tx + 3][c]};
+        for (int j = 0; j < kEdge / kDown; ++j) {
+            const int c = ty + kDown * j;
+            const f32x4_t o = {tile[(4 * tx + 0) * kPitch + c], tile[(4 * tx + 1) * kPitch + c], tile[(4 * tx + 2) * kPitch + c],
+                               tile[(4 * tx + 3) * kPitch + c]};
             __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t *>(out + (c0 + c) * rows + r0 + 4 * tx));
         }
     } else {
-        const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 across, 4 down, sixteen passes
+        constexpr int kDown = kLanes / kEdge;  // kEdge single floats across, kDown rows down
+        const int tx = threadIdx.x % kEdge, ty = threadIdx.x / kEdge;
 #pragma unroll 4
-        for (int j = 0; j < 64; j += 4) {
+        for (int j = 0; j < kEdge; j += kDown) {
             const int64_t r = r0 + ty + j, c = c0 + tx;
-            if (r < rows && c < cols) tile[ty + j][tx] = in[r * cols + c];
+            if (r < rows && c < cols) tile[(ty + j) * kPitch + tx] = in[r * cols + c];
         }
         __syncthreads();
 #pragma unroll 4
-        for (int j = 0; j < 64; j += 4) {
+        for (int j = 0; j < kEdge; j += kDown) {
             const int64_t c = c0 + ty + j, r = r0 + tx;
-            if (r < rows && c < cols) out[c * rows + r] = tile[tx][ty + j];
+            if (r < rows && c < cols) out[c * rows + r] = tile[tx * kPitch + ty + j];
         }
+    }
+}
+
+// The same on 128 x 128 tiles by a persistent grid (a workgroup of 1024 lanes per compute unit) that draws its tiles in
+// that order from a counter: the loads of a workgroup's next tile are in flight while it stores the current one.
+__global__ __launch_bounds__(1024) void transpose_drawn_kernel(const float *__restrict__ in, int64_t rows, int64_t cols,
+                                                               float *__restrict__ out, int64_t tiles_r, uint32_t tiles,
+                                                               uint32_t *__restrict__ counter) {
+    extern __shared__ float tile[];  // 128 rows of 129 floats
+    __shared__ uint32_t queue_slots[2];
+    constexpr int kEdge = 128, kPitch = kEdge + 1, kAcross = kEdge / 4, kDown = 1024 / kAcross;
+    const int tx = threadIdx.x % kAcross, ty = threadIdx.x / kAcross;
+    const int sx = threadIdx.x % kEdge, sy = threadIdx.x / kEdge;  // the element-wise form of ragged tiles: 128 across, 8 down
+    f32x4_t v[kEdge / kDown];
+    auto whole = [&](uint32_t t) {
+        const int64_t r0 = (int64_t)(t % tiles_r) * kEdge, c0 = (int64_t)(t / tiles_r) * kEdge;
+        return r0 + kEdge <= rows && c0 + kEdge <= cols;
+    };
+    auto request = [&](uint32_t t) {
+        const int64_t r0 = (int64_t)(t % tiles_r) * kEdge, c0 = (int64_t)(t / tiles_r) * kEdge;
+#pragma unroll
+        for (int j = 0; j < kEdge / kDown; ++j)
+            v[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t *>(in + (r0 + ty + kDown * j) * cols + c0 + 4 * tx));
+    };
+    TileQueue q = tile_queue(counter, tiles, queue_slots);
+    q.draw_ahead();
+    uint32_t cur = q.next();
+    if (cur < tiles) q.draw_ahead();  // every workgroup draws exactly one ticket past the last tile
+    if (cur < tiles && whole(cur)) request(cur);
+    while (cur < tiles) {
+        const int64_t r0 = (int64_t)(cur % tiles_r) * kEdge, c0 = (int64_t)(cur / tiles_r) * kEdge;
+        const bool is_whole = whole(cur);
+        if (is_whole) {
+#pragma unroll
+            for (int j = 0; j < kEdge / kDown; ++j) {
+                float *row = tile + (ty + kDown * j) * kPitch + 4 * tx;
+                row[0] = v[j].x; row[1] = v[j].y; row[2] = v[j].z; row[3] = v[j].w;
+            }
+        } else {
+            for (int j = 0; j < kEdge; j += 8) {
+                const int64_t r = r0 + sy + j, c = c0 + sx;
+                if (r < rows && c < cols) tile[(sy + j) * kPitch + sx] = in[r * cols + c];
+            }
+        }
+        const uint32_t nxt = q.next();  // a barrier: the tile is in LDS
+        if (nxt < tiles) q.draw_ahead();
+        if (nxt < tiles && whole(nxt)) request(nxt);
+        if (is_whole) {
+#pragma unroll
+            for (int j = 0; j < kEdge / kDown; ++j) {
+                const int c = ty + kDown * j;
+                const f32x4_t o = {tile[(4 * tx + 0) * kPitch + c], tile[(4 * tx + 1) * kPitch + c], tile[(4 * tx + 2) * kPitch + c],
+                                   tile[(4 * tx + 3) * kPitch + c]};
+                __builtin_nontemporal_store(o, reinterpret_cast<f32x4_t *>(out + (c0 + c) * rows + r0 + 4 * tx));
+            }
+        } else {
+            for (int j = 0; j < kEdge; j += 8) {
+                const int64_t c = c0 + sy + j, r = r0 + sx;
+                if (r < rows && c < cols) out[c * rows + r] = tile[sx * kPitch + sy + j];
+            }
+        }
+        __syncthreads();  // everyone has read the tile before the next one is written
+        cur = nxt;
     }
 }
 
@@ -333,16 +403,36 @@ cn_status cn_transpose_f32(const float *in, int64_t rows, int64_t cols, float *o
     CN_REQUIRE(in && out, CN_ERR_NULL, "transpose_f32: NULL pointer");
     CN_REQUIRE(in != out, CN_ERR_ARG, "transpose_f32: in-place transpose is not supported");
     CN_ENTER();
-    const int64_t tiles_r = (rows + 63) / 64, tiles64 = tiles_r * ((cols + 63) / 64);
     auto ok16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-    if (tiles64 <= 0x7fffffffLL && rows * cols >= (1 << 16)) {
-        if (ok16(in) && ok16(out) && rows % 4 == 0 && cols % 4 == 0)
-            hipLaunchKernelGGL(transpose64_kernel<true>, dim3((unsigned)tiles64), dim3(kT), 0, st, in, rows, cols, out, tiles_r);
-        else
-            hipLaunchKernelGGL(transpose64_kernel<false>, dim3((unsigned)tiles64), dim3(kT), 0, st, in, rows, cols, out, tiles_r);
+    const bool vec = ok16(in) && ok16(out) && rows % 4 == 0 && cols % 4 == 0;
+    auto tiled = [&](auto kernel, int edge) -> cn_status {
+        const int lds = edge * (edge + 1) * (int)sizeof(float);
+        static OncePerDevice configured[2][2];
+        if (configured[edge == 128][vec].first(ctx->device))
+            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        const int64_t tiles_r = (rows + edge - 1) / edge, tiles = tiles_r * ((cols + edge - 1) / edge);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(edge * edge / 16), lds, st, in, rows, cols, out, tiles_r);
+        CN_HIP(hipGetLastError());
+        return CN_OK;
+    };
+    const int64_t tiles128 = ((rows + 127) / 128) * ((cols + 127) / 128);
+    if (vec && (size_t)rows * (size_t)cols >= kDrawnFrom && tiles128 <= 0x7fffffffLL) {
+        // beyond the cache: a persistent workgroup per compute unit draws the tiles in the same order and has its next
+        // tile's loads in flight while it stores (100000 x 8192: 5.9 TB/s against 5.5 for a workgroup per tile; 20000 x
+        // 40000: 5.8 against 5.5; 8192 x 100096: 6.15 either way; 4096 x 4096: 31 us against 24, hence the bound)
+        const int lds = 128 * 129 * (int)sizeof(float);
+        static OncePerDevice drawn_configured;
+        if (drawn_configured.first(ctx->device))
+            CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&transpose_drawn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        hipLaunchKernelGGL(transpose_drawn_kernel, dim3(ctx->num_cu), dim3(1024), lds, st, in, rows, cols, out, (rows + 127) / 128,
+                           (uint32_t)tiles128, ctx->next_tile_counter());
         CN_HIP(hipGetLastError());
         return CN_OK;
     }
+    if (tiles128 >= 1024 && tiles128 <= 0x7fffffffLL)
+        return vec ? tiled(&transpose_tile_kernel<128, true>, 128) : tiled(&transpose_tile_kernel<128, false>, 128);
+    if (rows * cols >= (1 << 16) && tiles128 <= 0x7fffffffLL / 4)
+        return vec ? tiled(&transpose_tile_kernel<64, true>, 64) : tiled(&transpose_tile_kernel<64, false>, 64);
     int64_t tiles = ((rows + 31) / 32) * ((cols + 31) / 32);
     int64_t cap = (int64_t)ctx->num_cu * 8;
     hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)(tiles < cap ? tiles : cap)), dim3(kT), 0, st, in, rows, cols, out);

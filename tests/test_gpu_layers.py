@@ -427,14 +427,15 @@ def test_fill_on_every_path(dev):
 
 
 def test_transpose_on_every_path(dev):
-    """cn_transpose_f32: small matrices (32 x 32 tiles), whole and ragged 64 x 64 tiles, dimensions that are not
-    multiples of four and starts that are not 16-byte aligned (element-wise tiles), against torch's transposition."""
+    """cn_transpose_f32: small matrices (32 x 32 tiles), whole and ragged 64 x 64 tiles, whole and ragged 128 x 128 tiles
+    (a thousand of them and more), dimensions that are not multiples of four and starts that are not 16-byte aligned
+    (element-wise tiles), against torch's transposition."""
     import torch
     from clusternet_amd import _lib as L
     gen = torch.Generator(device=dev)
     gen.manual_seed(17)
     for r, c in ((1, 1), (3, 5), (63, 65), (64, 64), (128, 784), (1000, 1003), (260, 516), (4096, 4100), (516, 260),
-                 (1024, 4096), (8192, 384)):
+                 (1024, 4096), (8192, 384), (4096, 4096), (5000, 4097), (128, 140000)):
         for off in (0, 1, 4):
             buf = torch.randn(r * c + 8, device=dev, generator=gen)
             A = buf[off:off + r * c].view(r, c)
@@ -443,3 +444,14 @@ def test_transpose_on_every_path(dev):
             L.transpose(A, out)
             assert torch.equal(out, A.t()), (r, c, off)
             assert float(obuf[:off].sum()) == 7.0 * off and float(obuf[off + r * c:].min()) == 7.0, (r, c, off)
+    # beyond 2^26 elements a persistent grid draws 128 x 128 tiles from a counter: whole tiles, ragged ones on either edge,
+    # twice in a row (the second call finds the counter as the first left it)
+    for r, c in ((8320, 8200), (8200, 8320), (8192, 8192)):
+        A = torch.randn((r, c), device=dev, generator=gen)
+        out = torch.empty((c, r), device=dev)
+        for _ in range(2):
+            out.zero_()
+            L.transpose(A, out)
+            assert torch.equal(out, A.t()), (r, c)
+        del A, out
+    assert L.lib().cn_host_tile_counters_in_use() == 0
