@@ -125,15 +125,20 @@ constexpr int64_t kScanBlock = 4096;
 
 __global__ __launch_bounds__(kT) void block_sums_kernel(const int32_t *__restrict__ counts, int64_t n,
                                                         int32_t *__restrict__ sums) {
-    __shared__ int partial[kT / 64];
+    // A block's sum is carried in 64 bits and stored as at most INT32_MAX: a block that large makes the total reach
+    // INT32_MAX, which every caller refuses, instead of wrapping round to a small number that would pass.
+    __shared__ long long partial[kT / 64];
     const int64_t i0 = (int64_t)blockIdx.x * kScanBlock;
     const int64_t i1 = (i0 + kScanBlock < n) ? i0 + kScanBlock : n;
-    int c = 0;
+    long long c = 0;
     for (int64_t i = i0 + threadIdx.x; i < i1; i += kT) c += counts[i];
     for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off, 64);
     if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = c;
     __syncthreads();
-    if (threadIdx.x == 0) sums[blockIdx.x] = partial[0] + partial[1] + partial[2] + partial[3];
+    if (threadIdx.x == 0) {
+        const long long sum = partial[0] + partial[1] + partial[2] + partial[3];
+        sums[blockIdx.x] = sum > 0x7fffffffLL ? 0x7fffffff : (int32_t)sum;
+    }
 }
 
 __global__ __launch_bounds__(kT) void block_scan_kernel(const int32_t *counts, int64_t n,
@@ -1000,7 +1005,7 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
     }
     CN_HIP(hipMemcpyAsync(nnz_host, total_dev, sizeof(int64_t), hipMemcpyDeviceToHost, st));
     CN_HIP(hipStreamSynchronize(st));
-    if (*nnz_host > 0x7fffffffLL) { set_error("csr_from_dense_f32: more than 2^31 nonzeros"); return CN_ERR_SHAPE; }
+    if (*nnz_host >= 0x7fffffffLL) { set_error("csr_from_dense_f32: 2^31 - 1 nonzeros or more"); return CN_ERR_SHAPE; }
     if (*nnz_host > capacity) {
         set_error("csr_from_dense_f32: %lld nonzeros do not fit the capacity of %lld", (long long)*nnz_host, (long long)capacity);
         return CN_ERR_WORKSPACE;
@@ -1098,6 +1103,19 @@ static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, con
 }
 
 void cn_host_csr_strip_kernel(int enabled) { g_strip_kernel = enabled != 0; }
+
+// Test hook: the exclusive prefix sums the CSR builders use, on a caller's counts.
+cn_status cn_host_exclusive_scan(const int32_t *counts_device, int64_t n, int32_t *sums_device, int64_t *total_host) {
+    if (n < 0 || !total_host || (n > 0 && !counts_device) || !sums_device) { set_error("host_exclusive_scan: bad argument"); return CN_ERR_ARG; }
+    Context *ctx;
+    cn_status s = current_context(&ctx);
+    if (s != CN_OK) return s;
+    int64_t *total_dev = reinterpret_cast<int64_t *>(ctx->sum_scratch);
+    s = exclusive_scan(ctx, counts_device, n, sums_device, total_dev, (hipStream_t)0);
+    if (s != CN_OK) return s;
+    CN_HIP(hipMemcpy(total_host, total_dev, sizeof(int64_t), hipMemcpyDeviceToHost));
+    return CN_OK;
+}
 void cn_host_csr_rows_workgroups_per_cu(int per_cu) { g_rows_per_cu = per_cu > 0 ? per_cu : 0; }
 void cn_host_csr_lds_rows(int enabled) { g_lds_rows = enabled != 0; }
 

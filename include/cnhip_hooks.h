@@ -75,6 +75,11 @@ void cn_host_csr_strip_kernel(int enabled);
 void cn_host_csr_lds_rows(int enabled);
 /* Workgroups per compute unit of the passes that turn a sparse product into codes (and updates); 0 = their own. */
 void cn_host_csr_rows_workgroups_per_cu(int per_cu);
+/* sums_device[0 .. n] = exclusive prefix sums of counts_device[0 .. n - 1] (n + 1 entries; in place allowed) as the CSR
+ * builders form them, *total_host = the sum in 64 bits: exact whatever the entries add up to, and at least 2^31 - 1
+ * whenever they add up to that or more (then the 32-bit prefix sums are not to be used).  Synchronises; returns a
+ * cn_status. */
+int cn_host_exclusive_scan(const int32_t *counts_device, int64_t n, int32_t *sums_device, int64_t *total_host);
 
 /* The encoder's bucket table on the host.  cn_host_xlut_entries: number of 8-byte entries of a table;
  * cn_host_xlut_step_count: number of steps of the code function found at precision 1;

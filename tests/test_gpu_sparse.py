@@ -442,3 +442,37 @@ def test_dense_to_csr_on_random_shapes_strides_and_alignments(dev, seed):
             assert np.array_equal(S.row_ptr.cpu().numpy(), rp), case
             assert np.array_equal(S.col_idx.cpu().numpy(), ci), case
             assert np.array_equal(_bits(S.vals.cpu().numpy()), _bits(va)), case
+
+
+def test_prefix_sums_keep_their_total_in_64_bits(dev):
+    """The CSR builders size their outputs from a prefix sum whose total decides whether the 32-bit row pointers can be
+    used at all.  On synthetic counts: the prefix sums against numpy's on both forms of the scan (one workgroup; block
+    sums, their scan, blocks), the total exact when it passes 2^31 (3e9 from entries of a million and from a million
+    entries), and at least 2^31 - 1 when a single block of 4096 entries alone passes it, so that no overflow can
+    wrap round to a small total that the callers would accept."""
+    import ctypes as C
+    import torch
+    import clusternet_amd as cn
+    L = cn.lib()
+    L.cn_host_exclusive_scan.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.POINTER(C.c_int64)]
+    L.cn_host_exclusive_scan.restype = C.c_int
+
+    def scan(counts):
+        c = torch.from_numpy(counts.astype(np.int32)).to(dev)
+        out = torch.empty(counts.size + 1, dtype=torch.int32, device=dev)
+        total = C.c_int64(-1)
+        assert L.cn_host_exclusive_scan(c.data_ptr(), counts.size, out.data_ptr(), C.byref(total)) == 0
+        return out.cpu().numpy(), total.value
+
+    rng = np.random.default_rng(5)
+    for n in (1, 255, 256, 257, 5000, 8192, 8193, 100_000, 1_000_003):
+        counts = rng.integers(0, 2000, n)
+        sums, total = scan(counts)
+        want = np.concatenate([[0], np.cumsum(counts)])
+        assert total == want[-1] and np.array_equal(sums, want.astype(np.int32)), n
+    assert scan(np.full(3000, 1_000_000))[1] == 3_000_000_000          # one workgroup, entries of a million
+    assert scan(np.full(1_000_000, 3000))[1] == 3_000_000_000          # a million entries through block sums
+    assert scan(np.full(100_000, 600_000))[1] >= 2 ** 31 - 1           # every block of 4096 entries passes 2^31 by itself
+    mixed = np.zeros(50_000, np.int64)
+    mixed[10_000:14_096] = 600_000                                      # one such block among empty ones
+    assert scan(mixed)[1] >= 2 ** 31 - 1
