@@ -205,6 +205,16 @@ def test_gemm_plan_covers_k_and_fits_workspace():
                     assert tile_m == force
                 elif force == 0 and (M <= 64 or small):
                     assert tile_m == (64 if (32 < M <= 64 and not small) else 32)
+                elif force == 0:
+                    # sixteen and more chunks of K on the 128 x 128 tile become 64-row tiles with half as many
+                    ref = (C.c_int64 * 8)()
+                    L.cn_host_plan_gemm(M, N, K, 256, ws, 128, ref)
+                    wide = (C.c_int64 * 8)()
+                    L.cn_host_plan_gemm(M, N, K, 256, ws, 256, wide)
+                    if tile_n == 128 and list(ref)[3] >= 16:
+                        assert tile_m == 64 and splits <= (list(ref)[3] + 1) // 2
+                    else:
+                        assert tile_m == 128
                 else:
                     assert tile_m == 128
                 assert tile_n in (128, 256) and (force in (0, 32, 64) or tile_n == force) and (tile_m == 128 or tile_n == 128)
