@@ -1008,7 +1008,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         if (s != CN_OK) return s;
         return then ? finish_from(C) : CN_OK;
     }
-    GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->plan_bytes, g_force_tile_n);
+    GemmPlan plan = plan_gemm(M, N, K, ctx->num_cu, ctx->plan_bytes, g_force_tile_n, !ta);
     // K not split, whole 128-row tiles and pools of 1, 2 or 4: bias + maxout, or the expansion, happen in the
     // product's own write-out and the product never exists in memory (dot for the forward pass, dotT for the
     // backward one; the other transpositions go through the workspace like ragged shapes).

@@ -62,7 +62,7 @@ int64_t split_limit(int64_t k_iters, int min_iters, double out_bytes, size_t wor
 
 }  // namespace
 
-GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n) {
+GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n, bool a_along_k) {
     GemmPlan p;
     p.tile_m = kTileM;
     p.tiles_m = (M + kTileM - 1) / kTileM;
@@ -114,10 +114,14 @@ GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace
     // of the same length and halve the planes: 128 x 4096 x 8192 in 75.9 us instead of 78.8, 128 x 4096 x 4096 in 42.9
     // instead of 45.2 (with eight chunks the two are level: 128 x 8192 x 4096 73.1 against 74.5, 128 x 8192 x 8192
     // 142.0 against 139.7).
-    if (force_tile_n == 0 && !use_wide && p.splits >= 16) {
+    // Only an even number of chunks halves into the same number of work units (an odd one would add units, and with
+    // them a round: 128 x 3000 x 40000 went from 21 chunks on 504 units to 11 on 528 and from 248 us to 378).
+    // With A stored k by m (Tdot) the 64-row tile reads 256-byte pieces of A and loses what the planes save (128 x 4096 x
+    // 8192: 77.7 us against 75.2), so the rule is for A stored m by k.
+    if (force_tile_n == 0 && a_along_k && !use_wide && p.splits >= 16 && p.splits % 2 == 0) {
         p.tile_m = kTileMMid;
         p.tiles_m = (M + kTileMMid - 1) / kTileMMid;
-        const int64_t half = (p.splits + 1) / 2;
+        const int64_t half = p.splits / 2;
         p.iters_per_split = (p.k_iters + half - 1) / half;
         p.splits = (int)((p.k_iters + p.iters_per_split - 1) / p.iters_per_split);
     }
@@ -127,9 +131,19 @@ GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace
 
 }  // namespace cn
 
+static void report(const cn::GemmPlan &p, int64_t out[8]);
+
+extern "C" void cn_host_plan_gemm_rows_along_k(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes,
+                                               int force_tile_n, int64_t out[8]) {
+    report(cn::plan_gemm(M, N, K, num_cu, workspace_bytes, force_tile_n, true), out);
+}
+
 extern "C" void cn_host_plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes,
                                   int force_tile_n, int64_t out[8]) {
-    cn::GemmPlan p = cn::plan_gemm(M, N, K, num_cu, workspace_bytes, force_tile_n);
+    report(cn::plan_gemm(M, N, K, num_cu, workspace_bytes, force_tile_n, false), out);
+}
+
+static void report(const cn::GemmPlan &p, int64_t out[8]) {
     out[0] = p.tiles_m;
     out[1] = p.tiles_n;
     out[2] = p.k_iters;

@@ -121,7 +121,8 @@ bool gemm_small_applies(int ta, int tb, int64_t M, int64_t N, int64_t K, const f
 cn_status gemm_small(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
                      int64_t ldb, float *C, int64_t ldc, uint32_t *amax, hipStream_t st);
 
-GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n);
+// a_along_k: A is stored m by k (dot, dotT), which lets products with many K chunks take 64-row tiles.
+GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n, bool a_along_k);
 
 constexpr int kTileM = 128;
 constexpr int kTileMLow = 32;      // rows of the tile for products with a handful of rows or little work

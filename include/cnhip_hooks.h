@@ -21,6 +21,10 @@ extern "C" {
  * out = { tiles_m, tiles_n, k_iters, splits, iters_per_split, units, tile_n, tile_m }. */
 void cn_host_plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n,
                        int64_t out[8]);
+/* The same for a product whose A is stored m by k (dot, dotT): where the 128 x 128 tile would need an even number of
+ * sixteen and more K chunks, 64-row tiles with half as many take its place. */
+void cn_host_plan_gemm_rows_along_k(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes,
+                                    int force_tile_n, int64_t out[8]);
 
 /* 0 = the planner chooses the tile; 128 / 256 = that width of the 128-row tile; 32 / 64 = the 32 x 128 /
  * 64 x 128 tile.  Any other value means 0. */

@@ -205,18 +205,18 @@ def test_gemm_plan_covers_k_and_fits_workspace():
                     assert tile_m == force
                 elif force == 0 and (M <= 64 or small):
                     assert tile_m == (64 if (32 < M <= 64 and not small) else 32)
-                elif force == 0:
-                    # sixteen and more chunks of K on the 128 x 128 tile become 64-row tiles with half as many
-                    ref = (C.c_int64 * 8)()
-                    L.cn_host_plan_gemm(M, N, K, 256, ws, 128, ref)
-                    wide = (C.c_int64 * 8)()
-                    L.cn_host_plan_gemm(M, N, K, 256, ws, 256, wide)
-                    if tile_n == 128 and list(ref)[3] >= 16:
-                        assert tile_m == 64 and splits <= (list(ref)[3] + 1) // 2
-                    else:
-                        assert tile_m == 128
                 else:
                     assert tile_m == 128
+                    # with A stored m by k, an even number of sixteen and more chunks on the 128 x 128 tile becomes
+                    # 64-row tiles with half as many: as many work units, K covered as before
+                    along = (C.c_int64 * 8)()
+                    L.cn_host_plan_gemm_rows_along_k(M, N, K, 256, ws, force, along)
+                    a = list(along)
+                    if force == 0 and tile_n == 128 and splits >= 16 and splits % 2 == 0:
+                        assert a[7] == 64 and a[6] == 128 and a[3] == splits // 2 and a[5] == units and a[0] == -(-M // 64)
+                        assert a[4] * a[3] >= a[2] and a[4] * (a[3] - 1) < a[2] and a[3] * M * N * 4 <= ws
+                    else:
+                        assert a == list(out)
                 assert tile_n in (128, 256) and (force in (0, 32, 64) or tile_n == force) and (tile_m == 128 or tile_n == 128)
                 assert tm == -(-M // tile_m) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
                 assert splits >= 1 and units == tm * tn * splits
