@@ -184,7 +184,7 @@ def bench_codec(torch, cn, dev):
             res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
         if n >= 100000 * 8192:
             # movers that are not this library's: the runtime's device-to-device copy (above) and its fill, the latter a
-            # pure write stream.  What access patterns reach on this part at all is in profiles/ (stream_sweep).
+            # pure write stream.  What access patterns reach on this part at all is in profiles/stream_patterns_sweep_819M_elements.txt.
             t_fill = time_region(torch, lambda: back.fill_(1.0), iters, warm)
             res[name]["fill_GBps"] = 4.0 * n / t_fill / 1e6
         del x, codes, back

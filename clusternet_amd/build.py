@@ -1,6 +1,6 @@
 """Compiles the HIP sources under clusternet_amd/csrc into clusternet_amd/libcnhip.so (gfx950).
 
-Usage: python -m clusternet_amd.build [--facade] [--stream-sweep] | --host-asan
+Usage: python -m clusternet_amd.build [--facade] | --host-asan
 The library is built in-tree so that it travels with the source tree; nothing is installed.
 """
 import os
@@ -80,30 +80,6 @@ def build_facade(verbose=False):
     return FACADE_LIB
 
 
-def build_stream_sweep(verbose=False):
-    """The stand-alone measurement program under csrc/stream_sweep (not part of the library)."""
-    d = os.path.join(CSRC, "stream_sweep")
-    objdir = os.path.join(HERE, "build")
-    os.makedirs(objdir, exist_ok=True)
-    flags = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-             "-Wno-unused-command-line-argument"]
-    procs, objs = [], []
-    for kind in range(7):
-        obj = os.path.join(objdir, "stream_sweep_kind%d.o" % kind)
-        objs.append(obj)
-        procs.append(subprocess.Popen([hipcc()] + flags + ["-DSWEEP_KIND=%d" % kind, "-c", os.path.join(d, "kind.hip"), "-o", obj],
-                                      stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
-    main_obj = os.path.join(objdir, "stream_sweep_main.o")
-    _run([hipcc()] + flags + ["-c", os.path.join(d, "main.hip"), "-o", main_obj])
-    for p in procs:
-        out, _ = p.communicate()
-        if p.returncode != 0:
-            raise RuntimeError("build failed: stream_sweep\n%s" % out)
-    exe = os.path.join(HERE, "stream_sweep")
-    _run([hipcc(), "--offload-arch=" + ARCH, "-o", exe, main_obj] + objs)
-    return exe
-
-
 def host_asan(verbose=True):
     """CPU only: the host code of the library and the CPU checker under AddressSanitizer + UndefinedBehavior-
     Sanitizer, and the CPU tests that exercise them run once against those builds.  Device code is compiled as
@@ -161,8 +137,6 @@ def main(argv=None):
     print(build_library(verbose=True))
     if "--facade" in argv:
         print(build_facade(verbose=True))
-    if "--stream-sweep" in argv:
-        print(build_stream_sweep(verbose=True))
     if "--host-asan" in argv:
         print(host_asan())
 
