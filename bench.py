@@ -10,7 +10,7 @@ against the fp32 matrix-core peak.  After the timed region the codec kernels (co
 decompression_8bit, absmax) and the fused 8-bit-weight GEMM are measured on their own workloads and
 reported under "extra"; the CPU port of the same arithmetic is timed on a bounded sample.
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|codec|fused|step] [--no-cpu] [--zero-operands]
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--only gemm|codec|fused|step|products] [--no-cpu] [--zero-operands]
 """
 import argparse
 import json
@@ -377,6 +377,48 @@ def bench_step(torch, cn, dev):
     return out
 
 
+def bench_products(torch, cn, dev):
+    """The backward products of the maxout training step one by one at their full shapes, each on its own (the step's
+    phases above time several kernels together): the second layer's input gradient dotT 128 x 4096 x 8192, the first
+    layer's weight gradient Tdot 100000 x 8192 x 128, and the first layer's input gradient dotT 128 x 100000 x 8192
+    (reads all of W1).  Every call is timed by its own pair of events; mean, median and minimum are reported."""
+    gen = torch.Generator(device=dev).manual_seed(21)
+    B, D, H = 128, 100000, 8192
+    X = torch.rand((B, D), device=dev, generator=gen)
+    E = torch.empty((B, H), device=dev).normal_(0.0, 0.01, generator=gen)
+    W2 = make_uniform(torch, (H // 2, H), (6.0 / (H // 2 + H)) ** 0.5, dev, gen)
+    W1 = make_uniform(torch, (D, H), (6.0 / (D + H)) ** 0.5, dev, gen)
+    out = {}
+    for name, a, b, ta, tb, shape, iters in (("dotT_128x4096x8192", E, W2, False, True, (B, H // 2), 200),
+                                             ("Tdot_100000x8192x128", X, E, True, False, (D, H), 20),
+                                             ("dotT_128x100000x8192", E, W1, False, True, (B, D), 20)):
+        C = torch.empty(shape, device=dev)
+        flop = 2.0 * C.shape[0] * C.shape[1] * (a.shape[0] if ta else a.shape[1])
+        fn = lambda: cn.gemm(a, b, ta, tb, out=C)
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        ev = [event_pair(torch) for _ in range(iters)]
+        for s, e in ev:
+            s.record()
+            fn()
+            e.record()
+        torch.cuda.synchronize()
+        ts = sorted(s.elapsed_time(e) for s, e in ev)
+        mean, med, mn = sum(ts) / len(ts), ts[len(ts) // 2], ts[0]
+        rec = {"mean_us": mean * 1e3, "median_us": med * 1e3, "min_us": mn * 1e3,
+               "TFLOPs": flop / (med * 1e-3) / 1e12, "frac_mfma_peak": flop / (med * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+               "timing": "an event pair round every call, %d calls; TFLOPs from the median" % iters}
+        if C.numel() * 4 < (64 << 20):
+            t = time_replayed(torch, fn, 20, 20)
+            if t is not None:
+                rec["replayed_from_a_graph_us"] = t * 1e3
+                rec["replayed_frac_mfma_peak"] = flop / (t * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS
+        out[name] = rec
+        del C
+    return out
+
+
 def cpu_baseline(torch, tensors):
     """The CPU port (oracle/cpu_port.c, all OpenMP threads) on a column sample of the first dot,
     repeated until about ten seconds of CPU work have been timed."""
@@ -417,7 +459,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--only", choices=["gemm", "codec", "fused", "step"], default=None,
+    ap.add_argument("--only", choices=["gemm", "codec", "fused", "step", "products"], default=None,
                     help="run one part only (for profiling); prints a reduced JSON line")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--zero-operands", action="store_true",
@@ -484,6 +526,9 @@ def main():
         torch.cuda.empty_cache()
     if args.only in (None, "fused"):
         section("fused_w8_gemm_4096x4096", lambda: bench_fused(torch, cn, dev))
+    if args.only in (None, "products"):
+        torch.cuda.empty_cache()
+        section("maxout_step_backward_products", lambda: bench_products(torch, cn, dev))
     if args.only in (None, "step"):
         torch.cuda.empty_cache()
         section("maxout_step_128x100000_8192_8192_10", lambda: bench_step(torch, cn, dev))

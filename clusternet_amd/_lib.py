@@ -93,6 +93,10 @@ def lib():
     L.cn_host_gemm_w8_rows.restype = None
     L.cn_host_gemm_small.argtypes = [C.c_int]
     L.cn_host_gemm_small.restype = None
+    L.cn_host_gemm_persistent.argtypes = [C.c_int]
+    L.cn_host_gemm_persistent.restype = None
+    L.cn_host_last_gemm_kernel.argtypes = [C.c_void_p]
+    L.cn_host_last_gemm_kernel.restype = C.c_int
     L.cn_host_tile_counters_in_use.argtypes = []
     L.cn_host_tile_counters_in_use.restype = C.c_int
     L.cn_host_reduction_fences.argtypes = [C.c_int]

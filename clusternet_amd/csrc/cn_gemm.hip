@@ -62,6 +62,8 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *p) {
 constexpr int NT = 256;  // lanes per workgroup
 constexpr int NW = 4;    // wavefronts per workgroup
 constexpr int kNumXcd = 8;
+constexpr int kPersistentFromRounds = 3;   // rounds of resident workgroups from which an unsplit product keeps its workgroups ...
+constexpr int kPersistentMaxStages = 32;   // ... if a tile has no more stages than this
 
 // What the B operand is.
 enum BKind { B_IC = 0 /* fp32 [k][n] */, B_KC = 1 /* fp32 [n][k] */, B_CODES = 2 /* uint8 [k][n] */ };
@@ -91,6 +93,7 @@ struct GemmArgs {
     float scale;         // fused: decode scale
     const float *table;  // fused: 126-entry codebook
     uint32_t *amax;      // optional: receives max |C| as the bit pattern of a non-negative float
+    uint32_t *tile_counter;  // persistent form: the counter its workgroups draw their tiles from (0 between kernels), or NULL
     int units_in_order;  // work units in block-id order (one window of C in flight) instead of a contiguous slice per XCD
     int wide_store;      // the destination of the write-out (C, or the partial planes) allows 16-byte stores
     // What the write-out does instead of storing C when the kernel is instantiated with an epilogue (whole tiles
@@ -764,6 +767,274 @@ __global__ __launch_bounds__(NT, 2) void gemm_kernel(GemmArgs g) {
     if (want_amax) publish_absmax(amax, g.amax);
 }
 
+// ---- unsplit products of many short tiles: persistent workgroups ------------------------------------------------
+// A product whose K is not split and short (the weight gradient of a wide layer: K is the batch) and whose tiles are
+// many more than the chip holds at once spends a good part of every tile outside the matrix pipe: a workgroup is
+// started, works out its addresses, waits for its first stage, and at the end writes 128 KB out.  Here two workgroups
+// per compute unit stay for the whole product and draw their tiles from a counter: the stages of consecutive tiles form
+// one pipeline (the load issued during a tile's last stage is the first stage of the next tile), fragment reads run a
+// group of 8 k ahead of the MFMAs, and a tile is written out straight from the accumulators while its successor's
+// first stage is already in LDS.  Whole K stages and 16-byte operands only (the host checks; ragged tiles at the border of
+// C are written element by element); same MFMA order per tile as gemm_kernel, so the same bits.
+template <bool A_KC, bool B_IS_KC, int TN>
+__global__ __launch_bounds__(NT, 2) void gemm_persistent_kernel(GemmArgs g) {
+    using G = Geo<128, TN>;
+    constexpr int BM = 128, BN = TN, BK = G::BK, FM = G::FM, FN = G::FN;
+    constexpr int kGroups = BK / 8;
+    constexpr int kAStage = BM * BK, kBStage = TN * BK;
+    static_assert(G::NST == 2, "two LDS stages");
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    float *sA = smem;
+    float *sB = smem + 2 * kAStage;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wave_m = wave / G::WN, wave_n = wave % G::WN;
+    const int half = lane >> 5, l32 = lane & 31;
+    int row_a[FM], row_b[FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) row_a[i] = wave_m * (32 * FM) + i * 32 + l32;
+#pragma unroll
+    for (int i = 0; i < FN; ++i) row_b[i] = wave_n * (32 * FN) + i * 32 + l32;
+
+    f32x16 acc[FM][FN];
+    auto clear = [&]() {
+#pragma unroll
+        for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.0f;
+    };
+    clear();
+
+    const float *Bf = reinterpret_cast<const float *>(g.B);
+    const int64_t end_a = A_KC ? (g.M - 1) * g.lda + g.K : (g.K - 1) * g.lda + ((g.M + 3) & ~(int64_t)3);
+    const int64_t end_b = B_IS_KC ? (g.N - 1) * g.ldb + g.K : (g.K - 1) * g.ldb + ((g.N + 3) & ~(int64_t)3);
+    DirectLoader<A_KC, BM, BK> da;
+    DirectLoader<B_IS_KC, TN, BK> db;
+    da.init(g.lda, wave);
+    db.init(g.ldb, wave);
+    // The stage to be requested next: corner addresses of its A and B pieces and the bytes from each corner to the end
+    // of its matrix (the descriptor's range: rows of a ragged tile that lie outside the matrix read zeros instead of
+    // memory).  Kept as running values, a few scalar additions per stage: the loop has nothing else to work out.
+    const float *next_a, *next_b;
+    int64_t left_a, left_b;
+    constexpr int64_t kOne = 1;
+    const int64_t step_a = A_KC ? (int64_t)BK : (int64_t)BK * g.lda, step_b = B_IS_KC ? (int64_t)BK : (int64_t)BK * g.ldb;
+    auto first_stage_of = [&](int64_t m0, int64_t n0) {
+        next_a = A_KC ? g.A + m0 * g.lda : g.A + m0;
+        next_b = B_IS_KC ? Bf + n0 * g.ldb : Bf + n0;
+        left_a = (end_a - (next_a - g.A)) * 4;  // positive: the corner of a tile lies inside its matrix
+        left_b = (end_b - (next_b - Bf)) * 4;
+    };
+    // Requests that stage into LDS stage `slot` and moves on to the one behind it; not `live`: the same loads with a
+    // range of zero bytes (they touch no memory), so that the code is straight-line and its waits can count.
+    auto issue_next = [&](int slot, bool live) {
+        const uint32_t la = !live ? 0u : ((uint64_t)left_a >> 32) != 0 ? 0xffffffffu : (uint32_t)left_a;
+        const uint32_t lb = !live ? 0u : ((uint64_t)left_b >> 32) != 0 ? 0xffffffffu : (uint32_t)left_b;
+        da.issue(next_a, la, sA + slot * kAStage, wave);
+        db.issue(next_b, lb, sB + slot * kBStage, wave);
+        next_a += step_a; left_a -= step_a * 4;
+        next_b += step_b; left_b -= step_b * 4;
+        (void)kOne;
+    };
+    auto load_frag = [&](const float *pa, const float *pb, int gq, f32x4 (&a)[FM], f32x4 (&b)[FN]) {
+#pragma unroll
+        for (int i = 0; i < FM; ++i) {
+            if (A_KC) {
+                a[i] = *reinterpret_cast<const f32x4 *>(pa + lds_offset<BK>(row_a[i], 2 * gq + half));
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) a[i][s] = pa[(8 * gq + 4 * half + s) * BM + row_a[i]];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < FN; ++i) {
+            if (B_IS_KC) {
+                b[i] = *reinterpret_cast<const f32x4 *>(pb + lds_offset<BK>(row_b[i], 2 * gq + half));
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) b[i][s] = pb[(8 * gq + 4 * half + s) * TN + row_b[i]];
+            }
+        }
+    };
+    auto mfma_steps = [&](const f32x4 (&a)[FM], const f32x4 (&b)[FN], int s_begin, int s_end) {
+#pragma unroll
+        for (int s = s_begin; s < s_end; ++s)
+#pragma unroll
+            for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < FN; ++ni)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi][s], b[ni][s], acc[mi][ni], 0, 0, 0);
+    };
+    constexpr int kTailFrom = 4 - 8 / (FM * FN);
+    // Fragment reads run one group of 8 k ahead of the MFMAs, in two register sets that alternate: on entry to a stage
+    // the first set holds (or is receiving) group 0, requested behind the barrier that published the stage, in the
+    // shadow of the previous stage's last eight MFMAs.  A wavefront that has its SIMD to itself (its neighbour of the
+    // other workgroup is writing a tile out) then waits for LDS once per stage at most, not once per handful of MFMAs.
+    f32x4 a0[FM], b0[FN], a1[FM], b1[FN];
+    static_assert(kGroups == 2 || kGroups == 4, "two register sets, even number of groups");
+    auto stage_head = [&](const float *pa, const float *pb) {
+        load_frag(pa, pb, 1, a1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_steps(a0, b0, 0, 4);
+        if (kGroups == 4) {
+            __builtin_amdgcn_sched_barrier(0);
+            load_frag(pa, pb, 2, a0, b0);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_steps(a1, b1, 0, 4);
+            __builtin_amdgcn_sched_barrier(0);
+            load_frag(pa, pb, 3, a1, b1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_steps(a0, b0, 0, 4);
+        }
+        mfma_steps(a1, b1, 0, kTailFrom);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // Behind the barrier: group 0 of the stage just published, then the last eight MFMAs of the stage before it.
+    auto stage_tail = [&](const float *pa_next, const float *pb_next) {
+        load_frag(pa_next, pb_next, 0, a0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_steps(a1, b1, kTailFrom, 4);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    const uint32_t U = g.units, tiles_n32 = (uint32_t)g.tiles_n;
+    const int iters = (int)g.k_iters;
+    auto corner_of = [&](uint32_t unit, int64_t &m0, int64_t &n0) {
+        const uint32_t tm = unit / tiles_n32, tn = unit - tm * tiles_n32;
+        m0 = (int64_t)__builtin_amdgcn_readfirstlane((int)tm) * BM;
+        n0 = (int64_t)__builtin_amdgcn_readfirstlane((int)tn) * BN;
+    };
+    uint32_t amax = 0;
+
+    // The first tile of a workgroup is its block id (the grid is never larger than the number of tiles); the others
+    // are drawn from a counter, whichever workgroup is free taking the next one: two workgroups that share the SIMDs of
+    // a compute unit do not advance at the same pace, and with a fixed share of the tiles the slower ones would finish
+    // long after the faster.  Lane 0 draws the next tile at the top of the current one; the ticket travels during the
+    // tile's first stage, is handed to the other wavefronts through LDS at that stage's barrier, and is needed in the
+    // last stage, where the next tile's first stage is requested (so tiles of a single stage do not draw).  Every
+    // workgroup draws until its first ticket past the last tile, so exactly U tickets are drawn, and whoever holds
+    // the last of them puts the counter back to 0 (nobody draws after it).  Without a counter: tiles bid, bid + grid, ...
+    uint32_t *ticket_slot = reinterpret_cast<uint32_t *>(smem + 2 * (kAStage + kBStage));
+    // The counter's address passes through a register the compiler knows nothing about: a plain atomic on a uniform
+    // address is rewritten into a reduction over the wavefront whose result is waited for on the spot, and the point
+    // here is that nobody waits for the ticket.
+    uint32_t *counter = g.tile_counter;
+    const bool drawing = g.tile_counter != nullptr && iters >= 2;
+    if (drawing) {
+        uint32_t opaque_zero;
+        asm volatile("v_mov_b32 %0, 0" : "=v"(opaque_zero));
+        counter += opaque_zero;
+    }
+    uint32_t drawn = 0;  // lane 0: the raw ticket on its way (tile = gridDim.x + ticket)
+    uint32_t unit = blockIdx.x;
+    int64_t m0, n0;
+    corner_of(unit, m0, n0);
+    first_stage_of(m0, n0);
+    issue_next(0, true);
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    load_frag(sA, sB, 0, a0, b0);
+    int slot = 0;
+    for (;;) {
+        if (drawing && threadIdx.x == 0) drawn = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        uint32_t unit_next = unit + gridDim.x;
+        // all stages but the last: the stage requested is the next one of this tile
+        for (int it = 1; it < iters; ++it) {
+            issue_next(slot ^ 1, true);
+            stage_head(sA + slot * kAStage, sB + slot * kBStage);
+            // the next stage has landed (and the stores of the tile before this one have been acknowledged, and the
+            // ticket has come back)
+            __builtin_amdgcn_s_waitcnt(0x0f70);
+            if (drawing && it == 1 && threadIdx.x == 0) {
+                if (drawn == U - 1u) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                *ticket_slot = drawn + gridDim.x;
+            }
+            __syncthreads();
+            slot ^= 1;
+            stage_tail(sA + slot * kAStage, sB + slot * kBStage);
+        }
+        // the last stage: the stage requested is the first of the next tile.  The slot is not written again before
+        // the first barrier of the next tile's second stage, which lies behind this read for every wavefront.
+        if (drawing) unit_next = (uint32_t)__builtin_amdgcn_readfirstlane((int)*ticket_slot);
+        const bool more = unit_next < U;
+        int64_t m1 = m0, n1 = n0;
+        if (more) corner_of(unit_next, m1, n1);
+        first_stage_of(m1, n1);
+        issue_next(slot ^ 1, more);
+        stage_head(sA + slot * kAStage, sB + slot * kBStage);
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        slot ^= 1;
+        stage_tail(sA + slot * kAStage, sB + slot * kBStage);  // the next tile's first stage (stale data if there is none)
+        // Write-out.  Accumulator r of a lane is row 8 (r / 4) + 4 half + (r % 4), column l32 of its 32 x 32 block: for a
+        // fixed r the 32 lanes of a half write 128 contiguous bytes.  A whole tile leaves as 4-byte stores straight from
+        // the accumulators: the lane's part of the address is one register for the whole tile, the row's part travels in
+        // a scalar register, so a store reads two vector registers and nothing passes through LDS (a pass through LDS
+        // patches, which turns the 128 stores of a wavefront into 32 of 16 bytes, cost this product more than it saved:
+        // a tile is only eight stages long).
+        const bool want_amax = g.amax != nullptr;
+        if (m0 + BM <= g.M && n0 + BN <= g.N) {
+            const rsrc_t out = make_rsrc(g.C + m0 * g.ldc + n0);
+            const uint32_t ldc_bytes = (uint32_t)g.ldc * 4u;
+            const uint32_t mine = (uint32_t)(4 * half) * ldc_bytes + (uint32_t)(wave_n * (32 * FN) + l32) * 4u;
+            // the row's offset is a running scalar (kept opaque, or the compiler works out all 64 ahead and parks them
+            // in a vector register for want of scalar ones); the two blocks of a row differ by an immediate
+            uint32_t row_bytes = (uint32_t)(wave_m * (32 * FM)) * ldc_bytes;
+#pragma unroll
+            for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        asm volatile("" : "+s"(row_bytes));
+#pragma unroll
+                        for (int ni = 0; ni < FN; ++ni) {
+                            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(acc[mi][ni][4 * q + i]), out, mine + (uint32_t)(ni * 32 * 4),
+                                                                  row_bytes, 2 /* nt */);
+                        }
+                        row_bytes += ldc_bytes;
+                    }
+                    row_bytes += 4u * ldc_bytes;  // the other lane half's four rows
+                }
+            if (want_amax) {
+#pragma unroll
+                for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < FN; ++ni)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const uint32_t bits = __float_as_uint(acc[mi][ni][r]) & 0x7fffffffu;
+                            amax = bits > amax ? bits : amax;
+                        }
+            }
+        } else {
+#pragma unroll
+            for (int mi = 0; mi < FM; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < FN; ++ni) {
+                    const int64_t col = n0 + wave_n * (32 * FN) + ni * 32 + l32;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int64_t row = m0 + wave_m * (32 * FM) + mi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                        if (row < g.M && col < g.N) {
+                            g.C[row * g.ldc + col] = acc[mi][ni][r];
+                            const uint32_t bits = __float_as_uint(acc[mi][ni][r]) & 0x7fffffffu;
+                            amax = bits > amax ? bits : amax;
+                        }
+                    }
+                }
+        }
+        if (!more) break;
+        clear();
+        unit = unit_next;
+        m0 = m1;
+        n0 = n1;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the zero-range loads behind the last stage
+    if (g.amax != nullptr) publish_absmax(amax, g.amax);
+}
+
 // C[m][n] = sum over chunks of partial[chunk][m][n], chunks added in ascending order.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float *__restrict__ partial, int splits,
                                                             int64_t M, int64_t N, float *__restrict__ C,
@@ -919,10 +1190,35 @@ static cn_status launch(const GemmArgs &args, const GemmPlan &plan, int device, 
                               : launch_tile<A_KC, B_KIND, 128, kTileM>(args, device, st);
 }
 
+template <bool A_KC, bool B_IS_KC, int TN>
+static cn_status launch_persistent_tile(const GemmArgs &args, int num_cu, int device, hipStream_t st) {
+    using G = Geo<128, TN>;
+    const size_t lds = (size_t)(2 * (128 + TN) * G::BK + 4) * sizeof(float);  // the stages and the ticket word
+    static OncePerDevice configured;
+    if (configured.first(device)) {
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_persistent_kernel<A_KC, B_IS_KC, TN>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    }
+    const uint32_t slots = (uint32_t)num_cu * 2u;
+    hipLaunchKernelGGL((gemm_persistent_kernel<A_KC, B_IS_KC, TN>), dim3(args.units < slots ? args.units : slots), dim3(NT), lds, st, args);
+    CN_HIP(hipGetLastError());
+    return CN_OK;
+}
+
+template <bool A_KC, bool B_IS_KC>
+static cn_status launch_persistent(const GemmArgs &args, int tile_n, int num_cu, int device, hipStream_t st) {
+    return tile_n == 256 ? launch_persistent_tile<A_KC, B_IS_KC, 256>(args, num_cu, device, st)
+                         : launch_persistent_tile<A_KC, B_IS_KC, 128>(args, num_cu, device, st);
+}
+
 static int g_force_tile_n = 0;
 static bool g_wide_store = true;
 static bool g_w8_rows = true;  // test hook: false keeps the tiled kernel for every product on 8-bit weights
 static bool g_small = true;    // test hook: false keeps the tiled kernel for small products too
+static bool g_persistent = true;  // test hook: false starts a workgroup per tile for every product
+// Which kernel family the last product took and how many K chunks it had (test hook cn_host_last_gemm_kernel).
+enum { kTookNone = 0, kTookTiled = 1, kTookSmall = 2, kTookW8Rows = 3, kTookPersistent = 4 };
+static int g_last_kernel = kTookNone, g_last_splits = 0;
 static bool g_epilogue_in_kernel = true;  // test hook: false sends every fused product through the workspace
 
 // What follows the product instead of its delivery: bias and maxout (the forward pass of a maxout layer; `bias`
@@ -959,11 +1255,13 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     if ((M > 0 && N > 0) && ((!C && !then) || (K > 0 && (!A || !B)))) { set_error("%s: NULL operand", who); return CN_ERR_NULL; }
     cn_status s = CN_OK;
     GemmEnv from_context;
+    Context *context = nullptr;
     if (!given) {
         Context *c;
         s = current_context(&c);
         if (s != CN_OK) return s;
         from_context = GemmEnv{c->device, c->num_cu, c->workspace, c->workspace_bytes, c->workspace_bytes, c->table};
+        context = c;
     }
     const GemmEnv *ctx = given ? given : &from_context;
     hipStream_t st = (hipStream_t)stream;
@@ -990,6 +1288,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
         // up to 1024 rows: the kernel that decodes straight into the matrix instruction's registers
         const int chunks = gemm_w8_rows_splits(M, N, K, A, lda, (const uint8_t *)B, ldb, scale, C, ldc, ctx->num_cu, ctx->workspace_bytes);
         if (chunks > 1 || (chunks == 1 && !amax)) {
+            g_last_kernel = kTookW8Rows; g_last_splits = chunks;
             s = gemm_w8_rows(chunks, M, N, K, A, lda, (const uint8_t *)B, ldb, scale, C, ldc, ctx->table, ctx->workspace, ctx->device, st);
             if (s != CN_OK) return s;
             if (chunks > 1) return add_chunk_planes(ctx->workspace, ctx->num_cu, chunks, M, N, C, ldc, amax, st);
@@ -1004,6 +1303,7 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
             C = (float *)ctx->workspace;
             ldc = N;
         }
+        g_last_kernel = kTookSmall; g_last_splits = 1;
         s = gemm_small(ta, tb, M, N, K, A, lda, (const float *)B, ldb, C, ldc, amax, st);
         if (s != CN_OK) return s;
         return then ? finish_from(C) : CN_OK;
@@ -1049,10 +1349,12 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     a.vec_b = w8 ? (aligned(B, 4) && (ldb % 4 == 0)) : (aligned(B, 16) && (ldb % 4 == 0));
     a.scale = scale; a.table = ctx->table;
     a.amax = amax;
+    a.tile_counter = nullptr;
     a.wide_store = g_wide_store && (plan.splits > 1 ? (N % 4 == 0 && (M * N) % 4 == 0)
                                                      : (aligned(C, 16) && ldc % 4 == 0));
     a.epi_bias = nullptr; a.epi_arg_in = nullptr; a.epi_out = nullptr; a.epi_arg_out = nullptr; a.epi_pool = 1;
     if (in_write_out) {
+        g_last_kernel = kTookTiled; g_last_splits = 1;
         a.wide_store = 1;  // the tiles leave through the LDS patch whatever C would have allowed
         a.epi_pool = then->pool;
         a.epi_out = then->out;
@@ -1065,6 +1367,22 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
                                   : launch_tile<true, B_KC, 128, kTileM, EPI_EXPAND>(a, ctx->device, st);
     }
 
+    // K not split and short, 128-row tiles, several rounds of them, whole K stages, 16-byte operands and a result that
+    // 32-bit offsets reach: the workgroups stay and draw their tiles (100000 x 8192 x 128: 1.61 ms against 1.74 ms; from
+    // about 64 stages per tile on there is nothing left to gain and the workgroup per tile is ahead by a percent).
+    const bool persistent = g_persistent && !w8 && !then && plan.splits == 1 && plan.tile_m == kTileM &&
+                            plan.units >= (int64_t)ctx->num_cu * 2 * kPersistentFromRounds && plan.k_iters <= kPersistentMaxStages &&
+                            a.vec_a && a.vec_b && K % gemm_tile_k(plan.tile_n) == 0 && ldc <= (1 << 22);
+    g_last_kernel = persistent ? kTookPersistent : kTookTiled;
+    g_last_splits = plan.splits;
+    if (persistent) {
+        a.tile_counter = context ? context->next_tile_counter() : nullptr;  // without a context: a fixed share of the tiles each
+        if (!ta && !tb)     s = launch_persistent<true, false>(a, plan.tile_n, ctx->num_cu, ctx->device, st);
+        else if (ta && !tb) s = launch_persistent<false, false>(a, plan.tile_n, ctx->num_cu, ctx->device, st);
+        else if (!ta && tb) s = launch_persistent<true, true>(a, plan.tile_n, ctx->num_cu, ctx->device, st);
+        else                s = launch_persistent<false, true>(a, plan.tile_n, ctx->num_cu, ctx->device, st);
+        return s;
+    }
     if (w8)              s = launch<true, B_CODES>(a, plan, ctx->device, st);
     else if (!ta && !tb) s = launch<true, B_IC>(a, plan, ctx->device, st);
     else if (ta && !tb)  s = launch<false, B_IC>(a, plan, ctx->device, st);
@@ -1131,6 +1449,11 @@ void cn_host_gemm_wide_store(int enabled) { g_wide_store = enabled != 0; }
 // Test hook: 0 = bias + maxout and the maxout expansion never run inside the product's write-out.
 void cn_host_gemm_w8_rows(int enabled) { g_w8_rows = enabled != 0; }
 void cn_host_gemm_small(int enabled) { g_small = enabled != 0; }
+void cn_host_gemm_persistent(int enabled) { g_persistent = enabled != 0; }
+int cn_host_last_gemm_kernel(int *splits) {
+    if (splits) *splits = g_last_splits;
+    return g_last_kernel;
+}
 void cn_host_gemm_epilogue_in_kernel(int enabled) { g_epilogue_in_kernel = enabled != 0; }
 
 // Test and tuning hook: 0 = let the planner choose the tile, 128 / 256 = force that width of the 128-row

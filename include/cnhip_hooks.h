@@ -43,6 +43,13 @@ void cn_host_gemm_w8_rows(int enabled);
  * chip with tiles take the kernel that finishes them in one launch. */
 void cn_host_gemm_small(int enabled);
 void cn_host_gemm_epilogue_in_kernel(int enabled);
+/* 0 starts a workgroup per tile for every product; 1 (default) lets an unsplit product of several rounds of
+ * 128 x 256 tiles keep two workgroups per compute unit that walk the tiles.  Same bits. */
+void cn_host_gemm_persistent(int enabled);
+/* Which kernel the last product of this process took: 0 none yet, 1 the tiled kernel (a workgroup per tile and K chunk),
+ * 2 the one-launch kernel for small products, 3 the kernel that decodes 8-bit weights into registers, 4 the tiled
+ * kernel with persistent workgroups; *splits (if not NULL) receives its number of K chunks. */
+int cn_host_last_gemm_kernel(int *splits);
 
 /* Workgroups per compute unit for the codec and abs-max kernels; 0 = each kernel's own figure. */
 void cn_host_codec_workgroups_per_cu(int per_cu);
