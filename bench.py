@@ -377,18 +377,22 @@ def bench_step(torch, cn, dev):
     return out
 
 
-def bench_products(torch, cn, dev):
+def bench_products(torch, cn, dev, zeros=False):
     """The backward products of the maxout training step one by one at their full shapes, each on its own (the step's
     phases above time several kernels together): the second layer's input gradient dotT 128 x 4096 x 8192, the first
     layer's weight gradient Tdot 100000 x 8192 x 128, and the first layer's input gradient dotT 128 x 100000 x 8192
     (reads all of W1).  Every call is timed by its own pair of events; mean, median and minimum are reported."""
     gen = torch.Generator(device=dev).manual_seed(21)
     B, D, H = 128, 100000, 8192
-    X = torch.rand((B, D), device=dev, generator=gen)
-    E = torch.empty((B, H), device=dev).normal_(0.0, 0.01, generator=gen)
-    W2 = make_uniform(torch, (H // 2, H), (6.0 / (H // 2 + H)) ** 0.5, dev, gen)
-    W1 = make_uniform(torch, (D, H), (6.0 / (D + H)) ** 0.5, dev, gen)
-    out = {}
+    if zeros:  # profiling aid, as for the README pair: what the code can issue, without the power of switching data
+        X, E = torch.zeros((B, D), device=dev), torch.zeros((B, H), device=dev)
+        W2, W1 = torch.zeros((H // 2, H), device=dev), torch.zeros((D, H), device=dev)
+    else:
+        X = torch.rand((B, D), device=dev, generator=gen)
+        E = torch.empty((B, H), device=dev).normal_(0.0, 0.01, generator=gen)
+        W2 = make_uniform(torch, (H // 2, H), (6.0 / (H // 2 + H)) ** 0.5, dev, gen)
+        W1 = make_uniform(torch, (D, H), (6.0 / (D + H)) ** 0.5, dev, gen)
+    out = {"operands": "all zero (profiling aid, not a result)"} if zeros else {}
     for name, a, b, ta, tb, shape, iters in (("dotT_128x4096x8192", E, W2, False, True, (B, H // 2), 200),
                                              ("Tdot_100000x8192x128", X, E, True, False, (D, H), 20),
                                              ("dotT_128x100000x8192", E, W1, False, True, (B, D), 20)):
@@ -528,7 +532,7 @@ def main():
         section("fused_w8_gemm_4096x4096", lambda: bench_fused(torch, cn, dev))
     if args.only in (None, "products"):
         torch.cuda.empty_cache()
-        section("maxout_step_backward_products", lambda: bench_products(torch, cn, dev))
+        section("maxout_step_backward_products", lambda: bench_products(torch, cn, dev, zeros=args.zero_operands))
     if args.only in (None, "step"):
         torch.cuda.empty_cache()
         section("maxout_step_128x100000_8192_8192_10", lambda: bench_step(torch, cn, dev))
