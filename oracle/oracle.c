@@ -255,20 +255,54 @@ void cn_oracle_gemm_f64acc(int ta, int tb, int64_t M, int64_t N, int64_t K, cons
     }
 }
 
-/* Same as above but also returns sum_k |a||b| per output (the forward-error denominator). */
+/* Same as above but also returns sum_k |a||b| per output (the forward-error denominator).
+ * Every output adds its products in ascending k, one rounded fp64 addition each (the products of two floats are
+ * exact in fp64).  With B stored K x N the loops are blocked so that B is streamed by rows once per group of eight
+ * output rows; the order of the additions per output, and so every bit of the result, is that of the plain loops. */
 void cn_oracle_gemm_f64acc_abs(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A,
                                int64_t lda, const float *B, int64_t ldb, double *C, double *Cabs) {
+    if (tb) {
 #pragma omp parallel for schedule(static)
-    for (int64_t m = 0; m < M; ++m) {
-        for (int64_t n = 0; n < N; ++n) {
-            double s = 0.0, sa = 0.0;
-            for (int64_t k = 0; k < K; ++k) {
-                double p = (double)a_at(A, lda, ta, m, k) * (double)b_at(B, ldb, tb, k, n);
-                s += p;
-                sa += fabs(p);
+        for (int64_t m = 0; m < M; ++m) {
+            for (int64_t n = 0; n < N; ++n) {
+                double s = 0.0, sa = 0.0;
+                for (int64_t k = 0; k < K; ++k) {
+                    double p = (double)a_at(A, lda, ta, m, k) * (double)B[n * ldb + k];
+                    s += p;
+                    sa += fabs(p);
+                }
+                C[m * N + n] = s;
+                Cabs[m * N + n] = sa;
             }
-            C[m * N + n] = s;
-            Cabs[m * N + n] = sa;
+        }
+        return;
+    }
+    enum { RB = 8, NB = 2048 };
+    const int64_t groups = (M + RB - 1) / RB, blocks = (N + NB - 1) / NB;
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+    for (int64_t gi = 0; gi < groups; ++gi) {
+        for (int64_t bi = 0; bi < blocks; ++bi) {
+            const int64_t m0 = gi * RB, n0 = bi * NB;
+            const int64_t rows = M - m0 < RB ? M - m0 : RB, cols = N - n0 < NB ? N - n0 : NB;
+            double *acc = (double *)calloc((size_t)(2 * RB * NB), sizeof(double));
+            for (int64_t k = 0; k < K; ++k) {
+                const float *brow = B + k * ldb + n0;
+                for (int64_t r = 0; r < rows; ++r) {
+                    const double av = (double)a_at(A, lda, ta, m0 + r, k);
+                    double *s = acc + (size_t)r * NB, *sa = acc + (size_t)(RB + r) * NB;
+                    for (int64_t n = 0; n < cols; ++n) {
+                        const double p = av * (double)brow[n];
+                        s[n] += p;
+                        sa[n] += fabs(p);
+                    }
+                }
+            }
+            for (int64_t r = 0; r < rows; ++r)
+                for (int64_t n = 0; n < cols; ++n) {
+                    C[(m0 + r) * N + n0 + n] = acc[(size_t)r * NB + n];
+                    Cabs[(m0 + r) * N + n0 + n] = acc[(size_t)(RB + r) * NB + n];
+                }
+            free(acc);
         }
     }
 }

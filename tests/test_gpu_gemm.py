@@ -222,11 +222,14 @@ def test_linearity_and_transpose_identities_large(dev):
     assert float((cT - c1).abs().max()) / scale < gemm_tolerance(20000)
 
 
-def test_config3_full_size_sampled_columns(dev):
-    """README workload on one GPU: 128x100000 . 100000x40000, then . 40000x20000.  All rows and 48
-    sampled columns of each product are recomputed on the CPU in fp64."""
+def test_config3_full_size_sampled_columns(dev, tile_width):
+    """README workload on one GPU: 128x100000 . 100000x40000, then . 40000x20000 (source/clusterNet.cpp:404-461 on the
+    un-sharded operands of README.md:22-32).  Recomputed on the CPU in fp64: all of out2, and of out1 all rows of at
+    least 1024 columns: seven in each of its 157 tiles of 256 columns (every (K-chunk, tile) work unit of the product
+    contributes to some checked entry), both columns either side of every tile border, and the corners."""
     import torch
     import clusternet_amd as cn
+    thorough = tile_width == 0  # the library's own plan; a forced geometry gets a sample of 48 columns of each product
     g = torch.Generator(device=dev).manual_seed(11)
     batch = torch.rand((128, 100000), device=dev, generator=g)
     lim1, lim2 = float(np.sqrt(6.0 / 140000)), float(np.sqrt(6.0 / 60000))
@@ -238,18 +241,59 @@ def test_config3_full_size_sampled_columns(dev):
     out2 = cn.dot(out1, W2)
     assert tuple(out1.shape) == (128, 40000) and tuple(out2.shape) == (128, 20000)
     rng = np.random.default_rng(5)
-    for A, W, out, K in ((batch, W1, out1, 100000), (out1, W2, out2, 40000)):
-        N = W.shape[1]
-        cols = np.unique(np.concatenate([[0, 1, 127, 128, N - 129, N - 128, N - 1], rng.integers(0, N, 41)]))
-        Wc = W[:, torch.from_numpy(cols).to(dev)].contiguous().cpu().numpy()
-        Cref, Cabs = oracle.gemm_with_abs(A.cpu().numpy(), Wc)
-        got = out[:, torch.from_numpy(cols).to(dev)].cpu().numpy()
-        e1, e2 = gemm_errors(got, Cref, Cabs)
-        tol = gemm_tolerance(K)
-        assert e1 <= tol and e2 <= tol, (K, e1, e2, tol)
-    # every column got written: compare column sums against a torch matmul of the column-summed W
+    N1 = 40000
+    borders = np.arange(256, N1, 256)
+    cols = np.unique(np.concatenate([[0, 1, N1 - 2, N1 - 1], borders - 1, borders, borders - 129, borders - 128,
+                                     (np.arange(157)[:, None] * 256 + rng.integers(0, 256, (157, 7))).ravel()]))
+    cols = cols[(cols >= 0) & (cols < N1)]
+    assert cols.size >= 1024
+    if not thorough:
+        cols = np.unique(np.concatenate([[0, 1, 127, 128, N1 - 129, N1 - 128, N1 - 1], rng.integers(0, N1, 41)]))
+    idx = torch.from_numpy(cols).to(dev)
+    Cref, Cabs = oracle.gemm_with_abs(batch.cpu().numpy(), W1[:, idx].contiguous().cpu().numpy())
+    e1, e2 = gemm_errors(out1[:, idx].cpu().numpy(), Cref, Cabs)
+    tol = gemm_tolerance(100000)
+    assert e1 <= tol and e2 <= tol, ("out1", cols.size, e1, e2, tol)
+    # every column got written: compare column sums against a torch matmul of a strided sample
     colsum_ref = batch.double() @ W1[:, ::397].double()
-    assert float((out1[:, ::397].double() - colsum_ref).abs().max()) / float(colsum_ref.abs().max()) < gemm_tolerance(100000)
+    assert float((out1[:, ::397].double() - colsum_ref).abs().max()) / float(colsum_ref.abs().max()) < tol
+    del W1, Cref, Cabs
+    if thorough:
+        Cref, Cabs = oracle.gemm_with_abs(out1.cpu().numpy(), W2.cpu().numpy())
+        got = out2.cpu().numpy()
+    else:
+        idx = torch.from_numpy(np.unique(np.concatenate([[0, 1, 127, 128, 19871, 19872, 19999], rng.integers(0, 20000, 41)]))).to(dev)
+        Cref, Cabs = oracle.gemm_with_abs(out1.cpu().numpy(), W2[:, idx].contiguous().cpu().numpy())
+        got = out2[:, idx].cpu().numpy()
+    e1, e2 = gemm_errors(got, Cref, Cabs)
+    tol = gemm_tolerance(40000)
+    assert e1 <= tol and e2 <= tol, ("out2", e1, e2, tol)
+
+
+def test_first_layer_input_gradient_full_size(dev, tile_width):
+    """dotT 128 x 8192 . (100000 x 8192)^T -> 128 x 100000, the optional product of the training configuration that
+    reads all of W1 (source/clusterNet.cpp:262-284): 1024 sampled columns and the borders of its tiles in fp64."""
+    import torch
+    import clusternet_amd as cn
+    if tile_width != 0:
+        pytest.skip("one run is enough: the library's own plan")
+    g = torch.Generator(device=dev).manual_seed(12)
+    E = torch.empty((128, 8192), device=dev).normal_(0.0, 0.01, generator=g)
+    lim = float(np.sqrt(6.0 / 108192))
+    W1 = (torch.rand((100000, 8192), device=dev, generator=g) * 2 - 1) * lim
+    out = cn.dotT(E, W1)
+    assert tuple(out.shape) == (128, 100000)
+    rng = np.random.default_rng(8)
+    borders = np.arange(256, 100000, 256)
+    cols = np.unique(np.concatenate([[0, 1, 99998, 99999], borders[::8] - 1, borders[::8], rng.integers(0, 100000, 1024)]))
+    idx = torch.from_numpy(cols).to(dev)
+    Cref, Cabs = oracle.gemm_with_abs(E.cpu().numpy(), W1[idx].contiguous().cpu().numpy(), False, True)
+    e1, e2 = gemm_errors(out[:, idx].cpu().numpy(), Cref, Cabs)
+    tol = gemm_tolerance(8192)
+    assert cols.size >= 1024 and e1 <= tol and e2 <= tol, (cols.size, e1, e2, tol)
+    # every column written: a strided sample against torch in fp64
+    ref = E.double() @ W1[::97].double().t()
+    assert float((out[:, ::97].double() - ref).abs().max()) / float(ref.abs().max()) < tol
 
 
 def test_fused_w8_decode_is_bit_identical(dev):

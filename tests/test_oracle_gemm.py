@@ -96,3 +96,16 @@ def test_training_step_helpers_brute_force():
     np.testing.assert_allclose(s.sum(axis=1), 1.0, rtol=1e-6)
     e = np.exp(A.astype(np.float64) - A.max(axis=1, keepdims=True))
     np.testing.assert_allclose(s, e / e.sum(axis=1, keepdims=True), rtol=1e-6)
+
+
+def test_blocked_and_plain_loops_give_the_same_bits():
+    """gemm_with_abs streams B by rows in blocks (B stored K x N); gemm_cols is the plain triple loop.  Every output adds its
+    products in ascending k either way, so the fp64 results must agree bit for bit, also across block borders (8 rows,
+    2048 columns) and for A stored K x M."""
+    rng = np.random.default_rng(21)
+    for M, N, K, ta in ((19, 2051, 300, False), (8, 4100, 33, True), (1, 1, 1, False)):
+        A = rng.normal(size=(K, M) if ta else (M, K)).astype(np.float32)
+        B = rng.normal(size=(K, N)).astype(np.float32)
+        C, Cabs = oracle.gemm_with_abs(A, B, ta, False)
+        P, Pabs = oracle.gemm_cols(A, B, np.arange(N), ta, False)
+        assert np.array_equal(C.view(np.uint64), P.view(np.uint64)) and np.array_equal(Cabs.view(np.uint64), Pabs.view(np.uint64))
