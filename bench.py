@@ -65,10 +65,32 @@ def time_region(torch, fn, iters, warmup):
     return s.elapsed_time(e) / iters  # ms
 
 
-def time_replayed(torch, fn, calls, replays):
+def stats(ts):
+    """mean, median and minimum of a list of times."""
+    ts = sorted(ts)
+    return {"mean": sum(ts) / len(ts), "median": ts[len(ts) // 2], "min": ts[0]}
+
+
+def time_each(torch, fn, iters, warmup):
+    """ms per call from an event pair round every call: {"mean", "median", "min"}.  For calls long enough that the gap
+    a host launch leaves does not matter (tens of microseconds and more)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [event_pair(torch) for _ in range(iters)]
+    for s, e in ev:
+        s.record()
+        fn()
+        e.record()
+    torch.cuda.synchronize()
+    return stats([s.elapsed_time(e) for s, e in ev])
+
+
+def time_replayed(torch, fn, calls, replays, want_stats=False):
     """ms per call with the host out of the way: `calls` calls captured into one HIP graph, the graph
     replayed `replays` times between two events.  For kernels of a few microseconds, where the loop of
-    time_region measures how fast Python can launch.  None if the capture is refused."""
+    time_region measures how fast Python can launch.  Every replay has its own event pair; the mean over the replays
+    (or, want_stats, mean / median / min) is returned.  None if the capture is refused."""
     try:
         fn()
         torch.cuda.synchronize()
@@ -79,13 +101,16 @@ def time_replayed(torch, fn, calls, replays):
         for _ in range(replays):
             graph.replay()
         torch.cuda.synchronize()
-        s, e = event_pair(torch)
-        s.record()
-        for _ in range(replays):
+        ev = [event_pair(torch) for _ in range(replays)]
+        for s, e in ev:
+            s.record()
             graph.replay()
-        e.record()
+            e.record()
         torch.cuda.synchronize()
-        return s.elapsed_time(e) / (calls * replays)
+        st = stats([s.elapsed_time(e) / calls for s, e in ev])
+        if want_stats:
+            return st
+        return st["mean"]
     except Exception:  # noqa: BLE001 - any refusal means "not measured this way"
         torch.cuda.synchronize()
         return None
@@ -125,9 +150,10 @@ def bench_gemm(torch, cn, dev, steps, warmup, zeros=False):
         step(events[i])
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    g1 = sum(e[0].elapsed_time(e[1]) for e in events) / steps
-    g2 = sum(e[1].elapsed_time(e[2]) for e in events) / steps
-    return {"wall_ms": wall_ms, "gemm1_ms": g1, "gemm2_ms": g2,
+    g1 = stats([e[0].elapsed_time(e[1]) for e in events])
+    g2 = stats([e[1].elapsed_time(e[2]) for e in events])
+    pair = stats([e[0].elapsed_time(e[2]) for e in events])
+    return {"wall_ms": wall_ms, "gemm1_ms": g1["mean"], "gemm2_ms": g2["mean"], "gemm1": g1, "gemm2": g2, "pair": pair,
             "tensors": (batch, W1, W2, out1, out2)}
 
 
@@ -147,19 +173,33 @@ def bench_codec(torch, cn, dev):
         codes = torch.empty(n, dtype=torch.uint8, device=dev)
         back = torch.empty(n, device=dev)
         warm = 3 if n >= 100000 * 8192 else 1000  # microsecond kernels: let the clocks come up first
-        t_abs = time_region(torch, lambda: cn.absmax(x, prec_t), iters, warm)
-        t_c = time_region(torch, lambda: cn.compression_8bit(x, prec, codes), iters, warm)
-        t_d = time_region(torch, lambda: cn.decompression_8bit(codes, prec, back), iters, warm)
+        big = n >= 100000 * 8192
+        if big:  # hundreds of microseconds per call: an event pair round every call
+            st_abs = time_each(torch, lambda: cn.absmax(x, prec_t), iters, warm)
+            st_c = time_each(torch, lambda: cn.compression_8bit(x, prec, codes), iters, warm)
+            st_d = time_each(torch, lambda: cn.decompression_8bit(codes, prec, back), iters, warm)
+            t_abs, t_c, t_d = st_abs["median"], st_c["median"], st_d["median"]
+            how = "an event pair round every call, %d calls; figures from the median, mean and min beside it" % iters
+        else:    # microseconds per call: back-to-back launches between two events (mean); medians under replayed_from_a_graph
+            t_abs = time_region(torch, lambda: cn.absmax(x, prec_t), iters, warm)
+            t_c = time_region(torch, lambda: cn.compression_8bit(x, prec, codes), iters, warm)
+            t_d = time_region(torch, lambda: cn.decompression_8bit(codes, prec, back), iters, warm)
+            how = "%d back-to-back calls between two events (mean); per-call medians and minima under replayed_from_a_graph" % iters
         t_copy = time_region(torch, lambda: back.copy_(x), iters, warm)
         res[name] = {
-            "elements": n,
+            "elements": n, "timing": how,
             "absmax_GBps": 4.0 * n / t_abs / 1e6, "absmax_us": t_abs * 1e3,
             "compress_GBps": 5.0 * n / t_c / 1e6, "compress_us": t_c * 1e3,
             "decompress_GBps": 5.0 * n / t_d / 1e6, "decompress_us": t_d * 1e3,
             "copy_GBps": 8.0 * n / t_copy / 1e6,
             "compress_frac_hbm_peak": 5.0 * n / t_c / 1e6 / PEAK_HBM_GBPS,
             "decompress_frac_hbm_peak": 5.0 * n / t_d / 1e6 / PEAK_HBM_GBPS,
+            "absmax_frac_hbm_peak": 4.0 * n / t_abs / 1e6 / PEAK_HBM_GBPS,
         }
+        if big:
+            for key, st in (("absmax", st_abs), ("compress", st_c), ("decompress", st_d)):
+                res[name][key + "_us_mean"] = st["mean"] * 1e3
+                res[name][key + "_us_min"] = st["min"] * 1e3
         if n < 100000 * 8192:
             # small buffers: the kernels take a few microseconds, so also time them replayed from a graph
             replayed = {"absmax_us": time_replayed(torch, lambda: cn.absmax(x, prec_t), 20, 50),
@@ -182,6 +222,11 @@ def bench_codec(torch, cn, dev):
                 replayed[label] = time_replayed(torch, lambda: cn.compression_8bit(x, prec_t, codes), 20, 50)
                 cn.lib().cn_host_codec_encoder(0)
             res[name]["replayed_from_a_graph"] = {k: (v * 1e3 if v is not None else None) for k, v in replayed.items()}
+            for key, fn in (("absmax", lambda: cn.absmax(x, prec_t)), ("compress", lambda: cn.compression_8bit(x, prec_t, codes)),
+                            ("decompress", lambda: cn.decompression_8bit(codes, prec_t, back))):
+                st = time_replayed(torch, fn, 20, 50, want_stats=True)
+                if st is not None:
+                    res[name]["replayed_from_a_graph"][key + "_us_median_min"] = [st["median"] * 1e3, st["min"] * 1e3]
         if n >= 100000 * 8192:
             # movers that are not this library's: the runtime's device-to-device copy (above) and its fill, the latter a
             # pure write stream.  What access patterns reach on this part at all is in profiles/stream_patterns_sweep_819M_elements.txt.
@@ -204,11 +249,13 @@ def bench_cfg1(torch, cn, dev):
                             ("Tdot_784x1024x128", lambda c: cn.gemm(A, dC, True, False, out=c), (784, 1024)),
                             ("dotT_128x784x1024", lambda c: cn.gemm(dC, W, False, True, out=c), (128, 784))):
         C = torch.empty(shape, device=dev)
-        t = time_replayed(torch, lambda: fn(C), 20, 50)
-        how = "replayed from a graph"
-        if t is None:
-            t, how = time_region(torch, lambda: fn(C), 200, 1000), "launched one by one"
-        out[name] = {"us": t * 1e3, "TFLOPs": 2.0 * 128 * 784 * 1024 / t / 1e9, "timing": how}
+        st = time_replayed(torch, lambda: fn(C), 20, 50, want_stats=True)
+        how = "replayed from a graph, 50 replays of 20 calls"
+        if st is None:
+            st, how = time_each(torch, lambda: fn(C), 200, 1000), "launched one by one"
+        t = st["median"]
+        out[name] = {"us": t * 1e3, "us_mean": st["mean"] * 1e3, "us_min": st["min"] * 1e3,
+                     "TFLOPs": 2.0 * 128 * 784 * 1024 / t / 1e9, "timing": how + "; figures from the median"}
     return out
 
 
@@ -255,7 +302,13 @@ def bench_fused(torch, cn, dev):
         t_g = time_region(torch, lambda: cn.dot(A, Wd, C), 200, 5)
         res["batch%d" % b] = {"fused_us": t_f * 1e3, "decompress_plus_dot_us": t_u * 1e3,
                               "dot_fp32_only_us": t_g * 1e3, "speedup": t_u / t_f,
-                              "fused_TFLOPs": 2.0 * b * 4096 * 4096 / t_f / 1e9}
+                              "fused_TFLOPs": 2.0 * b * 4096 * 4096 / t_f / 1e9,
+                              "timing": "200 back-to-back calls between two events (mean); replayed: 50 replays of a graph of 20 calls, "
+                                        "[median, min] per call"}
+        for key, fn in (("fused", lambda: cn.gemm_w8(A, codes, scale, C)), ("decompress_plus_dot", unfused)):
+            st = time_replayed(torch, fn, 20, 50, want_stats=True)
+            if st is not None:
+                res["batch%d" % b][key + "_us_replayed_median_min"] = [st["median"] * 1e3, st["min"] * 1e3]
         # these batches take the kernel that decodes into registers; the tiled kernel it replaces there, for comparison
         cn.lib().cn_host_gemm_w8_rows(0)
         res["batch%d" % b]["fused_tiled_kernel_us"] = time_region(torch, lambda: cn.gemm_w8(A, codes, scale, C), 200, 5) * 1e3
@@ -355,7 +408,9 @@ def bench_step(torch, cn, dev):
                      ("codec_and_update_unfused", codec_update_unfused), ("codec_and_rmsprop", codec_rmsprop),
                      ("codec_and_rmsprop_unfused", codec_rmsprop_unfused),
                      ("first_layer_codes_and_rmsprop_sparse", first_layer_rmsprop)):
-        out[name + "_ms"] = time_region(torch, fn, 5, 2)
+        st = time_each(torch, fn, 7, 2)
+        out[name + "_ms"] = st["median"]
+        out[name + "_ms_mean_min"] = [st["mean"], st["min"]]
     flop_f = 2.0 * B * (D * H + (H // pool) * H + (H // pool) * C)
     flop_b = flop_f + 2.0 * B * ((H // pool) * H + (H // pool) * C)
     elems = D * H + (H // pool) * H + (H // pool) * C
@@ -371,6 +426,7 @@ def bench_step(torch, cn, dev):
     out["step_sparse_fused_ms"] = (out["sparse_input_ms"] + out["forward_sparse_ms"] + out["backward_deferred_sparse_ms"] +
                                    out["first_layer_codes_and_update_sparse_ms"] + out["other_layers_compress_and_update_ms"])
     out["step_unfused_ms"] = out["forward_ms"] + out["backward_ms"] + out["codec_and_update_unfused_ms"]
+    out["timing"] = "an event pair round every call of a phase, 7 calls; figures from the median"
     out["note"] = ("bytes per gradient element: absmax 4, then codes and update in one pass 13 (unfused: compress 5 + "
                    "decompress 5 + update 12), or compress 5 + fused decode+RMSprop 17 (unfused 5 + 5 + 20); "
                    "the gradient GEMM of layer 1 is 100000 x 8192 x 128")
@@ -423,26 +479,47 @@ def bench_products(torch, cn, dev, zeros=False):
     return out
 
 
+def describe_plan(cn, torch, m, n, k):
+    """The decomposition the library plans for an m x n x k dot on this GPU, in words, from its own planner."""
+    import ctypes
+    out = (ctypes.c_int64 * 8)()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    ws = (int(os.environ.get("CNHIP_WORKSPACE_MB", "1024")) << 20)
+    cn.lib().cn_host_plan_gemm_rows_along_k(m, n, k, cus, ws, 0, out)
+    tiles_m, tiles_n, k_iters, splits, ips, units, tile_n, tile_m = [int(v) for v in out]
+    text = "gemm_kernel on %d x %d tiles, %d tiles x %d K-chunks = %d workgroups" % (tile_m, tile_n, tiles_m * tiles_n, splits, units)
+    return text + (", followed by splitk_reduce_kernel over the %d planes" % splits if splits > 1 else ", K not split")
+
+
 def cpu_baseline(torch, tensors):
-    """The CPU port (oracle/cpu_port.c, all OpenMP threads) on a column sample of the first dot,
-    repeated until about ten seconds of CPU work have been timed."""
+    """The CPU port (oracle/cpu_port.c, all OpenMP threads) on the full README pair, once: out1 = batch . W1 with W1 (16 GB)
+    brought to the host in blocks of 10000 rows and the product accumulated block by block, then out2 = out1 . W2.  Only the
+    time inside the port's GEMM counts; the copies from the device do not."""
     import numpy as np
     import oracle
-    batch, W1 = tensors[0], tensors[1]
+    batch, W1, W2 = tensors[0], tensors[1], tensors[2]
     A = batch.cpu().numpy()
-    cols = 4096
-    Ws = np.ascontiguousarray(W1[:, :cols].cpu().numpy())
-    oracle.port_gemm_nn(A[:, :1024].copy(), Ws[:1024].copy())  # thread pool warm-up
-    reps, total = 0, 0.0
-    while total < 10.0 and reps < 64:
+    oracle.port_gemm(A[:, :1024].copy(), np.ones((1024, 512), np.float32))  # thread pool warm-up
+    out1 = np.zeros((M, N1), np.float32)
+    t1 = 0.0
+    rows = 10000
+    for r in range(0, K1, rows):
+        blk = W1[r:r + rows].cpu().numpy()
         t0 = time.perf_counter()
-        oracle.port_gemm_nn(A, Ws)
-        total += time.perf_counter() - t0
-        reps += 1
-    return {"value": reps * 2.0 * M * cols * K1 / total / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(),
-            "kind": "port",
-            "sample": "first dot of the step restricted to the first %d of %d output columns "
-                      "(128 x %d x %d fp32), %d repetitions, %.1f s of CPU time" % (cols, N1, K1, cols, reps, total)}
+        oracle.port_gemm(A[:, r:r + rows], blk, out=out1, accumulate=True, lda=K1)
+        t1 += time.perf_counter() - t0
+        del blk
+    W2h = W2.cpu().numpy()
+    t0 = time.perf_counter()
+    out2 = oracle.port_gemm(out1, W2h)
+    t2 = time.perf_counter() - t0
+    # the port's result against the GPU's, as a plausibility check of what was timed (fp32 accumulation in another order)
+    dev2 = float(np.abs(out2 - tensors[4].cpu().numpy()).max() / max(float(np.abs(out2).max()), 1e-30))
+    return {"value": (FLOP1 + FLOP2) / (t1 + t2) / 1e12, "unit": "TFLOP/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": "the full README pair once: 128x100000 . 100000x40000 (W1 streamed to the host in blocks of %d rows, %.2f s in "
+                      "the port's GEMM, %.3f TFLOP/s) then 128x40000 . 40000x20000 (%.2f s, %.3f TFLOP/s); copies from the device not "
+                      "timed; max deviation of out2 from the GPU's %.1e of max|out2|"
+                      % (rows, t1, FLOP1 / t1 / 1e12, t2, FLOP2 / t2 / 1e12, dev2)}
 
 
 def cpu_codec_baseline():
@@ -456,6 +533,51 @@ def cpu_codec_baseline():
     t0 = time.perf_counter(); oracle.port_decompress(codes, prec); td = time.perf_counter() - t0
     return {"elements": x.size, "cores": oracle.num_threads(), "kind": "port",
             "compress_GBps": 5.0 * x.size / tc / 1e9, "decompress_GBps": 5.0 * x.size / td / 1e9}
+
+
+def cpu_port_configs():
+    """The CPU port on the other configurations, all OpenMP threads: the three products of the 784 -> 1024 layer (batch 128), the
+    128 x 40000 round-trip tensor (abs-max, compression, decompression), and decompression of 4096 x 4096 weights followed by the
+    product at batch 32 / 128 / 512.  Each timed as the best of a few repetitions (small workloads; the first pass pays for
+    the threads and the caches)."""
+    import numpy as np
+    import oracle
+    rng = np.random.default_rng(1)
+
+    def best(fn, reps):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return min(ts)
+
+    out = {"cores": oracle.num_threads(), "kind": "port", "timing": "best of several repetitions, host clock"}
+    A = rng.uniform(0, 1, (128, 784)).astype(np.float32)
+    W = rng.uniform(-0.0576, 0.0576, (784, 1024)).astype(np.float32)
+    dC = rng.normal(0, 0.01, (128, 1024)).astype(np.float32)
+    flop = 2.0 * 128 * 784 * 1024
+    for name, fn in (("dot_128x1024x784", lambda: oracle.port_gemm(A, W)), ("Tdot_784x1024x128", lambda: oracle.port_gemm(A, dC, True, False)),
+                     ("dotT_128x784x1024", lambda: oracle.port_gemm(dC, W, False, True))):
+        t = best(fn, 20)
+        out["layer_784x1024_" + name] = {"us": t * 1e6, "TFLOPs": flop / t / 1e12}
+    x = rng.normal(0.0, 0.02, 128 * 40000).astype(np.float32)
+    x[::100] = rng.normal(0.0, 0.5, x[::100].size).astype(np.float32)
+    prec = oracle.port_absmax(x)
+    codes = oracle.port_compress(x, prec)
+    out["round_trip_128x40000"] = {"absmax_us": best(lambda: oracle.port_absmax(x), 10) * 1e6,
+                                   "compress_us": best(lambda: oracle.port_compress(x, prec), 10) * 1e6,
+                                   "decompress_us": best(lambda: oracle.port_decompress(codes, prec), 10) * 1e6}
+    Wq = rng.normal(0.0, 1.0 / 64.0, (4096, 4096)).astype(np.float32)
+    scale = oracle.port_absmax(Wq)
+    Wc = oracle.port_compress(Wq, scale)
+    t_dec = best(lambda: oracle.port_decompress(Wc, scale), 5)
+    Wd = oracle.port_decompress(Wc, scale)
+    for b in (32, 128, 512):
+        Ab = rng.normal(0.0, 1.0, (b, 4096)).astype(np.float32)
+        t = best(lambda: oracle.port_gemm(Ab, Wd), 5)
+        out["w8_gemm_batch%d" % b] = {"decompress_us": t_dec * 1e6, "dot_us": t * 1e6, "TFLOPs_of_the_pair": 2.0 * b * 4096 * 4096 / (t + t_dec) / 1e12}
+    return out
 
 
 def main():
@@ -506,14 +628,20 @@ def main():
         line["value"] = (FLOP1 + FLOP2) / (g["wall_ms"] * 1e-3) / 1e12
         line["ms_per_step"] = g["wall_ms"]
         achieved = FLOP1 / (g["gemm1_ms"] * 1e-3) / 1e12
+        line["ms_per_step_median"] = g["pair"]["median"]
+        line["ms_per_step_min"] = g["pair"]["min"]
         line["roofline"] = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                             "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                             "traffic": TRAFFIC_BYTES_GEMM1,
-                            "kernel": "gemm_kernel<true, 0, 256, 128> (13 K-chunks x 157 tiles of 128x256) followed by "
-                                      "splitk_reduce_kernel, 128x40000x100000; both are inside the timed bracket",
-                            "avg_ms": g["gemm1_ms"]}
-        extra["gemm2_128x20000x40000"] = {"ms": g["gemm2_ms"], "TFLOPs": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12,
-                                          "frac_mfma_peak": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS}
+                            "traffic_source": "profiles/gemm_and_codec_kernels_hbm_traffic.txt (FETCH_SIZE x 2.0 + WRITE_SIZE of this "
+                                              "launch; the file names the commit it was measured on); not re-measured by this run",
+                            "kernel": "128x40000x100000: %s; both are inside the timed bracket" % describe_plan(cn, torch, M, N1, K1),
+                            "avg_ms": g["gemm1_ms"], "median_ms": g["gemm1"]["median"], "min_ms": g["gemm1"]["min"],
+                            "frac_at_median": FLOP1 / (g["gemm1"]["median"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS}
+        extra["gemm2_128x20000x40000"] = {"ms": g["gemm2_ms"], "ms_median": g["gemm2"]["median"], "ms_min": g["gemm2"]["min"],
+                                          "TFLOPs": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12,
+                                          "frac_mfma_peak": FLOP2 / (g["gemm2_ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                                          "kernel": describe_plan(cn, torch, M, N2, N1)}
         extra["readme_pair_ms_reference_unknown_hw"] = 117.704285
         section("cfg1_layer_128x784x1024", lambda: bench_cfg1(torch, cn, dev))
         if not args.no_cpu and args.only is None:
@@ -525,6 +653,7 @@ def main():
         torch.cuda.empty_cache()
         if not args.no_cpu and args.only is None and "error" not in extra["codec"]:
             extra["codec"]["cpu_port"] = cpu_codec_baseline()
+            section("cpu_port_other_configs", cpu_port_configs)
     if args.only in (None, "codec"):
         section("layout_100000x8192", lambda: bench_layout(torch, cn, dev))
         torch.cuda.empty_cache()

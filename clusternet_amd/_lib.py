@@ -79,6 +79,8 @@ def lib():
     L.cn_host_encode_exact.argtypes = [f32, f32]
     L.cn_host_plan_gemm.argtypes = [i64, i64, i64, C.c_int, sz, C.c_int, C.POINTER(i64)]
     L.cn_host_plan_gemm.restype = None
+    L.cn_host_plan_gemm_rows_along_k.argtypes = [i64, i64, i64, C.c_int, sz, C.c_int, C.POINTER(i64)]
+    L.cn_host_plan_gemm_rows_along_k.restype = None
     L.cn_host_force_gemm_tile_n.argtypes = [C.c_int]
     L.cn_host_force_gemm_tile_n.restype = None
     L.cn_host_gemm_epilogue_in_kernel.argtypes = [C.c_int]

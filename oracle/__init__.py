@@ -69,6 +69,8 @@ def _load():
     lib.cn_port_absmax.restype = _c.c_float
     lib.cn_port_gemm_nn.argtypes = [_c.c_int64, _c.c_int64, _c.c_int64, _f32p, _c.c_int64, _f32p,
                                     _c.c_int64, _f32p, _c.c_int64]
+    lib.cn_port_gemm.argtypes = [_c.c_int, _c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
+                                 _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64]
     return lib
 
 
@@ -274,3 +276,24 @@ def port_gemm_nn(A, B):
     C = np.empty((M, N), np.float32)
     _lib.cn_port_gemm_nn(M, N, K, A, K, B, N, C, N)
     return C
+
+
+def port_gemm(A, B, ta=False, tb=False, out=None, accumulate=False, lda=None):
+    """out (+)= op(A) op(B) on all OpenMP threads, fp32 accumulation; `lda` lets A be a column block of a wider
+    row-major matrix (pass the block as a view, its leading dimension here)."""
+    M, K = (A.shape[1], A.shape[0]) if ta else A.shape
+    K2, N = (B.shape[1], B.shape[0]) if tb else B.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ")
+    B = _f32(B)
+    if lda is None:
+        A = _f32(A)
+        lda = A.shape[1]
+    elif A.dtype != np.float32 or A.strides[1] != 4 or A.strides[0] != 4 * lda:
+        raise ValueError("A is not a float32 block with leading dimension %d" % lda)
+    if out is None:
+        out = np.empty((M, N), np.float32)
+        accumulate = False
+    _lib.cn_port_gemm(int(ta), int(tb), int(accumulate), M, N, K, A.ctypes.data, lda, B.ctypes.data, B.shape[1],
+                      out.ctypes.data, N)
+    return out

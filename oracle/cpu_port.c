@@ -65,28 +65,54 @@ float cn_port_absmax(const float *x, size_t n) {
     return best;
 }
 
-/* C[M x N] = A[M x K] B[K x N], row-major, fp32 accumulation, beta = 0.  Threads own column
- * panels of 256; K is walked in slabs of 128 so the A slab and the C panel stay in cache. */
+/* C[M x N] = op(A) op(B) (+ C if `accumulate`), row-major, fp32 accumulation: ClusterNet::dot / Tdot / dotT
+ * (source/clusterNet.cpp:230-298,404-461).  trans_a: A stored K x M; trans_b: B stored N x K.  Threads own column
+ * panels of 256; with B stored K x N, K is walked in slabs of 128 so the A slab and the C panel stay in cache, and
+ * the inner loop runs along a row of B; with B stored N x K an output is a dot product of two contiguous rows,
+ * summed in eight interleaved partial sums. */
 #define NB 256
 #define KB 128
-void cn_port_gemm_nn(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
-                     int64_t ldb, float *C, int64_t ldc) {
+void cn_port_gemm(int trans_a, int trans_b, int accumulate, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda,
+                  const float *B, int64_t ldb, float *C, int64_t ldc) {
     int64_t panels = (N + NB - 1) / NB;
 #pragma omp parallel for schedule(dynamic, 1)
     for (int64_t p = 0; p < panels; ++p) {
         int64_t n0 = p * NB, nw = n0 + NB <= N ? NB : N - n0;
-        for (int64_t m = 0; m < M; ++m) memset(C + m * ldc + n0, 0, (size_t)nw * sizeof(float));
-        for (int64_t k0 = 0; k0 < K; k0 += KB) {
-            int64_t kw = k0 + KB <= K ? KB : K - k0;
-            for (int64_t m = 0; m < M; ++m) {
-                float *restrict crow = C + m * ldc + n0;
-                const float *arow = A + m * lda + k0;
-                for (int64_t k = 0; k < kw; ++k) {
-                    float av = arow[k];
-                    const float *restrict brow = B + (k0 + k) * ldb + n0;
-                    for (int64_t n = 0; n < nw; ++n) crow[n] += av * brow[n];
+        if (!accumulate)
+            for (int64_t m = 0; m < M; ++m) memset(C + m * ldc + n0, 0, (size_t)nw * sizeof(float));
+        if (!trans_b) {
+            for (int64_t k0 = 0; k0 < K; k0 += KB) {
+                int64_t kw = k0 + KB <= K ? KB : K - k0;
+                for (int64_t m = 0; m < M; ++m) {
+                    float *restrict crow = C + m * ldc + n0;
+                    for (int64_t k = 0; k < kw; ++k) {
+                        float av = trans_a ? A[(k0 + k) * lda + m] : A[m * lda + k0 + k];
+                        const float *restrict brow = B + (k0 + k) * ldb + n0;
+                        for (int64_t n = 0; n < nw; ++n) crow[n] += av * brow[n];
+                    }
                 }
             }
+        } else {
+            for (int64_t m = 0; m < M; ++m)
+                for (int64_t n = 0; n < nw; ++n) {
+                    const float *restrict brow = B + (n0 + n) * ldb;
+                    float part[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                    int64_t k = 0;
+                    if (!trans_a) {
+                        const float *restrict arow = A + m * lda;
+                        for (; k + 8 <= K; k += 8)
+                            for (int u = 0; u < 8; ++u) part[u] += arow[k + u] * brow[k + u];
+                        for (; k < K; ++k) part[0] += arow[k] * brow[k];
+                    } else {
+                        for (; k < K; ++k) part[k & 7] += A[k * lda + m] * brow[k];
+                    }
+                    C[m * ldc + n0 + n] += ((part[0] + part[1]) + (part[2] + part[3])) + ((part[4] + part[5]) + (part[6] + part[7]));
+                }
         }
     }
+}
+
+void cn_port_gemm_nn(int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
+                     int64_t ldb, float *C, int64_t ldc) {
+    cn_port_gemm(0, 0, 0, M, N, K, A, lda, B, ldb, C, ldc);
 }

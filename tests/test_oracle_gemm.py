@@ -109,3 +109,24 @@ def test_blocked_and_plain_loops_give_the_same_bits():
         C, Cabs = oracle.gemm_with_abs(A, B, ta, False)
         P, Pabs = oracle.gemm_cols(A, B, np.arange(N), ta, False)
         assert np.array_equal(C.view(np.uint64), P.view(np.uint64)) and np.array_equal(Cabs.view(np.uint64), Pabs.view(np.uint64))
+
+
+def test_cpu_port_gemm_all_transpositions_and_accumulation():
+    """The multi-threaded port timed as the CPU baseline: every transposition against the fp64 yard-stick, and a product
+    accumulated over row blocks of B (how the baseline streams a 16 GB weight matrix) against the product in one go."""
+    rng = np.random.default_rng(33)
+    M, N, K = 37, 700, 515
+    for ta in (False, True):
+        for tb in (False, True):
+            A = rng.uniform(0, 1, (K, M) if ta else (M, K)).astype(np.float32)
+            B = rng.normal(0, 0.05, (N, K) if tb else (K, N)).astype(np.float32)
+            ref, refabs = oracle.gemm_with_abs(A, B, ta, tb)
+            got = oracle.port_gemm(A, B, ta, tb)
+            assert float((np.abs(got - ref) / refabs).max()) <= 1e-5, (ta, tb)
+    A = rng.uniform(0, 1, (M, K)).astype(np.float32)
+    B = rng.normal(0, 0.05, (K, N)).astype(np.float32)
+    whole = oracle.port_gemm(A, B)
+    acc = np.zeros((M, N), np.float32)
+    for k0 in range(0, K, 128):   # the port's own K slabs: the accumulated product adds in the same order
+        oracle.port_gemm(A[:, k0:k0 + 128], B[k0:k0 + 128], out=acc, accumulate=True, lda=K)
+    assert np.array_equal(whole.view(np.uint32), acc.view(np.uint32))
