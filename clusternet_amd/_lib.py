@@ -101,6 +101,8 @@ def lib():
     L.cn_host_last_gemm_kernel.restype = C.c_int
     L.cn_host_tile_counters_in_use.argtypes = []
     L.cn_host_tile_counters_in_use.restype = C.c_int
+    L.cn_host_stream_slots.argtypes = [C.POINTER(C.c_uint64), C.c_int, C.POINTER(C.c_int)]
+    L.cn_host_stream_slots.restype = None
     L.cn_host_reduction_fences.argtypes = [C.c_int]
     L.cn_host_reduction_fences.restype = None
     L.cn_host_csr_strip_kernel.argtypes = [C.c_int]

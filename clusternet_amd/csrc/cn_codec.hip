@@ -565,7 +565,7 @@ constexpr int kResultWord = 8;  // in a group's line (64-bit): call number << 32
 
 __global__ __launch_bounds__(kThreads) void absmax_compress_kernel(
     const float *__restrict__ x, size_t n, uint8_t *__restrict__ codes, float *__restrict__ precision_out,
-    uint32_t *__restrict__ tickets, uint32_t spin_limit, const XEntry *__restrict__ quotient_table) {
+    uint32_t *__restrict__ tickets, uint32_t spin_limit, const XEntry *__restrict__ quotient_table, int fenced) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     XEntry *lut = reinterpret_cast<XEntry *>(smem_raw);  // kXEntries entries
     QuotientTableCopy<kThreads> copy;
@@ -625,8 +625,8 @@ __global__ __launch_bounds__(kThreads) void absmax_compress_kernel(
         uint32_t *first = tickets + (1 + group) * kTicketStride, *second = tickets;
         uint32_t key = m;
         // a grid of one workgroup still publishes: the wait below is the same for every grid
-        if ((gridDim.x == 1 || ticket_arrive(first, m, members, 0, &key)) &&
-            (groups == 1 || ticket_arrive(second, key, groups, 0, &key))) {
+        if ((gridDim.x == 1 || ticket_arrive(first, m, members, fenced, &key)) &&
+            (groups == 1 || ticket_arrive(second, key, groups, fenced, &key))) {
             // everyone has arrived, hence read the call number: publish, then advance it
             const unsigned long long word = ((unsigned long long)call << 32) | key;
             for (uint32_t g = 0; g < groups; ++g)
@@ -834,12 +834,13 @@ static cn_status compress_impl(const char *who, const float *x, float precision,
             hipLaunchKernelGGL(kernel, dim3(wgs), dim3(lanes), lds, st, x, precision, precision_dev, n, codes, ctx->xsteps,
                                ctx->xstep_count, ctx->table, queue, alpha, y, ctx->quotient_table);
         };
+        uint32_t *const counter = (y || drawn) ? ctx->tile_counter_for(st) : nullptr;  // NULL: a grid-stride walk instead
         if (y) {
-            if (q) launch(&compress_stream_kernel<1024, 4, true, true>, ctx->num_cu, 1024, ctx->next_tile_counter());
-            else   launch(&compress_stream_kernel<1024, 4, true, false>, ctx->num_cu, 1024, ctx->next_tile_counter());
-        } else if (drawn) {
-            if (q) launch(&compress_stream_kernel<1024, 12, false, true>, ctx->num_cu, 1024, ctx->next_tile_counter());
-            else   launch(&compress_stream_kernel<1024, 12, false, false>, ctx->num_cu, 1024, ctx->next_tile_counter());
+            if (q) launch(&compress_stream_kernel<1024, 4, true, true>, ctx->num_cu, 1024, counter);
+            else   launch(&compress_stream_kernel<1024, 4, true, false>, ctx->num_cu, 1024, counter);
+        } else if (drawn && counter) {
+            if (q) launch(&compress_stream_kernel<1024, 12, false, true>, ctx->num_cu, 1024, counter);
+            else   launch(&compress_stream_kernel<1024, 12, false, false>, ctx->num_cu, 1024, counter);
         } else {
             if (q) launch(&compress_stream_kernel<512, 10, false, true>, ctx->num_cu * 2, 512, nullptr);
             else   launch(&compress_stream_kernel<512, 10, false, false>, ctx->num_cu * 2, 512, nullptr);
@@ -1009,7 +1010,7 @@ cn_status cn_absmax_compress_8bit(const float *x, size_t n, uint8_t *codes, floa
     if (grid > tiles) grid = tiles;
     if (grid < 1) grid = 1;
     hipLaunchKernelGGL(absmax_compress_kernel, dim3((unsigned)grid), dim3(kThreads), kTableBytes, st, x, n, codes,
-                       precision_out, ctx->tickets, g_absmax_compress_spins, ctx->quotient_table);
+                       precision_out, ctx->tickets, g_absmax_compress_spins, ctx->quotient_table, g_reduction_fences);
     CN_HIP(hipGetLastError());
     return CN_OK;
 }
@@ -1047,9 +1048,10 @@ cn_status cn_fill_f32(float *dst, float value, size_t n, void *stream) {
     if (s != CN_OK) return s;
     constexpr int kFillLanes = 1024, kFillVecs = 8;
     const size_t tiles = (n / 4 + (size_t)kFillLanes * kFillVecs - 1) / ((size_t)kFillLanes * kFillVecs);
-    if (aligned(dst, 16) && n >= kDrawnFrom && n < kDrawnBelow) {
+    uint32_t *const counter = (aligned(dst, 16) && n >= kDrawnFrom && n < kDrawnBelow) ? ctx->tile_counter_for((hipStream_t)stream) : nullptr;
+    if (counter) {
         hipLaunchKernelGGL((fill_tiles_kernel<kFillLanes, kFillVecs, true>), dim3(ctx->num_cu), dim3(kFillLanes), 0, (hipStream_t)stream,
-                           dst, value, n, ctx->next_tile_counter());
+                           dst, value, n, counter);
     } else if (aligned(dst, 16) && n >= ((size_t)1 << 20) && tiles <= 0x7fffffffu) {
         hipLaunchKernelGGL((fill_tiles_kernel<kFillLanes, kFillVecs, false>), dim3((unsigned)tiles), dim3(kFillLanes), 0,
                            (hipStream_t)stream, dst, value, n, (uint32_t *)nullptr);

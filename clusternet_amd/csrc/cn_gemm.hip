@@ -1370,13 +1370,19 @@ static cn_status gemm_impl(int ta, int tb, bool w8, int64_t M, int64_t N, int64_
     // K not split and short, 128-row tiles, several rounds of them, whole K stages, 16-byte operands and a result that
     // 32-bit offsets reach: the workgroups stay and draw their tiles (100000 x 8192 x 128: 1.61 ms against 1.74 ms; from
     // about 64 stages per tile on there is nothing left to gain and the workgroup per tile is ahead by a percent).
-    const bool persistent = g_persistent && !w8 && !then && plan.splits == 1 && plan.tile_m == kTileM &&
-                            plan.units >= (int64_t)ctx->num_cu * 2 * kPersistentFromRounds && plan.k_iters <= kPersistentMaxStages &&
-                            a.vec_a && a.vec_b && K % gemm_tile_k(plan.tile_n) == 0 && ldc <= (1 << 22);
+    bool persistent = g_persistent && !w8 && !then && plan.splits == 1 && plan.tile_m == kTileM &&
+                      plan.units >= (int64_t)ctx->num_cu * 2 * kPersistentFromRounds && plan.k_iters <= kPersistentMaxStages &&
+                      a.vec_a && a.vec_b && K % gemm_tile_k(plan.tile_n) == 0 && ldc <= (1 << 22);
+    if (persistent) {
+        // its workgroups draw their tiles: without a counter (the stream is being captured, or the library has no context
+        // yet and may not create one) the workgroup per tile stays
+        if (!context) context = ready_context(ctx->device);
+        a.tile_counter = context ? context->tile_counter_for(st) : nullptr;
+        persistent = a.tile_counter != nullptr;
+    }
     g_last_kernel = persistent ? kTookPersistent : kTookTiled;
     g_last_splits = plan.splits;
     if (persistent) {
-        a.tile_counter = context ? context->next_tile_counter() : nullptr;  // without a context: a fixed share of the tiles each
         if (!ta && !tb)     s = launch_persistent<true, false>(a, plan.tile_n, ctx->num_cu, ctx->device, st);
         else if (ta && !tb) s = launch_persistent<false, false>(a, plan.tile_n, ctx->num_cu, ctx->device, st);
         else if (!ta && tb) s = launch_persistent<true, true>(a, plan.tile_n, ctx->num_cu, ctx->device, st);

@@ -26,6 +26,18 @@ void host_table(float out[126]);
 // ---- per-device state ------------------------------------------------------------------------
 constexpr int kTileQueues = 32;  // ticket counters of the streaming kernels, each on a 128-byte line of its own
 constexpr int kTileQueueWords = kTileQueues * 32;
+// Host-side table: the first kTileQueues distinct keys get slots 0, 1, ... for good; later ones get -1.
+struct StreamSlots {
+    const void *owner[kTileQueues] = {};
+    int used = 0;
+    int slot_for(const void *key) {
+        for (int i = 0; i < used; ++i)
+            if (owner[i] == key) return i;
+        if (used == kTileQueues) return -1;
+        owner[used] = key;
+        return used++;
+    }
+};
 struct Context {
     bool ready = false;
     int device = -1;
@@ -40,10 +52,12 @@ struct Context {
     uint32_t *tickets = nullptr;         // running maximum and arrival count of the max reductions (kTicketWords words)
     double *sum_scratch = nullptr;       // per-workgroup partial sums (1024 doubles)
     uint32_t *tile_queue = nullptr;      // ticket counters of the streaming kernels (kTileQueueWords words, left at 0)
-    unsigned tile_queue_turn = 0;        // which of the counters the next launch takes
-    // A counter for one launch of a kernel that draws its tiles.  The launches take the kTileQueues counters in turn, so
-    // that kernels which overlap (on different streams) do not draw from the same one unless that many are in flight.
-    uint32_t *next_tile_counter() { return tile_queue + (size_t)(tile_queue_turn++ % (unsigned)kTileQueues) * 32u; }
+    StreamSlots tile_queue_owners;       // which launch stream holds which counter
+    // The counter a kernel launched on `stream` draws its tiles from, or NULL: take the form that does not draw.  A
+    // counter belongs to one stream for good, so the kernels that share it are ordered by that stream, each finding the 0
+    // its predecessor left.  NULL while the stream is being captured (a graph would carry the counter into replays that
+    // nothing orders against later launches) and when more streams than counters have asked.
+    uint32_t *tile_counter_for(hipStream_t stream);
 };
 constexpr int kMaxDevices = 16;
 constexpr int kReduceSlots = 4096;
@@ -70,6 +84,8 @@ extern int g_reduction_fences;
 
 // Returns the context of the current device, initialising it on first use.
 cn_status current_context(Context **out);
+// The context of `device` if it is initialised, else NULL (never initialises, never allocates).
+Context *ready_context(int device);
 
 // Bytes of split-K workspace cn_init allocates (CNHIP_WORKSPACE_MB, default 1 GiB), and the figure the planner
 // sees on `device`: the context's if it is initialised, else what initialisation would allocate.

@@ -209,11 +209,12 @@ static cn_status launch_flat(Context *ctx, hipStream_t st, const float *a, const
     auto ok16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     const bool vec = ok16(a) && ok16(out) && (!kTwo || ok16(b));
     constexpr int kFT = 512;
-    if (vec && (size_t)n >= kDrawnFrom && (size_t)n < kDrawnBelow) {
+    uint32_t *const counter = (vec && (size_t)n >= kDrawnFrom && (size_t)n < kDrawnBelow) ? ctx->tile_counter_for(st) : nullptr;
+    if (counter) {
         // beyond the cache: one workgroup per compute unit, tiles of 512 lanes x 8 vectors drawn from the counter (the
         // weight update on 819.2 M elements: 1.46 ms; 1024 x 4: 1.48, 256 x 16: 1.50, 512 x 4: 1.49, 1024 x 8: 1.58)
         hipLaunchKernelGGL((flat_kernel<Op, kTwo, true, kFT, 8, true>), dim3(ctx->num_cu), dim3(kFT), 0, st, a, b, n, out, f,
-                           ctx->next_tile_counter());
+                           counter);
     } else if (vec) {
         // a workgroup per tile of 512 lanes x 2 vectors, as many workgroups as tiles
         int64_t grid = (n / 4 + kFT * 2 - 1) / (kFT * 2);
@@ -416,7 +417,8 @@ cn_status cn_transpose_f32(const float *in, int64_t rows, int64_t cols, float *o
         return CN_OK;
     };
     const int64_t tiles128 = ((rows + 127) / 128) * ((cols + 127) / 128);
-    if (vec && (size_t)rows * (size_t)cols >= kDrawnFrom && tiles128 <= 0x7fffffffLL) {
+    uint32_t *const counter = (vec && (size_t)rows * (size_t)cols >= kDrawnFrom && tiles128 <= 0x7fffffffLL) ? ctx->tile_counter_for(st) : nullptr;
+    if (counter) {
         // beyond the cache: a persistent workgroup per compute unit draws the tiles in the same order and has its next
         // tile's loads in flight while it stores (100000 x 8192: 5.9 TB/s against 5.5 for a workgroup per tile; 20000 x
         // 40000: 5.8 against 5.5; 8192 x 100096: 6.15 either way; 4096 x 4096: 31 us against 24, hence the bound)
@@ -425,7 +427,7 @@ cn_status cn_transpose_f32(const float *in, int64_t rows, int64_t cols, float *o
         if (drawn_configured.first(ctx->device))
             CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&transpose_drawn_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         hipLaunchKernelGGL(transpose_drawn_kernel, dim3(ctx->num_cu), dim3(1024), lds, st, in, rows, cols, out, (rows + 127) / 128,
-                           (uint32_t)tiles128, ctx->next_tile_counter());
+                           (uint32_t)tiles128, counter);
         CN_HIP(hipGetLastError());
         return CN_OK;
     }

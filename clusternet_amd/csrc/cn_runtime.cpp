@@ -156,11 +156,35 @@ cn_status current_context(Context **out) {
     return CN_OK;
 }
 
+Context *ready_context(int device) {
+    return (device >= 0 && device < kMaxDevices && g_ctx[device].ready) ? &g_ctx[device] : nullptr;
+}
+
+static std::mutex g_slots_mutex;
+
+uint32_t *Context::tile_counter_for(hipStream_t stream) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capture) != hipSuccess) {
+        (void)hipGetLastError();  // the query's failure is not the caller's: the kernel simply does not draw
+        return nullptr;
+    }
+    if (capture != hipStreamCaptureStatusNone) return nullptr;
+    std::lock_guard<std::mutex> lock(g_slots_mutex);
+    const int slot = tile_queue_owners.slot_for(stream);
+    return slot < 0 ? nullptr : tile_queue + (size_t)slot * 32u;
+}
+
 }  // namespace cn
 
 using namespace cn;
 
 extern "C" {
+
+// Test hook: the slots a fresh table of counter owners hands to the keys in turn (pure host logic).
+void cn_host_stream_slots(const uint64_t *keys, int n, int *slots_out) {
+    StreamSlots table;
+    for (int i = 0; i < n; ++i) slots_out[i] = table.slot_for(reinterpret_cast<const void *>((uintptr_t)keys[i]));
+}
 
 const char *cn_status_string(cn_status s) {
     switch (s) {

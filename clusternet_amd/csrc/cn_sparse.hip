@@ -899,9 +899,9 @@ __global__ __launch_bounds__(kT) void transpose_fill_kernel(int64_t R, const int
         const int64_t r_end = (b + 1) * rows_per_block < R ? (b + 1) * rows_per_block : R;
         for (int64_t r = b * rows_per_block; r < r_end; ++r) {
             for (int32_t j = row_ptr[r] + threadIdx.x; j < row_ptr[r + 1]; j += kT) {
-                int32_t *slot = &cursor[(int64_t)col_idx[j] * blocks + b];
-                const int32_t at = *slot;
-                *slot = at + 1;
+                // an atomic, so that a row that names a column twice (the layout does not forbid it) still gives both
+                // entries a place of their own; entries of different columns never meet on a slot
+                const int32_t at = atomicAdd(&cursor[(int64_t)col_idx[j] * blocks + b], 1);
                 out_col[at] = (int32_t)r;
                 out_val[at] = vals[j];
             }

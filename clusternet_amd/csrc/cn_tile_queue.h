@@ -11,7 +11,9 @@
 // The counter must be 0 when the kernel starts and is left at 0: every workgroup draws until its ticket is past the
 // last tile, so exactly gridDim.x tickets fail, and the workgroup that draws the last of them (ticket tiles +
 // gridDim.x - 1) knows that nobody will draw again and clears the counter.  Kernels that share a counter must not
-// overlap: the library keeps several and gives them to its launches in turn (Context::next_tile_counter).
+// overlap: the library keeps several and ties each to one launch stream (Context::tile_counter_for), whose order then is
+// the order of the kernels on the counter; a launch that is being captured into a graph gets none and walks its tiles
+// in a fixed pattern instead.
 #pragma once
 
 #include "cn_internal.h"

@@ -176,9 +176,10 @@ cn_status axpy_impl(const uint8_t *codes, float precision, const float *precisio
     const bool vec = aligned(codes, 4) && aligned(y, 16);
     const int grid = grid_of(ctx, n, vec);
     uint32_t *const none = nullptr;
-    if (vec && n >= kDrawnFrom && n < kDrawnBelow)
+    uint32_t *const counter = (vec && n >= kDrawnFrom && n < kDrawnBelow) ? ctx->tile_counter_for(st) : nullptr;
+    if (counter)
         hipLaunchKernelGGL((decompress_axpy_kernel<true, kDrawnVecs, true>), dim3(ctx->num_cu), dim3(kThreads), 0, st, codes,
-                           precision, precision_dev, alpha, n, y, ctx->table, ctx->next_tile_counter());
+                           precision, precision_dev, alpha, n, y, ctx->table, counter);
     else if (vec)
         hipLaunchKernelGGL((decompress_axpy_kernel<true, kTileVecsSmall, false>), dim3(grid), dim3(kThreads), 0, st, codes,
                            precision, precision_dev, alpha, n, y, ctx->table, none);
@@ -198,9 +199,9 @@ cn_status rmsprop_impl(float *rms, const float *grad, const uint8_t *codes, floa
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
     const bool vec = aligned(rms, 16) && aligned(w, 16) && (codes ? aligned(codes, 4) : aligned(grad, 16));
-    const bool drawn = vec && n >= kDrawnFrom && n < kDrawnBelow;
+    uint32_t *const queue = (vec && n >= kDrawnFrom && n < kDrawnBelow) ? ctx->tile_counter_for(st) : nullptr;
+    const bool drawn = queue != nullptr;
     const int grid = drawn ? ctx->num_cu : grid_of(ctx, n, vec);
-    uint32_t *const queue = drawn ? ctx->next_tile_counter() : nullptr;
     auto go = [&](auto kernel) {
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), 0, st, rms, grad, codes, precision, precision_dev, w, mult, rate, n,
                            ctx->table, queue);

@@ -8,9 +8,17 @@
  * without a usable GPU, cn_init and every compute entry point return CN_ERR_NO_DEVICE.
  *
  * One stream at a time per device, as in the reference (one host thread, the default stream,
- * source/clusterNet.cpp:406-407): the products that split K, the reductions and the sparse conversions
- * keep partial results in per-device scratch memory owned by the library, so calls that may run at the
- * same time on one device (different streams without an ordering between them) race on it.
+ * source/clusterNet.cpp:406-407), for every call that keeps partial results in per-device memory owned by
+ * the library; calls that may run at the same time on one device (different streams without an ordering
+ * between them) race on it silently:
+ *   - the split-K workspace: every product that splits K, cn_csr_from_dense_f32, cn_csr_transpose, and the
+ *     fused products (bias + maxout, maxout expansion) for the shapes they do not fuse;
+ *   - the ticket lines and slots of the reductions: cn_absmax_f32, cn_max_f32, cn_sum_f32,
+ *     cn_absmax_compress_8bit, and the products that also deliver max|C|;
+ *   - the array of cn_gemm_f32_noalloc.
+ * Kernels that draw their tiles from a counter (the streaming passes on tensors of 2^26 elements and more, the
+ * persistent form of an unsplit product) may overlap: a counter is tied to one stream, and a call that is being
+ * captured into a graph takes the form that does not draw, so replays may run beside eager calls.
  *
  * Storage convention: matrices are ROW-major with an explicit leading dimension (elements per
  * row).  The reference keeps device matrices column-major (source/basicOps.cu:14-33) and calls
@@ -260,8 +268,9 @@ cn_status cn_csr_to_dense_f32(int64_t R, int64_t C, const int32_t *row_ptr_devic
                               const float *vals_device, float *out_device, int64_t ldo, void *stream);
 
 /* CSR of S^T from the CSR of the R x C matrix S with nnz nonzeros (t_row_ptr: C + 1 entries, t_col_idx
- * and t_vals: nnz entries, column indices ascending within a row).  A counting sort over (column, block of rows) in
- * the library's workspace: the result does not depend on scheduling, and a column of any number of nonzeros costs
+ * and t_vals: nnz entries, column indices ascending within a row; a source row that names a column twice keeps both
+ * entries, in no fixed order).  A counting sort over (column, block of rows) whose cursor array lives in the library's
+ * split-K workspace (do not overlap it with a product on another stream): the result does not depend on scheduling, and a column of any number of nonzeros costs
  * what its nonzeros cost.  `scratch` is not used any more and may be NULL.  With it Tdot_sparse (the transposed operand of cusparseScsrmm2, source/clusterNet.cpp:304,307)
  * is cn_csr_gemm_f32 on the transposed arrays. */
 cn_status cn_csr_transpose(int64_t R, int64_t C, int64_t nnz, const int32_t *row_ptr_device,

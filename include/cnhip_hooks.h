@@ -70,6 +70,10 @@ void cn_host_reduction_fences(int enabled);
 /* Synchronises the current device and returns how many of its ticket counters (the ones the streaming kernels draw
  * their tiles from) are not zero: 0 whenever no kernel is running; -1 if the device is not initialised. */
 int cn_host_tile_counters_in_use(void);
+/* The library's table of counter owners, on a fresh instance: slots_out[i] = the counter the i-th key (a stream handle) is
+ * given when the keys ask in turn: the same key always the same slot, the first 32 distinct keys slots 0 .. 31, any later
+ * key -1 (its kernels then take the form that does not draw).  Pure host logic. */
+void cn_host_stream_slots(const uint64_t *keys, int n, int *slots_out);
 
 /* cn_absmax_compress_8bit as one launch (abs-max, a wait across the resident grid, compression) instead of as two
  * kernels: 1 = wherever the single launch can run (aligned tensors below 2^26 elements), 0 = never, negative = the

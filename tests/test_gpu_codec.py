@@ -66,8 +66,9 @@ def test_reductions_with_and_without_writer_fences(dev):
     rng = np.random.default_rng(123)
     x = rng.normal(0, 3, 6_000_011).astype(np.float32)
     xt = _t(x, dev)
+    want_codes = {}
     try:
-        for n in (1, 4096, 4097, 70_000, 1_000_003, 6_000_011):
+        for n in (1, 4096, 4097, 70_000, 1_000_003, 6_000_011, 1_000_000):
             want_max = float(np.abs(x[:n]).max())
             want_sum = None
             for per_cu in (0, 1, 3, 16):
@@ -79,10 +80,21 @@ def test_reductions_with_and_without_writer_fences(dev):
                     got = float(L.reduce_sum(xt[:n]).cpu()[0])
                     want_sum = got if want_sum is None else want_sum
                     assert got == want_sum, (n, per_cu, fenced)
+                    # abs-max -> compression as one launch shares the ticket lines and honours the same switch
+                    if per_cu == 0 and n % 4 == 0:
+                        L.lib().cn_host_absmax_compress_single_launch(1)
+                        prec_out = torch.zeros(1, device=dev)
+                        codes, _ = cn.absmax_compression_8bit(xt[:n], precision_out=prec_out)
+                        L.lib().cn_host_absmax_compress_single_launch(-1)
+                        assert float(prec_out.cpu()[0]) == want_max, (n, fenced)
+                        if want_codes.get(n) is None:
+                            want_codes[n] = oracle.compress(x[:n], want_max)
+                        assert np.array_equal(codes.cpu().numpy(), want_codes[n]), (n, fenced)
             assert abs(want_sum - float(x[:n].astype(np.float64).sum())) <= 1e-6 * np.abs(x[:n]).astype(np.float64).sum()
     finally:
         L.lib().cn_host_reduction_fences(0)
         L.lib().cn_host_codec_workgroups_per_cu(0)
+        L.lib().cn_host_absmax_compress_single_launch(-1)
 
 
 def test_compress_config2_bit_exact(dev):

@@ -95,9 +95,9 @@ def test_with_the_maximum_and_a_padded_result(dev):
     assert torch.equal(plain.view(torch.int32), out.contiguous().view(torch.int32))
 
 
-def test_without_a_counter_and_into_an_unaligned_result(dev):
-    """cn_gemm_f32_noalloc has no context to take a counter from: its persistent workgroups walk a fixed share of the tiles.
-    Same bits; here also with a result whose rows start at odd addresses (the write-out is 4-byte stores)."""
+def test_entry_point_that_allocates_nothing_and_an_unaligned_result(dev):
+    """cn_gemm_f32_noalloc takes the same persistent form once the library is initialised (it borrows a counter, it does not
+    create a context).  Same bits; here also with a result whose rows start at odd addresses (the write-out is 4-byte stores)."""
     import torch
     import clusternet_amd as cn
     M, N, K = 12836, 4096, 64

@@ -225,3 +225,20 @@ def test_gemm_plan_covers_k_and_fits_workspace():
                     assert splits * M * N * 4 <= ws
     L.cn_host_plan_gemm(128, 40000, 100000, 256, 1 << 30, 128, out)
     assert list(out)[:6] == [1, 313, 3125, 13, 241, 4069]
+
+
+def test_tile_counters_are_tied_to_streams():
+    """Kernels that draw their tiles from a counter may share one only if a stream orders them.  The table behind
+    Context::tile_counter_for: a stream keeps the counter it was first given, 32 distinct streams get the 32 counters, a
+    33rd gets none (its kernels walk their tiles in a fixed pattern), and the default stream (handle 0) is a stream like
+    any other."""
+    import ctypes
+    L = cn.lib()
+    keys = [0, 0x7f00, 0, 0x7f10, 0x7f00] + [0x9000 + 16 * i for i in range(40)] + [0x7f10, 0]
+    arr = (ctypes.c_uint64 * len(keys))(*keys)
+    out = (ctypes.c_int * len(keys))()
+    L.cn_host_stream_slots(arr, len(keys), out)
+    got = list(out)
+    assert got[:5] == [0, 1, 0, 2, 1]
+    assert got[5:5 + 29] == list(range(3, 32)) and got[5 + 29:5 + 40] == [-1] * 11
+    assert got[-2:] == [2, 0]
