@@ -1,24 +1,44 @@
 // Host-side work decomposition for the fp32 GEMM kernels (pure function, no HIP calls).
 //
-// The output is cut into tiles of 128 rows and 128 or 256 columns, two workgroups per compute unit
-// either way (of 64 rows where K would otherwise be cut into sixteen chunks and more), or, when it has no more than
-// 64 rows or is small altogether, into tiles of 32 rows and 128 columns: a 128-row tile would spend most of its matrix-core work on rows that do not exist, while a 32-row
-// tile leaves such a product to what it is bound by, the one pass over B; and a small product becomes four
-// times as many workgroups.  The batches this library serves are skinny (M = 128), so tiles alone cannot fill 256
-// compute units; K is therefore cut into `splits` chunks, every (chunk, tile) pair becomes one
-// workgroup, and a second kernel adds the chunk results in a fixed order (deterministic, no
-// atomics).  Chunks are ordered chunk-major so that workgroups running at the same time walk the
-// same K range and share the A panel in L2.
+// The output is cut into tiles of one of four geometries (rows x columns): 128 x 128, 128 x 256, 64 x 128 or 32 x 128,
+// two workgroups per compute unit for each.  The batches this library serves are skinny (M = 128), so tiles alone cannot
+// fill 256 compute units; K is therefore cut into `splits` chunks, every (chunk, tile) pair becomes one workgroup, and a
+// second kernel adds the chunk results in a fixed order (deterministic, no atomics).  Chunks are ordered chunk-major so
+// that workgroups running at the same time walk the same K range and share the A panel in L2.
 //
-// Tile width.  A 256-column tile fetches the A tile once per 256 output columns and reads less from
-// LDS per flop, and halves the number of work units (and their fill / write-out overheads); a
-// 128-column tile gives twice as many work units and wins when the problem would otherwise not fill
-// the machine or would leave a round mostly empty.
+// One cost model decides both the geometry and the split: rounds of resident workgroups, each costing its stages plus a
+// fixed part, a last partial round that runs faster when its workgroups have a compute unit to themselves, and the chunk
+// sum.  Its six kinds of constants are microseconds measured on this part (a least-squares fit over forty shapes times
+// four geometries, 9 % rms); tests/test_gpu_planner.py times the planned form of those shapes against every forced
+// geometry and fails when a rule change leaves one more than 7 % behind the best.
+//   128 x 256  fetches the A tile once per 256 output columns and reads less from LDS per flop: 2.5 % faster per flop
+//              than 128 x 128 on streaming shapes, half as many, longer work units
+//   128 x 128  twice as many work units: wins when the wide tile would leave a round mostly empty
+//   64 x 128   half the flops per stage at 52 % of the time: mid-size products, and products whose K would otherwise be
+//              cut into sixteen and more chunks (half the planes to write and add)
+//   32 x 128   a quarter of the flops at 30 % of the time: products of a handful of rows (a 128-row tile would spend
+//              most of its matrix-core work on rows that do not exist) and small products (four times as many workgroups)
 #include "cn_internal.h"
 
 namespace cn {
 
 namespace {
+
+struct Geometry {
+    int tile_m, tile_n;
+    int min_iters;     // a chunk is at least this many stages (128 k) deep
+    double stage_us;   // one pipeline stage of a workgroup that shares its compute unit with another
+    double unit_us;    // per work unit: first stage's latency, write-out, start of the workgroup
+};
+// 256 compute units at the clock the part holds under this load.
+constexpr Geometry kGeometries[] = {{128, 128, 4, 3.91, 2.3}, {128, 256, 8, 3.81, 3.4}, {64, 128, 4, 2.03, 2.0}, {32, 128, 4, 1.18, 1.25}};
+constexpr double kAlone = 0.57;            // a stage of a workgroup that has its compute unit to itself, relative to stage_us
+constexpr double kLaunchUs = 3.3;          // a launch
+constexpr double kChunkSumUs = 4.9;        // the second kernel ...
+constexpr double kChunkSumUsPerMB = 0.17;  // ... and what it moves: (chunks + 1) planes at 6 TB/s (52 us for the 287 MB of the README product)
+constexpr double kPlaneWriteUsPerMB = 0.15; // what writing the chunk planes costs the product itself (128 x 100000 x 8192: nine planes of 51 MB
+                                           // instead of five cost 40 us more than the rounds they even out save)
+constexpr double kRowsAlongMPenalty = 1.10;  // 64- and 32-row tiles of an A stored k by m read it in short pieces
 
 struct Choice {
     double cost;
@@ -26,14 +46,8 @@ struct Choice {
     int64_t ips;
 };
 
-// Cost in units of "32 k of a 128 x 128 tile on a compute unit shared by two workgroups".
-// `iter_cost` is the cost of one pipeline stage of this tile width in that unit; a last, partial
-// round that leaves every workgroup a compute unit of its own runs at `alone` of that.
-Choice best_split(int64_t tiles, int64_t k_iters, int64_t cus, double iter_cost, int64_t max_splits,
+Choice best_split(int64_t tiles, int64_t k_iters, int64_t cus, double stage_us, double unit_us, int64_t max_splits,
                   double out_bytes) {
-    const double unit_seconds = 2.0 * 4096.0 / 2.4e9;
-    const double unit_overhead = 6.0;  // pipeline fill + C write-out
-    const double alone = 0.6;
     const int64_t slots = cus * 2;
     Choice best{0.0, 1, k_iters};
     for (int64_t s = 1; s <= max_splits; ++s) {
@@ -42,9 +56,9 @@ Choice best_split(int64_t tiles, int64_t k_iters, int64_t cus, double iter_cost,
         if (eff != s && s != 1) continue;  // same decomposition as a smaller s
         int64_t units = tiles * eff;
         const int64_t full = units / slots, rest = units % slots;
-        double cost = (double)full * ((double)ips * iter_cost + unit_overhead);
-        if (rest) cost += (double)ips * iter_cost * (rest <= cus ? alone : 1.0) + unit_overhead;
-        if (eff > 1) cost += (double)(eff + 1) * out_bytes / 4.0e12 / unit_seconds + 3.0;
+        double cost = kLaunchUs + (double)full * ((double)ips * stage_us + unit_us);
+        if (rest) cost += (double)ips * stage_us * (rest <= cus ? kAlone : 1.0) + unit_us;
+        if (eff > 1) cost += kChunkSumUs + (kChunkSumUsPerMB * (double)(eff + 1) + kPlaneWriteUsPerMB * (double)eff) * out_bytes / 1.0e6;
         if (s == 1 || cost < best.cost) best = Choice{cost, (int)eff, ips};
     }
     return best;
@@ -63,70 +77,39 @@ int64_t split_limit(int64_t k_iters, int min_iters, double out_bytes, size_t wor
 }  // namespace
 
 GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int num_cu, size_t workspace_bytes, int force_tile_n, bool a_along_k) {
-    GemmPlan p;
-    p.tile_m = kTileM;
-    p.tiles_m = (M + kTileM - 1) / kTileM;
     const int64_t cus = num_cu > 0 ? num_cu : 1;
     const double out_bytes = (double)M * (double)N * 4.0;
-    const int64_t tiles_n128 = (N + 127) / 128, tiles_n256 = (N + 255) / 256;
-    int64_t it128 = (K + gemm_tile_k(128) - 1) / gemm_tile_k(128), it256 = (K + gemm_tile_k(256) - 1) / gemm_tile_k(256);
-    if (it128 < 1) it128 = 1;
-    if (it256 < 1) it256 = 1;
-
-    // A product too small to fill the machine with 128-row tiles even at the deepest split also takes the small
-    // tile: four times as many, lighter workgroups (measured: 128 x 1024 x 784 in 9.7 us instead of 18.5 us,
-    // 784 x 1024 x 128 in 5.6 us instead of 11.8 us).
-    const bool small = p.tiles_m * tiles_n128 * split_limit(it128, 4, out_bytes, workspace_bytes) < cus * 2;
-    if (force_tile_n == kTileMLow || force_tile_n == kTileMMid || (force_tile_n == 0 && (M <= kLowTileMaxRows || small))) {
-        // A stage of the 32 x 128 tile moves 20 KB for a quarter of the unit's flops: it costs what its
-        // loads cost, about a third of the unit; the 64 x 128 tile, for 33 .. 64 rows, half of the unit.
-        const bool mid = force_tile_n == kTileMMid || (force_tile_n == 0 && !small && M > kTileMLow);
-        p.tile_m = mid ? kTileMMid : kTileMLow;
-        p.tiles_m = (M + p.tile_m - 1) / p.tile_m;
-        const Choice c = best_split(p.tiles_m * tiles_n128, it128, cus, mid ? 0.55 : 0.35, split_limit(it128, 4, out_bytes, workspace_bytes), out_bytes);
-        p.tile_n = 128;
-        p.tiles_n = tiles_n128;
-        p.k_iters = it128;
-        p.splits = c.splits;
-        p.iters_per_split = c.ips;
-        p.units = p.tiles_m * p.tiles_n * p.splits;
-        return p;
+    GemmPlan best;
+    double best_cost = 0.0;
+    bool have = false;
+    for (const Geometry &g : kGeometries) {
+        // force_tile_n: 128 / 256 name the width of the 128-row tile, 32 / 64 the rows of the 128-wide one
+        const int name = g.tile_m == kTileM ? g.tile_n : g.tile_m;
+        if (force_tile_n != 0 && force_tile_n != name) continue;
+        if (force_tile_n == 0) {
+            // a tile taller than twice the product only multiplies rows that do not exist
+            if (g.tile_m > kTileMLow && M <= g.tile_m / 2) continue;
+        }
+        const int64_t tiles_m = (M + g.tile_m - 1) / g.tile_m, tiles_n = (N + g.tile_n - 1) / g.tile_n;
+        int64_t k_iters = (K + gemm_tile_k(g.tile_n) - 1) / gemm_tile_k(g.tile_n);
+        if (k_iters < 1) k_iters = 1;
+        const double stage_us = g.stage_us * ((g.tile_m < kTileM && !a_along_k) ? kRowsAlongMPenalty : 1.0);
+        const Choice c = best_split(tiles_m * tiles_n, k_iters, cus, stage_us, g.unit_us,
+                                    split_limit(k_iters, g.min_iters, out_bytes, workspace_bytes), out_bytes);
+        if (!have || c.cost < best_cost) {
+            have = true;
+            best_cost = c.cost;
+            best.tile_m = g.tile_m;
+            best.tile_n = g.tile_n;
+            best.tiles_m = tiles_m;
+            best.tiles_n = tiles_n;
+            best.k_iters = k_iters;
+            best.splits = c.splits;
+            best.iters_per_split = c.ips;
+            best.units = tiles_m * tiles_n * c.splits;
+        }
     }
-
-    // a chunk is at least 128 k deep
-    Choice narrow = best_split(p.tiles_m * tiles_n128, it128, cus, 1.0, split_limit(it128, 4, out_bytes, workspace_bytes), out_bytes);
-    // One 16-deep stage of a 128 x 256 tile is as many flops as the unit.  Measured per flop the wide
-    // tile is within 1 % of the narrow one on streaming shapes (its lower traffic buys a little clock),
-    // so the choice is left to what the model sees: fewer, longer work units and rounding of rounds.
-    const double kWideGain = 1.0;
-    Choice wide = best_split(p.tiles_m * tiles_n256, it256, cus, kWideGain, split_limit(it256, 8, out_bytes, workspace_bytes), out_bytes);
-    bool use_wide = wide.cost < narrow.cost;
-    if (force_tile_n == 128) use_wide = false;
-    if (force_tile_n == 256) use_wide = true;
-    const Choice &c = use_wide ? wide : narrow;
-    p.tile_n = use_wide ? 256 : 128;
-    p.tiles_n = use_wide ? tiles_n256 : tiles_n128;
-    p.k_iters = use_wide ? it256 : it128;
-    p.splits = c.splits;
-    p.iters_per_split = c.ips;
-    // A product cut into sixteen and more chunks of K spends a noticeable part of its time on the chunk sum (sixteen
-    // planes of the result written and read back).  Tiles of 64 rows with half as many chunks are as many work units
-    // of the same length and halve the planes: 128 x 4096 x 8192 in 75.9 us instead of 78.8, 128 x 4096 x 4096 in 42.9
-    // instead of 45.2 (with eight chunks the two are level: 128 x 8192 x 4096 73.1 against 74.5, 128 x 8192 x 8192
-    // 142.0 against 139.7).
-    // Only an even number of chunks halves into the same number of work units (an odd one would add units, and with
-    // them a round: 128 x 3000 x 40000 went from 21 chunks on 504 units to 11 on 528 and from 248 us to 378).
-    // With A stored k by m (Tdot) the 64-row tile reads 256-byte pieces of A and loses what the planes save (128 x 4096 x
-    // 8192: 77.7 us against 75.2), so the rule is for A stored m by k.
-    if (force_tile_n == 0 && a_along_k && !use_wide && p.splits >= 16 && p.splits % 2 == 0) {
-        p.tile_m = kTileMMid;
-        p.tiles_m = (M + kTileMMid - 1) / kTileMMid;
-        const int64_t half = p.splits / 2;
-        p.iters_per_split = (p.k_iters + half - 1) / half;
-        p.splits = (int)((p.k_iters + p.iters_per_split - 1) / p.iters_per_split);
-    }
-    p.units = p.tiles_m * p.tiles_n * p.splits;
-    return p;
+    return best;
 }
 
 }  // namespace cn

@@ -129,7 +129,7 @@ cn_status gemm_w8_rows(int splits, int64_t M, int64_t N, int64_t K, const float 
 
 // The product in one launch for shapes too small to fill the chip with tiles (cn_gemm_small.hip): a workgroup per
 // 32 x 32 block of the result, K split among its wavefronts.
-constexpr int64_t kSmallMaxBlocks = 512;           // of 32 x 32 results
+constexpr int64_t kSmallMaxBlocks = 256;           // of 32 x 32 results: a workgroup per compute unit (288 of them lost to the tiled kernel: 18.0 us against 11.6)
 constexpr int64_t kSmallMaxWork = (int64_t)1 << 28;  // M * N * K; half of it where the blocks are 16 x 16
 bool gemm_small_applies(int ta, int tb, int64_t M, int64_t N, int64_t K, const float *A, int64_t lda, const float *B,
                         int64_t ldb);

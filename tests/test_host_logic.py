@@ -185,6 +185,8 @@ def test_encoder_table_shape():
 
 
 def test_gemm_plan_covers_k_and_fits_workspace():
+    """Whatever the planner chooses: one of the four tile geometries, K covered by non-empty chunks, the chunk planes inside
+    the workspace, a forced geometry respected, and no tile more than twice as tall as the product when it chooses itself."""
     L = cn.lib()
     out = (C.c_int64 * 8)()
     rng = np.random.default_rng(0)
@@ -194,37 +196,70 @@ def test_gemm_plan_covers_k_and_fits_workspace():
     shapes += [tuple(int(v) for v in rng.integers(1, 3000, 3)) for _ in range(200)]
     for ws in (16 << 20, 1 << 30):
         for force in (0, 128, 256, 32, 64):
-            for (M, N, K) in shapes:
-                L.cn_host_plan_gemm(M, N, K, 256, ws, force, out)
-                tm, tn, kit, splits, ips, units, tile_n, tile_m = list(out)
-                # the 32-row tile when asked for; unasked for products of at most 64 rows and for those too
-                # small to give every compute unit two 128-row tiles even at the deepest split
-                deepest = max(1, min(64, max(1, -(-K // 32)) // 4, ws // (M * N * 4)))
-                small = -(-M // 128) * -(-N // 128) * deepest < 512
-                if force in (32, 64):
-                    assert tile_m == force
-                elif force == 0 and (M <= 64 or small):
-                    assert tile_m == (64 if (32 < M <= 64 and not small) else 32)
-                else:
-                    assert tile_m == 128
-                    # with A stored m by k, an even number of sixteen and more chunks on the 128 x 128 tile becomes
-                    # 64-row tiles with half as many: as many work units, K covered as before
-                    along = (C.c_int64 * 8)()
-                    L.cn_host_plan_gemm_rows_along_k(M, N, K, 256, ws, force, along)
-                    a = list(along)
-                    if force == 0 and tile_n == 128 and splits >= 16 and splits % 2 == 0:
-                        assert a[7] == 64 and a[6] == 128 and a[3] == splits // 2 and a[5] == units and a[0] == -(-M // 64)
-                        assert a[4] * a[3] >= a[2] and a[4] * (a[3] - 1) < a[2] and a[3] * M * N * 4 <= ws
+            for fn in (L.cn_host_plan_gemm, L.cn_host_plan_gemm_rows_along_k):
+                for (M, N, K) in shapes:
+                    fn(M, N, K, 256, ws, force, out)
+                    tm, tn, kit, splits, ips, units, tile_n, tile_m = list(out)
+                    assert (tile_m, tile_n) in ((128, 128), (128, 256), (64, 128), (32, 128))
+                    if force in (32, 64):
+                        assert tile_m == force and tile_n == 128
+                    elif force in (128, 256):
+                        assert tile_m == 128 and tile_n == force
                     else:
-                        assert a == list(out)
-                assert tile_n in (128, 256) and (force in (0, 32, 64) or tile_n == force) and (tile_m == 128 or tile_n == 128)
-                assert tm == -(-M // tile_m) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
-                assert splits >= 1 and units == tm * tn * splits
-                assert ips * splits >= kit and ips * (splits - 1) < kit  # every chunk non-empty
-                if splits > 1:
-                    assert splits * M * N * 4 <= ws
+                        assert tile_m == 32 or M > tile_m // 2
+                    assert tm == -(-M // tile_m) and tn == -(-N // tile_n) and kit == max(1, -(-K // (32 if tile_n == 128 else 16)))
+                    assert splits >= 1 and units == tm * tn * splits
+                    assert ips * splits >= kit and ips * (splits - 1) < kit  # every chunk non-empty
+                    if splits > 1:
+                        assert splits * M * N * 4 <= ws
+                        assert ips >= (8 if tile_n == 256 else 4)  # a chunk is at least 128 k deep
     L.cn_host_plan_gemm(128, 40000, 100000, 256, 1 << 30, 128, out)
     assert list(out)[:6] == [1, 313, 3125, 13, 241, 4069]
+
+
+# (tile rows, tile columns, K chunks, stages per chunk) on 256 compute units with a 1 GiB workspace, as measured best or within
+# 2 % of the best geometry on an MI355X (tests/test_gpu_planner.py holds the planner to that on the GPU; this freezes the
+# answers so that a change of a rule or a constant shows up without one).
+FROZEN_PLANS = {
+    ("dot", 128, 1024, 784): (32, 128, 5, 5),
+    ("Tdot", 784, 1024, 128): (32, 128, 1, 4),
+    ("dotT", 128, 784, 1024): (32, 128, 8, 4),
+    ("dot", 128, 40000, 100000): (128, 256, 13, 481),
+    ("dot", 128, 20000, 40000): (128, 128, 13, 97),
+    ("dot", 32, 4096, 4096): (32, 128, 8, 16),
+    ("dot", 128, 4096, 4096): (64, 128, 8, 16),
+    ("dot", 512, 4096, 4096): (64, 128, 2, 64),
+    ("dot", 128, 8192, 100000): (128, 256, 16, 391),
+    ("dot", 128, 8192, 4096): (64, 128, 4, 32),
+    ("dot", 128, 10, 4096): (32, 128, 32, 4),
+    ("Tdot", 100000, 8192, 128): (128, 256, 1, 8),
+    ("Tdot", 4096, 8192, 128): (128, 256, 1, 8),
+    ("Tdot", 4096, 10, 128): (32, 128, 1, 4),
+    ("dotT", 128, 4096, 8192): (64, 128, 8, 32),
+    ("dotT", 128, 4096, 10): (32, 128, 1, 1),
+    ("dotT", 128, 100000, 8192): (128, 256, 5, 103),
+    ("dot", 128, 3000, 40000): (128, 128, 21, 60),
+    ("dot", 128, 8192, 8192): (64, 128, 4, 64),
+    ("Tdot", 128, 8192, 4096): (128, 128, 8, 16),
+    ("Tdot", 128, 4096, 8192): (128, 128, 16, 16),
+    ("dot", 4096, 4096, 4096): (128, 256, 1, 256),
+    ("dot", 8192, 8192, 512): (128, 256, 1, 32),
+    ("dot", 32, 40000, 100000): (32, 128, 13, 241),
+    ("dot", 64, 40000, 100000): (64, 128, 13, 241),
+    ("dot", 256, 1024, 1024): (32, 128, 4, 8),
+    ("Tdot", 3000, 3000, 300): (64, 128, 1, 10),
+    ("dot", 500, 1024, 784): (32, 128, 2, 13),
+    ("Tdot", 37, 1029, 515): (32, 128, 4, 5),
+}
+
+
+def test_plans_of_the_benchmark_shapes_are_the_measured_ones():
+    L = cn.lib()
+    out = (C.c_int64 * 8)()
+    for (op, M, N, K), want in FROZEN_PLANS.items():
+        (L.cn_host_plan_gemm if op == "Tdot" else L.cn_host_plan_gemm_rows_along_k)(M, N, K, 256, 1 << 30, 0, out)
+        tm, tn, kit, splits, ips, units, tile_n, tile_m = list(out)
+        assert (tile_m, tile_n, splits, ips) == want, (op, M, N, K, (tile_m, tile_n, splits, ips), want)
 
 
 def test_tile_counters_are_tied_to_streams():
