@@ -590,6 +590,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--zero-operands", action="store_true",
                     help="profiling aid: the two products run on all-zero operands (the line is marked; not a result)")
+    ap.add_argument("--whole-rows", action="store_true",
+                    help="profiling aid: the sparse first-layer update runs every wavefront on whole rows instead of "
+                         "splitting a workgroup into code-producing and weight-streaming wavefronts (the line is marked)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build runs the un-sharded workload on a single "
@@ -601,6 +604,8 @@ def main():
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     cn.init(0)
+    if args.whole_rows:
+        cn.lib().cn_host_csr_paired_rows(0)
 
     line = {"metric": "fp32 GEMM TFLOP/s at 128x100000x40000 (%MFMA peak); 8-bit codec GB/s",
             "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -665,6 +670,8 @@ def main():
     if args.only in (None, "step"):
         torch.cuda.empty_cache()
         section("maxout_step_128x100000_8192_8192_10", lambda: bench_step(torch, cn, dev))
+    if args.whole_rows:
+        line["data"] += "; sparse update passes on whole rows (profiling aid, not the library's choice)"
     line["extra"] = extra
     print(json.dumps(line))
 

@@ -111,6 +111,8 @@ def lib():
     L.cn_host_csr_rows_workgroups_per_cu.restype = None
     L.cn_host_csr_lds_rows.argtypes = [C.c_int]
     L.cn_host_csr_lds_rows.restype = None
+    L.cn_host_csr_paired_rows.argtypes = [C.c_int]
+    L.cn_host_csr_paired_rows.restype = None
     _lib = L
     return L
 

@@ -320,13 +320,29 @@ __global__ __launch_bounds__(kT) void csr_gemm_kernel(int64_t R, int64_t N, cons
 // issued after the one it needs.  Rows with more than four nonzeros, and rows of a block beyond its first
 // 64 nonzeros, take what is missing from memory as the plain kernel does.  The sums run in the same order
 // as there.
-//   kMode 1: max |S B| only            2: codes of S B            3: codes and w += alpha * decode(codes)
-//         4: codes and RMSprop with weight update on decode(codes)  (alpha = multiplier of the mean squares)
+//   form 1: max |S B| only            2: codes of S B            3: codes and w += alpha * decode(codes)
+//        4: codes and RMSprop with weight update on decode(codes)  (alpha = multiplier of the mean squares)
+//        5, 6: what 3 and 4 do, with producing and streaming wavefronts (below)
 constexpr int kRowThreads = 256;
-// The codes-only form (kMode 2) needs no ring of weights and fits four wavefronts per SIMD: it runs 512 threads
+// The codes-only form (2) needs no ring of weights and fits four wavefronts per SIMD: it runs 512 threads
 // on one encoder table, two workgroups per compute unit (0.66 ms instead of 0.77 ms on the first-layer gradient).
-// The forms that stream the weights gain nothing from that (1.73 ms against 1.69 ms) and keep 256.
-template <int kMode> constexpr int row_threads() { return kMode == 2 ? 512 : kRowThreads; }
+// Forms 3 and 4, which stream the weights as well, gain nothing from that (1.73 ms against 1.69 ms) and keep 256.
+template <int kForm> constexpr int row_threads() { return kForm >= 5 ? 1024 : kForm == 2 ? 512 : kRowThreads; }
+// Forms 5 and 6 are forms 3 and 4 with the work split between the sixteen wavefronts of one workgroup per compute
+// unit.  A wavefront that does everything waits for its B rows (from the L2, a row ahead) with the same in-order
+// counter that its weight loads and its stores run on: each such wait also waits for every older weight load and
+// store, so the weights are never more than two rows ahead in effect, whatever the ring holds.  (Measured on the
+// first-layer gradient, 819.2 M elements: 1.71 ms; without the stores 1.08, without the weight loads 1.16, both
+// gone 0.86; taking the encoder out changed nothing.)  Here twelve wavefronts produce codes exactly as form 2 does
+// and leave each 16 x 256 patch of codes in LDS as well; four wavefronts take the patches of the round before
+// (three each), read the weights sixteen rows ahead, add the decoded values and write; their waits see nothing but
+// their own stream.  One barrier per round, the patches are double-buffered.  1.58 ms (RMSprop: 2.71 against
+// 2.93).  The two halves do not overlap fully: the producers alone take 0.88 ms, the streaming wavefronts alone
+// 1.10 (6.0 TB/s, what that mix of loads and stores reaches), and neither other splits (8 + 8, 10 + 5, 12 + 3,
+// 12 + 2) nor B rows two ahead came closer; the producers' B rows come out of an L2 that the streams keep busy.
+constexpr int kProducers = 12, kStreamers = 4, kPerStreamer = kProducers / kStreamers;
+constexpr int kPatchWords = 16 * 64;  // a patch of codes: 16 rows, one word (four codes) per lane
+static_assert(kProducers % kStreamers == 0 && (kProducers + kStreamers) * 64 == 1024, "sixteen wavefronts");
 constexpr int kRowBlock = 16;  // rows per block
 constexpr int kBAhead = 1;     // B values are requested this many rows ahead
 constexpr int kBRing = 2 * kBAhead;
@@ -346,14 +362,24 @@ __device__ __forceinline__ u32x4 as_u32x4(f32x4 v) {
     return u32x4{__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
 }
 
+// A 16-byte store whose row offset travels in a scalar register.  The compiler guards the two wait states between
+// such a store and a vector instruction that overwrites its data registers only when the scalar offset is a
+// constant; with a register there the next instruction may overwrite the data before the store has read it, and on
+// this hardware the store then wrote the new contents now and then (seen as single wrong words, the first of a
+// lane's four, under full memory load).  Here the data registers stay alive across two wait states.
+__device__ __forceinline__ void store_row_b128(u32x4 data, rsrc_t r, uint32_t lane_offset, uint32_t row_offset) {
+    __builtin_amdgcn_raw_buffer_store_b128(data, r, lane_offset, row_offset, kRowAuxNt);
+    asm volatile("s_nop 1" ::"v"(data) : "memory");  // ordered behind the store, and the data registers are its operands
+}
+
 struct RowBlockMeta {
     int rp;    // lane l: row_ptr[first row + l], l <= 16
     int c;     // lane l: column index of the block's nonzero l
     float v;   // lane l: its value
 };
 
-template <int kMode>
-__global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_rows_kernel(
+template <int kForm>
+__global__ __launch_bounds__(row_threads<kForm>(), kForm == 2 ? 4 : 1) void csr_rows_kernel(
     int64_t R, int64_t N, const int32_t *__restrict__ row_ptr, const int32_t *__restrict__ col_idx,
     const float *__restrict__ vals, const float *__restrict__ B, int64_t ldb, int64_t col_blocks, uint32_t *amax_out,
     const float *__restrict__ precision_ptr, uint8_t *__restrict__ codes, float *__restrict__ w, int64_t ldw, float alpha,
@@ -362,6 +388,10 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     EncodeShared &sh = *reinterpret_cast<EncodeShared *>(smem_raw);
     float *dlut = reinterpret_cast<float *>(smem_raw + sizeof(EncodeShared));  // decode table times alpha
+    uint32_t *patches = reinterpret_cast<uint32_t *>(smem_raw + sizeof(EncodeShared) + 256 * sizeof(float));  // [2][kProducers][16][64]
+    constexpr bool kPaired = kForm >= 5;
+    constexpr int kMode = kPaired ? 2 : kForm;  // what this wavefront's rows do; the paired forms' producers are form 2
+    constexpr int kWaves = kPaired ? kProducers : row_threads<kForm>() / 64;  // wavefronts that take units
     const int t = threadIdx.x;
     float precision = 0.0f;
     bool exact_only = false;
@@ -369,7 +399,7 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
     if (kMode >= 2) {
         precision = *precision_ptr;
         exact_only = !build_table(sh, steps, step_count, precision, table);
-        if (kMode == 4) alpha = 1.0f;  // RMSprop takes the decoded gradient itself; `alpha` then carries the multiplier
+        if (kForm == 4 || kForm == 6) alpha = 1.0f;  // RMSprop takes the decoded gradient itself; `alpha` then carries the multiplier
         if (t < 126) {
             const float v = table[t] * precision;
             dlut[t] = alpha * v;
@@ -390,11 +420,14 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
     };
 
     const int lane = t & 63;
+    // the wavefront's number as a scalar: what follows from it (the unit, its buffer descriptors) then lives in scalar
+    // registers, and no buffer instruction has to be wrapped in a loop over the lanes' descriptors
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const int32_t nnz = row_ptr[R];
     const int32_t last = nnz > 0 ? nnz - 1 : 0;
     const int64_t row_blocks = (R + kRowBlock - 1) / kRowBlock;
     const int64_t units = row_blocks * col_blocks;
-    const int64_t unit_stride = (int64_t)gridDim.x * (row_threads<kMode>() / 64);
+    const int64_t unit_stride = (int64_t)gridDim.x * kWaves;
     uint32_t amax = 0;
 
     auto load_rp = [&](int64_t row0) -> int {
@@ -409,7 +442,7 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
         v = nnz > 0 ? vals[j] : 0.0f;
     };
 
-    const int64_t unit_first = (int64_t)blockIdx.x * (row_threads<kMode>() / 64) + (t >> 6);
+    const int64_t unit_first = (int64_t)blockIdx.x * kWaves + wave;
     const uint32_t b_row_bytes = (uint32_t)(ldb * (int64_t)sizeof(float));  // B spans less than 4 GiB on this path
     const char *Bbytes = reinterpret_cast<const char *>(B);
     // Everything a row touches is addressed through buffer descriptors: the part of an address that is the same for all
@@ -438,8 +471,8 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
         p.lane_off = (uint32_t)(nc * (int64_t)sizeof(float));
         const int64_t c0 = (int64_t)cb * 256, cols_here = N - c0 < 256 ? N - c0 : 256;
         p.w_lane = p.live ? (uint32_t)(4 * lane) : 0u;
-        if (kMode >= 3) p.rw = row_rsrc(w + p.row0 * ldw + c0, (uint32_t)(((p.rows - 1) * ldw + cols_here) * (int64_t)sizeof(float)));
-        if (kMode == 4) p.rr = row_rsrc(rms + p.row0 * ldw + c0, (uint32_t)(((p.rows - 1) * ldw + cols_here) * (int64_t)sizeof(float)));
+        if (kForm >= 3) p.rw = row_rsrc(w + p.row0 * ldw + c0, (uint32_t)(((p.rows - 1) * ldw + cols_here) * (int64_t)sizeof(float)));
+        if (kForm == 4 || kForm == 6) p.rr = row_rsrc(rms + p.row0 * ldw + c0, (uint32_t)(((p.rows - 1) * ldw + cols_here) * (int64_t)sizeof(float)));
         if (kMode >= 2) p.rc = row_rsrc(codes + p.row0 * N + c0, (uint32_t)((p.rows - 1) * N + cols_here));
         return p;
     };
@@ -476,6 +509,81 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
         if (kMode == 4) dst2 = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(p.rr, 4u * p.w_lane, row, kRowAuxNt));
     };
 
+    if constexpr (kPaired) {
+        if (wave >= kProducers) {  // a streaming wavefront: the patches its three producers left a round ago
+            constexpr bool kRms = kForm == 6;
+            constexpr int kDepth = kRms ? 8 : 16;  // rows requested ahead (of the weights, and of the mean squares)
+            const int s = wave - kProducers;
+            const int64_t rounds = (units + unit_stride - 1) / unit_stride;
+            const int64_t mine = (int64_t)blockIdx.x * kProducers + s * kPerStreamer;
+            auto patch_at = [&](int64_t round, int j) -> UnitPos {
+                const int64_t unit = round * unit_stride + mine + j;
+                if (unit < units) return locate(unit);
+                UnitPos p;  // beyond the last unit: loads give zero and stores go nowhere
+                p.row0 = 0;
+                p.rows = 0;
+                p.live = false;
+                p.lane_off = 0;
+                p.w_lane = 0;
+                p.rw = row_rsrc(w, 0);
+                p.rr = row_rsrc(w, 0);
+                p.rc = row_rsrc(codes, 0);
+                return p;
+            };
+            auto request = [&](const UnitPos &p, int u, f32x4 &dw, f32x4 &dr) {
+                int uu = u < p.rows ? u : p.rows - 1;
+                uu = uu < 0 ? 0 : uu;
+                const uint32_t row = (uint32_t)uu * w_row_bytes;
+                dw = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(p.rw, 4u * p.w_lane, row, kRowAuxNt));
+                if (kRms) dr = as_f32x4(__builtin_amdgcn_raw_buffer_load_b128(p.rr, 4u * p.w_lane, row, kRowAuxNt));
+            };
+            f32x4 sw[kDepth], sr[kRms ? kDepth : 1];
+            UnitPos pos = patch_at(0, 0);
+#pragma unroll
+            for (int u = 0; u < kDepth; ++u) request(pos, u, sw[u], sr[kRms ? u : 0]);
+            __syncthreads();  // round 0: the producers' first patches
+            for (int64_t round = 1; round <= rounds; ++round) {
+                const uint32_t *left = patches + (((round - 1) & 1) * kProducers + s * kPerStreamer) * kPatchWords + lane;
+                for (int j = 0; j < kPerStreamer; ++j) {
+                    const UnitPos nxt = j + 1 < kPerStreamer ? patch_at(round - 1, j + 1) : patch_at(round, 0);
+                    // The loads and stores of a row are issued whatever the row is, so that every wait counts exactly
+                    // what was issued behind the load it needs; a store that must not happen gets an offset beyond
+                    // the patch and is dropped.
+                    const uint32_t lane_bytes = pos.live ? 16u * (uint32_t)lane : 0xffffffffu;
+#pragma unroll
+                    for (int u = 0; u < kRowBlock; ++u) {
+                        const uint32_t c = left[j * kPatchWords + u * 64];
+                        const float g[4] = {dlut[c & 255u], dlut[(c >> 8) & 255u], dlut[(c >> 16) & 255u], dlut[c >> 24]};
+                        f32x4 wv = sw[u % kDepth];
+                        const uint32_t at = u < pos.rows ? lane_bytes : 0xffffffffu;
+                        if (kRms) {  // kRMSprop_with_weight_update on the decoded gradient, operation by operation
+                            f32x4 rv = sr[u % kDepth];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const float r2 = (rms_multiplier * rv[e]) + ((g[e] * g[e]) * one_minus);
+                                const float step = rate * (g[e] / (sqrtf(r2) + 1.0e-08f));
+                                rv[e] = r2;
+                                wv[e] = wv[e] - step;
+                            }
+                            store_row_b128(as_u32x4(rv), pos.rr, at, (uint32_t)u * w_row_bytes);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) wv[e] = wv[e] + g[e];
+                        }
+                        store_row_b128(as_u32x4(wv), pos.rw, at, (uint32_t)u * w_row_bytes);
+                        if (u + kDepth < kRowBlock)
+                            request(pos, u + kDepth, sw[u % kDepth], sr[kRms ? u % kDepth : 0]);
+                        else
+                            request(nxt, u + kDepth - kRowBlock, sw[u % kDepth], sr[kRms ? u % kDepth : 0]);
+                    }
+                    pos = nxt;
+                }
+                __syncthreads();  // the patches of this round are complete, those of the round before are free
+            }
+            return;
+        }
+    }
+    int64_t round = 0;  // paired forms: rounds this wavefront has produced
     f32x4 b[kBRing][kFixed];
     constexpr int kWRing = kMode == 4 ? 4 : 8;  // weights (and mean squares) this many rows ahead
     f32x4 wr[kWRing], rr[kMode == 4 ? kWRing : 1];
@@ -545,9 +653,9 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
                     }
                 } else {
                     const uint32_t c0 = encode(acc.x), c1 = encode(acc.y), c2 = encode(acc.z), c3 = encode(acc.w);
-                    if (pos.live)
-                        __builtin_amdgcn_raw_buffer_store_b32(c0 | (c1 << 8) | (c2 << 16) | (c3 << 24), pos.rc, pos.w_lane,
-                                                              (uint32_t)u * (uint32_t)N, kRowAuxNt);
+                    const uint32_t four = c0 | (c1 << 8) | (c2 << 16) | (c3 << 24);
+                    if (pos.live) __builtin_amdgcn_raw_buffer_store_b32(four, pos.rc, pos.w_lane, (uint32_t)u * (uint32_t)N, kRowAuxNt);
+                    if (kPaired) patches[((round & 1) * kProducers + wave) * kPatchWords + u * 64 + lane] = four;
                     if (kMode == 4) {  // kRMSprop_with_weight_update on the decoded gradient, operation by operation
                         f32x4 wv = wr[u % kWRing], rv = rr[u % kWRing];
                         const float g[4] = {dlut[c0], dlut[c1], dlut[c2], dlut[c3]};
@@ -559,8 +667,8 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
                             wv[e] = wv[e] - step;
                         }
                         if (pos.live) {
-                            __builtin_amdgcn_raw_buffer_store_b128(as_u32x4(rv), pos.rr, 4u * pos.w_lane, (uint32_t)u * w_row_bytes, kRowAuxNt);
-                            __builtin_amdgcn_raw_buffer_store_b128(as_u32x4(wv), pos.rw, 4u * pos.w_lane, (uint32_t)u * w_row_bytes, kRowAuxNt);
+                            store_row_b128(as_u32x4(rv), pos.rr, 4u * pos.w_lane, (uint32_t)u * w_row_bytes);
+                            store_row_b128(as_u32x4(wv), pos.rw, 4u * pos.w_lane, (uint32_t)u * w_row_bytes);
                         }
                     }
                     if (kMode == 3) {
@@ -570,7 +678,7 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
                         wv.z = wv.z + dlut[c2];
                         wv.w = wv.w + dlut[c3];
                         if (pos.live)
-                            __builtin_amdgcn_raw_buffer_store_b128(as_u32x4(wv), pos.rw, 4u * pos.w_lane, (uint32_t)u * w_row_bytes, kRowAuxNt);
+                            store_row_b128(as_u32x4(wv), pos.rw, 4u * pos.w_lane, (uint32_t)u * w_row_bytes);
                     }
                 }
             }
@@ -585,6 +693,14 @@ __global__ __launch_bounds__(row_threads<kMode>(), kMode == 2 ? 4 : 1) void csr_
             }
             if (u == kRowBlock - kBAhead - 1) m_next = prepare(next);
         }
+        if (kPaired) {
+            __syncthreads();  // this round's patches are complete
+            ++round;
+        }
+    }
+    if (kPaired) {  // a wavefront with a unit less than the others, and the round in which only the streamers work
+        const int64_t rounds = (units + unit_stride - 1) / unit_stride;
+        for (; round <= rounds; ++round) __syncthreads();
     }
     if (kMode == 1) {  // every lane of every wave arrives here
 #pragma unroll
@@ -1028,6 +1144,7 @@ cn_status cn_csr_from_dense_f32(const float *A, int64_t rows, int64_t cols, int6
 static bool g_strip_kernel = true;  // the test hooks below switch these kernels off to compare
 static int g_rows_per_cu = 0;  // tuning hook: workgroups per compute unit of the fused row passes, 0 = their own figure
 static bool g_lds_rows = true;
+static bool g_paired_rows = true;  // fused update passes: producing and streaming wavefronts (forms 5, 6) instead of forms 3, 4
 
 static cn_status csr_gemm(const char *who, int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
                           const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, float *absmax_out,
@@ -1118,6 +1235,7 @@ cn_status cn_host_exclusive_scan(const int32_t *counts_device, int64_t n, int32_
 }
 void cn_host_csr_rows_workgroups_per_cu(int per_cu) { g_rows_per_cu = per_cu > 0 ? per_cu : 0; }
 void cn_host_csr_lds_rows(int enabled) { g_lds_rows = enabled != 0; }
+void cn_host_csr_paired_rows(int enabled) { g_paired_rows = enabled != 0; }
 
 cn_status cn_csr_gemm_f32(int64_t R, int64_t Cc, int64_t N, const int32_t *row_ptr, const int32_t *col_idx,
                           const float *vals, const float *B, int64_t ldb, float *out, int64_t ldo, void *stream) {
@@ -1184,6 +1302,7 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
     if (s != CN_OK) return s;
     hipStream_t st = (hipStream_t)stream;
     const int lds = (int)sizeof(EncodeShared) + 256 * (int)sizeof(float);
+    const int lds_paired = lds + 2 * kProducers * kPatchWords * (int)sizeof(uint32_t);
     static OncePerDevice configured;
     if (configured.first(ctx->device)) {
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_gemm_coded_kernel),
@@ -1194,6 +1313,10 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
         CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<4>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<5>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_paired));
+        CN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&csr_rows_kernel<6>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_paired));
     }
     const bool vec = Cc > 0 && Cc * ldb < (1LL << 30) && aligned(B, 16) && ldb % 4 == 0 && N % 4 == 0 && aligned(codes, 4) &&
                      (!w || (aligned(w, 16) && ldw % 4 == 0)) && (!rms || aligned(rms, 16));
@@ -1201,13 +1324,16 @@ static cn_status csr_gemm_coded(const char *who, int64_t R, int64_t Cc, int64_t 
         const int64_t col_blocks = (N + 255) / 256;
         const int64_t units = ((R + kRowBlock - 1) / kRowBlock) * col_blocks;
         const bool codes_only = !rms && !w;
-        const int threads = codes_only ? row_threads<2>() : kRowThreads;
-        const int64_t per_wg = threads / 64;
-        // the encoder table allows three workgroups of 256 threads per compute unit, the registers two of 512
-        int64_t grid = (int64_t)ctx->num_cu * (g_rows_per_cu > 0 ? g_rows_per_cu : (codes_only ? 2 : 3));
+        const bool paired = !codes_only && g_paired_rows;
+        const int threads = paired ? row_threads<5>() : codes_only ? row_threads<2>() : kRowThreads;
+        const int64_t per_wg = paired ? kProducers : threads / 64;
+        // the encoder table allows three workgroups of 256 threads per compute unit, the registers two of 512;
+        // a paired workgroup fills a compute unit
+        int64_t grid = (int64_t)ctx->num_cu * (paired ? 1 : g_rows_per_cu > 0 ? g_rows_per_cu : (codes_only ? 2 : 3));
         if (grid > (units + per_wg - 1) / per_wg) grid = (units + per_wg - 1) / per_wg;
-        auto kernel = rms ? csr_rows_kernel<4> : (w ? csr_rows_kernel<3> : csr_rows_kernel<2>);
-        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), lds, st, R, N, row_ptr, col_idx, vals, B, ldb, col_blocks,
+        auto kernel = paired ? (rms ? csr_rows_kernel<6> : csr_rows_kernel<5>)
+                             : rms ? csr_rows_kernel<4> : (w ? csr_rows_kernel<3> : csr_rows_kernel<2>);
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3((unsigned)threads), paired ? lds_paired : lds, st, R, N, row_ptr, col_idx, vals, B, ldb, col_blocks,
                            (uint32_t *)nullptr, precision_device, codes, w, ldw, alpha, rms, rate, ctx->xsteps, ctx->xstep_count,
                            ctx->table, (uint32_t)(((Cc - 1) * ldb + N) * (int64_t)sizeof(float)));
     } else {

@@ -88,6 +88,10 @@ void cn_host_absmax_compress_spin_limit(int spins);
  * LDS (maximum only); they then run on the general kernels, which the tests compare against. */
 void cn_host_csr_strip_kernel(int enabled);
 void cn_host_csr_lds_rows(int enabled);
+/* 0 = the passes that turn a sparse product into codes and update the weights with them run every wavefront on
+ * whole rows (product, codes, weights) instead of splitting a workgroup into wavefronts that produce codes and
+ * wavefronts that stream the weights.  Same bits. */
+void cn_host_csr_paired_rows(int enabled);
 /* Workgroups per compute unit of the passes that turn a sparse product into codes (and updates); 0 = their own. */
 void cn_host_csr_rows_workgroups_per_cu(int per_cu);
 /* sums_device[0 .. n] = exclusive prefix sums of counts_device[0 .. n - 1] (n + 1 entries; in place allowed) as the CSR

@@ -18,14 +18,18 @@ def dev():
     return torch.device("cuda:0")
 
 
-@pytest.fixture(autouse=True, params=["b_in_lds", "b_from_l2"])
+@pytest.fixture(autouse=True, params=["b_in_lds", "b_from_l2", "whole_rows"])
 def short_row_kernel(request, dev):
     """The max-only pass has two kernels (B strip in LDS when B has at most 128 rows, B from the L2
-    otherwise): every test runs with the first one allowed and with it switched off."""
+    otherwise), the passes that also update the weights two forms (a workgroup split into wavefronts that
+    produce codes and wavefronts that stream the weights, or every wavefront on whole rows): every test runs
+    with the library's choices, with the first kernel switched off, and with the split switched off."""
     from clusternet_amd import _lib as L
-    L.lib().cn_host_csr_lds_rows(1 if request.param == "b_in_lds" else 0)
+    L.lib().cn_host_csr_lds_rows(0 if request.param == "b_from_l2" else 1)
+    L.lib().cn_host_csr_paired_rows(0 if request.param == "whole_rows" else 1)
     yield
     L.lib().cn_host_csr_lds_rows(1)
+    L.lib().cn_host_csr_paired_rows(1)
 
 
 def _t(a, dev):
@@ -151,7 +155,8 @@ def test_gather_product_absmax_of_an_empty_result(dev):
 
 
 @pytest.mark.parametrize("R,Cc,N,density", [(2000, 128, 1024, 0.02), (777, 64, 4100, 0.05), (37, 211, 19, 0.05),
-                                            (5, 9, 1, 0.5), (301, 16, 2052, 0.0), (4096, 128, 8192, 0.02)])
+                                            (5, 9, 1, 0.5), (301, 16, 2052, 0.0), (4096, 128, 8192, 0.02),
+                                            (2005, 100, 8196, 0.03)])  # the last two: several rounds of a split workgroup
 @pytest.mark.parametrize("with_update", [False, True])
 def test_product_to_codes_and_update_equals_the_three_separate_calls(dev, R, Cc, N, density, with_update):
     """max|S B| without storing, then codes (and the weight update) straight from the recomputed product:
@@ -189,7 +194,7 @@ def test_product_to_codes_and_update_equals_the_three_separate_calls(dev, R, Cc,
 
 
 @pytest.mark.parametrize("R,Cc,N,density", [(2000, 128, 1024, 0.02), (777, 64, 4100, 0.05), (37, 211, 19, 0.05),
-                                            (301, 16, 2052, 0.0)])
+                                            (301, 16, 2052, 0.0), (2005, 100, 8196, 0.03)])
 def test_product_to_codes_and_rmsprop_equals_the_separate_calls(dev, R, Cc, N, density):
     """The RMSprop form: codes, running mean squares and weights bit for bit those of csr_gemm, absmax,
     compression_8bit and rmsprop_update on the codes; and those of the CPU checker."""
