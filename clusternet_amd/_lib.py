@@ -51,6 +51,7 @@ def lib():
     L.cn_gemm_f32_noalloc.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp]
     L.cn_gemm_f32_absmax.argtypes = [C.c_int, C.c_int, i64, i64, i64, vp, i64, vp, i64, vp, i64, vp, vp]
     L.cn_gemm_f32_w8.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, vp, i64, vp]
+    L.cn_gemm_c8c8_add.argtypes = [i64, i64, i64, vp, i64, vp, i64, f32, f32, vp, i64, vp]
     L.cn_csr_from_dense_f32.argtypes = [vp, i64, i64, i64, C.c_int, vp, vp, vp, i64, C.POINTER(i64), vp]
     L.cn_csr_gemm_f32.argtypes = [i64, i64, i64, vp, vp, vp, vp, i64, vp, i64, vp]
     L.cn_csr_transpose.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, vp, vp]
@@ -209,6 +210,21 @@ def gemm_w8(A, W, scale, out=None):
         raise CnError(2, "Matrix size error")
     check(lib().cn_gemm_f32_w8(M, N, K, A.data_ptr(), _ld(A), W.data_ptr(), _ld(W), float(scale),
                                out.data_ptr(), _ld(out), _stream()))
+    return out
+
+
+def gemm_c8c8_add(A, B, precision_a, precision_b, out):
+    """out += decodeA(A) decodeB(B): A uint8 codes M x K, B uint8 codes K x N, with kDot8bit's two tables."""
+    import torch
+    _need(A, torch.uint8, "A")
+    _need(B, torch.uint8, "B")
+    _need(out, torch.float32, "out")
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2 or tuple(out.shape) != (M, N):
+        raise CnError(2, "Matrix size error")
+    check(lib().cn_gemm_c8c8_add(M, N, K, A.data_ptr(), _ld(A), B.data_ptr(), _ld(B), float(precision_a),
+                                 float(precision_b), out.data_ptr(), _ld(out), _stream()))
     return out
 
 

@@ -23,7 +23,7 @@ HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-ffp-contr
              "-Wno-unused-command-line-argument",
              # the direct-to-LDS loads set M0 inside their inline assembly and say so
              "-Wno-inline-asm"]
-SOURCES = ["cn_runtime.cpp", "cn_encode_lut.cpp", "cn_gemm_plan.cpp", "cn_codec.hip", "cn_gemm.hip", "cn_gemm_w8_rows.hip", "cn_gemm_small.hip",
+SOURCES = ["cn_runtime.cpp", "cn_encode_lut.cpp", "cn_gemm_plan.cpp", "cn_codec.hip", "cn_gemm.hip", "cn_gemm_w8_rows.hip", "cn_gemm_small.hip", "cn_gemm_c8c8.hip",
            "cn_layers.hip", "cn_update.hip", "cn_sparse.hip"]
 
 

@@ -105,47 +105,11 @@ Matrix *ClusterNet::dot8bit_weights(Matrix *A, Matrix *B, float precisionB) {
     return out;
 }
 
-// The two decode tables of kDot8bit (source/clusterKernels.cu:1725-1739), literally.
-static void dot8bit_tables(float precisionA, float precisionB, float (&a)[256], float (&b)[256]) {
-    float t[126];
-    cn_throw_on_error(cn_table_get(t));
-    for (int i = 0; i < 256; ++i) a[i] = b[i] = 0.0f;  // 126 + 128 = 254 and 127 + 128 = 255 are set below
-    for (int i = 0; i < 126; ++i) {
-        a[i] = t[i] * precisionA;
-        a[i + 128] = -a[i];
-        b[i] = t[i] * precisionB;
-        b[i + 128] = -b[i];
-    }
-    a[126] = 0.0f;
-    b[126] = 0.0f;
-    a[127] = precisionA;
-    b[127] = -precisionA;
-    a[254] = -0.0f;
-    b[254] = -0.0f;
-    a[255] = precisionB;
-    b[255] = -precisionB;
-}
-
+// out += decodeA(A) decodeB(B) with kDot8bit's own two tables (source/clusterKernels.cu:1725-1739): one launch.
 void ClusterNet::dot8bit(Matrix *A, Matrix *B, float precisionA, float precisionB, Matrix *out) {
     if (checkMatrixOperation(A, B, out, OP_N, OP_N, 1) == 1) throw "Matrix *size error:\n";
-    const long long M = A->rows, K = A->cols, N = B->cols;
-    if (M == 0 || N == 0) return;
-    float ta[256], tb[256];
-    dot8bit_tables(precisionA, precisionB, ta, tb);
-    // temporaries: the two tables, both operands decoded, the product
-    void *p = nullptr;
-    const size_t floats = 512 + (size_t)(M * K + K * N + M * N);
-    cn_throw_on_error(cn_malloc(&p, floats * sizeof(float)));
-    float *lut_a = (float *)p, *lut_b = lut_a + 256, *da = lut_b + 256, *db = da + M * K, *prod = db + K * N;
-    cn_status s = cn_memcpy_h2d(lut_a, ta, sizeof(ta));
-    if (s == CN_OK) s = cn_memcpy_h2d(lut_b, tb, sizeof(tb));
-    if (s == CN_OK) s = cn_decode_8bit_lut(A->char_data, lut_a, (size_t)(M * K), da, nullptr);
-    if (s == CN_OK) s = cn_decode_8bit_lut(B->char_data, lut_b, (size_t)(K * N), db, nullptr);
-    if (s == CN_OK) s = cn_gemm_f32(0, 0, M, N, K, da, K, db, N, prod, N, nullptr);
-    if (s == CN_OK) s = cn_sgd_update_f32(out->data, prod, -1.0f, (size_t)(M * N), nullptr);  // out -= -1 * product
-    if (s == CN_OK) s = cn_synchronize(nullptr);
-    cn_free(p);
-    cn_throw_on_error(s);
+    cn_throw_on_error(cn_gemm_c8c8_add(out->rows, out->cols, A->cols, A->char_data, A->cols, B->char_data, B->cols,
+                                       precisionA, precisionB, out->data, out->cols, nullptr));
 }
 Matrix *ClusterNet::dot8bit(Matrix *A, Matrix *B, float precisionA, float precisionB) {
     Matrix *out = zeros(A->rows, B->cols);

@@ -118,6 +118,18 @@ cn_status cn_gemm_f32_w8(int64_t M, int64_t N, int64_t K, const float *A_device,
                          const uint8_t *W_device, int64_t ldw, float scale, float *C_device,
                          int64_t ldc, void *stream);
 
+/* C[M x N] += decodeA(A[M x K]) decodeB(B[K x N]), both operands 8-bit codes (row-major, lda >= K, ldb >= N), in one
+ * launch with nothing staged in memory.  Replaces ClusterNet::dot8bit and dot8bit_shared (source/clusterNet.cpp:1409-1431
+ * -> source/basicOps.cu:1455-1472 -> kDot8bit, source/clusterKernels.cu:1717-1762, and kDot8bit_shared, :1764-1843),
+ * which add the product to `out`.  The two decode tables are those kernels' own, entry by entry (:1725-1739): entry
+ * i < 126 is table[i] * precision of its operand and entry i + 128 its negative; code 126 decodes to 0 and 254 to -0 in
+ * both; 127 gives precision_a in A and -precision_a in B, 255 gives precision_b in A and -precision_b in B.  The sum over
+ * k runs in fp32 in the order of the matrix instructions, not one k after the other as in kDot8bit: results agree to
+ * fp32 rounding of a K-term sum, and bit for bit where a row of A holds a single code that decodes to non-zero. */
+cn_status cn_gemm_c8c8_add(int64_t M, int64_t N, int64_t K, const uint8_t *A_codes_device, int64_t lda,
+                           const uint8_t *B_codes_device, int64_t ldb, float precision_a, float precision_b,
+                           float *C_device, int64_t ldc, void *stream);
+
 /* *out_device = max_i |x_i| (n == 0 gives -1, the start value of the reference's reduction; a NaN
  * input gives NaN).  One pass, no temporary.
  * Replaces the abs + max pair callers use to obtain `precision` (source/basicOps.cu:810-822 and

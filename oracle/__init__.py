@@ -56,6 +56,9 @@ def _load():
     lib.cn_oracle_gemm_w8_f64acc.argtypes = [_c.c_int64, _c.c_int64, _c.c_int64, _f32p,
                                              _c.c_int64, _u8p, _c.c_int64, _c.c_float, _f32p,
                                              _c.c_int64]
+    lib.cn_oracle_dot8bit_tables.argtypes = [_c.c_float, _c.c_float, _f32p, _f32p]
+    lib.cn_oracle_dot8bit.argtypes = [_u8p, _u8p, _f32p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_float, _c.c_float,
+                                      _c.c_void_p]
     lib.cn_oracle_add_row_vector.argtypes = [_f32p, _f32p, _c.c_int64, _c.c_int64, _f32p]
     lib.cn_oracle_maxout.argtypes = [_f32p, _c.c_int64, _c.c_int64, _c.c_int, _f32p, _f32p]
     lib.cn_oracle_expand_to_maxout_grad.argtypes = [_f32p, _f32p, _c.c_int64, _c.c_int64,
@@ -209,6 +212,26 @@ def gemm_w8(A, W, scale):
     C = np.empty((M, N), np.float32)
     _lib.cn_oracle_gemm_w8_f64acc(M, N, K, A, K, W, N, float(scale), C, N)
     return C
+
+
+def dot8bit_tables(precision_a, precision_b):
+    ta, tb = np.empty(256, np.float32), np.empty(256, np.float32)
+    _lib.cn_oracle_dot8bit_tables(float(precision_a), float(precision_b), ta, tb)
+    return ta, tb
+
+
+def dot8bit(A, B, precision_a, precision_b, out=None):
+    """(out + decodeA(A) decodeB(B), sum_k |a||b|): kDot8bit's sum, term by term in fp32, added to `out` (zeros if None)."""
+    A = np.ascontiguousarray(A, dtype=np.uint8)
+    B = np.ascontiguousarray(B, dtype=np.uint8)
+    M, K = A.shape
+    K2, N = B.shape
+    if K != K2:
+        raise ValueError("inner dimensions differ")
+    res = np.zeros((M, N), np.float32) if out is None else np.array(out, dtype=np.float32, order="C")
+    mag = np.empty((M, N), np.float64)
+    _lib.cn_oracle_dot8bit(A, B, res, M, K, N, float(precision_a), float(precision_b), mag.ctypes.data)
+    return res, mag
 
 
 def add_row_vector(A, v):

@@ -38,6 +38,10 @@
  *   cn_oracle_gemm_w8            C = A * decode(W codes, scale) with decode == cn_oracle_decompress
  *                                (no counterpart kernel in the reference; its nearest relatives
  *                                are kDot8bit / kDot8bit_shared, source/clusterKernels.cu:1717-1843)
+ *   cn_oracle_dot8bit            source/clusterKernels.cu:1717-1762 (kDot8bit): the two tables, then out +=
+ *                                term by term in ascending k.  The reference has no test of it; pinned by
+ *                                closed forms (constant operands, one-hot rows against cn_oracle_decompress,
+ *                                the special codes read off the source lines), tests/test_oracle_gemm.py
  *   helpers of the training step source/clusterKernels.cu:706-718 (bias add), :1432-1458
  *                                (maxout), :1481-1495 (expand to maxout grad), :651-688 (softmax);
  *                                definitions taken from the brute-force expectations in
@@ -357,6 +361,51 @@ void cn_oracle_gemm_w8_f64acc(int64_t M, int64_t N, int64_t K, const float *A, i
         for (int64_t n = 0; n < N; ++n) C[m * ldc + n] = (float)row[n];
         free(row);
     }
+}
+
+/* The two decode tables of kDot8bit, statement by statement (source/clusterKernels.cu:1725-1739; kDot8bit_shared builds
+ * the same two, :1775-1792). */
+void cn_oracle_dot8bit_tables(float pa, float pb, float ta[256], float tb[256]) {
+    float t[126];
+    cn_oracle_table(t);
+    for (int i = 0; i < 256; ++i) ta[i] = tb[i] = 0.0f; /* slots the kernel never writes (none is reachable: see below) */
+    for (int i = 0; i < 126; ++i) {
+        ta[i] = t[i] * pa;
+        ta[i + 128] = -ta[i];
+        tb[i] = t[i] * pb;
+        tb[i + 128] = -tb[i];
+    }
+    ta[126] = 0.0f;
+    tb[126] = 0.0f;
+    ta[127] = pa;
+    tb[127] = -pa;
+    ta[254] = -0.0f;
+    tb[254] = -0.0f;
+    ta[255] = pb;
+    tb[255] = -pb;
+}
+
+/* out[M x N] += decodeA(A) decodeB(B) as kDot8bit computes it (source/clusterKernels.cu:1744-1752): for every output
+ * the products are added to out one k after the other, in fp32.  Row-major here; the kernel's column-major indices
+ * A[Acol * rowsA + Arow], B[colsA * Bcol + Acol], out[Bcol * rowsA + Arow] name the same elements of the same matrices.
+ * out_abs (optional) receives sum_k |a||b| in fp64, the scale of the rounding error of any summation order.
+ * Pinned by closed forms (tests/test_oracle_gemm.py): the reference holds no test of dot8bit. */
+void cn_oracle_dot8bit(const uint8_t *A, const uint8_t *B, float *out, int64_t M, int64_t K, int64_t N, float pa, float pb,
+                       double *out_abs) {
+    float ta[256], tb[256];
+    cn_oracle_dot8bit_tables(pa, pb, ta, tb);
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            float acc = out[m * N + n];
+            double mag = 0.0;
+            for (int64_t k = 0; k < K; ++k) {
+                const float p = ta[A[m * K + k]] * tb[B[k * N + n]];
+                acc = acc + p;
+                mag += fabs((double)p);
+            }
+            out[m * N + n] = acc;
+            if (out_abs) out_abs[m * N + n] = mag;
+        }
 }
 
 /* ---- helpers of the training step (row-major, flat). */

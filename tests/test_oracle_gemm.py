@@ -130,3 +130,50 @@ def test_cpu_port_gemm_all_transpositions_and_accumulation():
     for k0 in range(0, K, 128):   # the port's own K slabs: the accumulated product adds in the same order
         oracle.port_gemm(A[:, k0:k0 + 128], B[k0:k0 + 128], out=acc, accumulate=True, lda=K)
     assert np.array_equal(whole.view(np.uint32), acc.view(np.uint32))
+
+
+def test_dot8bit_restatement_is_pinned_by_closed_forms():
+    """The reference has no test of dot8bit / dot8bit_shared, so the restatement of kDot8bit
+    (source/clusterKernels.cu:1717-1762) is held to what its source lines fix:
+      * the special codes of the two tables, read off :1731-1738 (126 -> 0, 254 -> -0 in both; 127 -> precisionA in A and
+        -precisionA in B; 255 -> precisionB in A and -precisionB in B), and the ordinary entries against the codec's
+        decode table (same t[i] * precision, :1727-1730 against :1141-1146);
+      * constant operands: K equal products, exact when they are powers of two;
+      * a row of A with one code that decodes to non-zero among codes that decode to zero picks out a decoded row of B,
+        scaled, bit for bit, and adds it to what out held;
+      * linearity in out (out + P from zero equals out0 + P to one rounding) and the fp64 product of the decoded
+        operands within the bound of a K-term fp32 sum."""
+    pa, pb = 0.75, 2.5
+    ta, tb = oracle.dot8bit_tables(pa, pb)
+    assert ta[126] == 0 and not np.signbit(ta[126]) and tb[126] == 0 and not np.signbit(tb[126])
+    assert ta[254] == 0 and np.signbit(ta[254]) and tb[254] == 0 and np.signbit(tb[254])
+    assert (ta[127], tb[127], ta[255], tb[255]) == (np.float32(pa), np.float32(-pa), np.float32(pb), np.float32(-pb))
+    la, lb = oracle.decode_lut(pa), oracle.decode_lut(pb)
+    ordinary = np.r_[0:126, 128:254]
+    assert np.array_equal(ta[ordinary].view(np.uint32), la[ordinary].view(np.uint32))
+    assert np.array_equal(tb[ordinary].view(np.uint32), lb[ordinary].view(np.uint32))
+    # constant operands: codes 127 (A: 0.75) and 255 (B: -2.5), K = 16 -> 16 * -1.875 = -30 exactly
+    out, mag = oracle.dot8bit(np.full((3, 16), 127, np.uint8), np.full((16, 5), 255, np.uint8), pa, pb)
+    assert np.all(out == np.float32(-30.0)) and np.all(mag == 30.0)
+    # one-hot rows: row m of A holds code 127 (-> pa) at k = m and 126 / 254 (-> +0 / -0) elsewhere
+    rng = np.random.default_rng(8)
+    K, N = 40, 33
+    B = rng.integers(0, 256, (K, N)).astype(np.uint8)
+    A = np.where(rng.random((K, K)) < 0.5, 126, 254).astype(np.uint8)
+    A[np.arange(K), np.arange(K)] = 127
+    out0 = rng.normal(size=(K, N)).astype(np.float32)
+    out, _ = oracle.dot8bit(A, B, pa, pb, out0)
+    want = out0 + np.float32(pa) * tb[B]          # a single product and a single addition per output, both fp32
+    assert np.array_equal(out.view(np.uint32), want.astype(np.float32).view(np.uint32))
+    # general case against the fp64 product of the decoded operands
+    M, K, N = 37, 150, 29
+    A = rng.integers(0, 256, (M, K)).astype(np.uint8)
+    B = rng.integers(0, 256, (K, N)).astype(np.uint8)
+    out0 = rng.normal(size=(M, N)).astype(np.float32)
+    out, mag = oracle.dot8bit(A, B, pa, pb, out0)
+    ref = out0.astype(np.float64) + ta[A].astype(np.float64) @ tb[B].astype(np.float64)
+    # the magnitudes are sums of the fp32 products: equal to the fp64 ones to the rounding of a product
+    assert np.allclose(mag, np.abs(ta[A].astype(np.float64)) @ np.abs(tb[B].astype(np.float64)), rtol=2.0 ** -23)
+    assert float((np.abs(out - ref) / (mag + np.abs(out0))).max()) <= K * 2.0 ** -24
+    from_zero, _ = oracle.dot8bit(A, B, pa, pb)
+    assert float((np.abs(out - (out0 + from_zero)) / (mag + np.abs(out0))).max()) <= K * 2.0 ** -24
