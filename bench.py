@@ -30,10 +30,10 @@ FLOP1 = 2.0 * M * N1 * K1
 FLOP2 = 2.0 * M * N2 * N1
 
 # HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (profiles/gemm_and_codec_kernels_hbm_traffic.txt): FETCH_SIZE 7955760 KiB x 2.0 (the factor
+# file (profiles/gemm_and_codec_kernels_hbm_traffic.txt): FETCH_SIZE 7956620 KiB x 2.0 (the factor
 # that makes the same counter read 3276.8 MB on a 3276.8 MB device-to-device copy) + WRITE_SIZE
 # 260000 KiB x 1.0.  Algorithmic bytes of the same launch: 16.07e9.
-TRAFFIC_BYTES_GEMM1 = 7955760 * 1024 * 2.0 + 260000 * 1024 * 1.0
+TRAFFIC_BYTES_GEMM1 = 7956620 * 1024 * 2.0 + 260000 * 1024 * 1.0
 
 
 def log(*a):
