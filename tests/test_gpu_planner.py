@@ -5,7 +5,8 @@ planned form may not be more than 7 % slower than the best of them.  Shapes: the
 configurations (source/clusterNet.cpp:230-298 as called from source/Layer.cpp:256,327,334), the shapes the planner's own
 rules were fitted on, and a ragged set.  Kernels of a few microseconds are timed replayed from a HIP graph (the host
 cannot launch them as fast as they run), longer ones with an event pair round every call.  The table of the run is
-written to gpurun_out/planner_choice_table.txt."""
+written to planner_choice_table.txt in the directory CN_TEST_OUTPUT names (default: the run's output folder at the
+top of the checkout)."""
 import os
 
 import numpy as np
@@ -146,7 +147,7 @@ def test_planned_geometry_is_within_seven_percent_of_the_best(dev):
     finally:
         L.cn_host_gemm_small(1)
         L.cn_host_force_gemm_tile_n(0)
-    out_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    out_dir = os.environ.get("CN_TEST_OUTPUT") or os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
     try:
         os.makedirs(out_dir, exist_ok=True)
         with open(os.path.join(out_dir, "planner_choice_table.txt"), "w") as f:
