@@ -277,3 +277,13 @@ def test_tile_counters_are_tied_to_streams():
     assert got[:5] == [0, 1, 0, 2, 1]
     assert got[5:5 + 29] == list(range(3, 32)) and got[5 + 29:5 + 40] == [-1] * 11
     assert got[-2:] == [2, 0]
+
+
+def test_bench_refuses_more_than_one_gpu_before_touching_any():
+    """The benchmark measures one GPU; asked for more it says so and exits, before it imports torch or the library."""
+    import subprocess
+    import sys
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode != 0 and proc.stdout.strip() == ""
+    assert "one GPU" in proc.stderr and "--gpus 2" in proc.stderr
