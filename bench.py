@@ -535,6 +535,69 @@ def cpu_codec_baseline():
             "compress_GBps": 5.0 * x.size / tc / 1e9, "decompress_GBps": 5.0 * x.size / td / 1e9}
 
 
+def cpu_port_maxout_step():
+    """The maxout training step of the fifth configuration on the host cores, once, composed from the CPU port's pieces the
+    way the reference composes its kernels (dense batch; source/Layer.cpp:256-334, source/DeepNeuralNetwork.cpp:334-339):
+    three products with bias and maxout (softmax at the end), the backward products with the maxout expansions, and for
+    every weight gradient abs-max, compression_8bit, decompression_8bit and the update.  Products and codec run on all
+    OpenMP threads; the helpers on 128-row matrices and the update (numpy) on one.  Only the step itself is timed, not
+    the making of the 3.3 GB of weights."""
+    import numpy as np
+    import torch
+    import oracle
+    B, D, H, O, pool, rate = 128, 100000, 8192, 10, 2, 0.01
+    g = torch.Generator().manual_seed(3)
+    X = (torch.rand((B, D), generator=g) * (torch.rand((B, D), generator=g) < 0.02)).numpy()
+    # the large weights: a cheap pattern instead of 819 M random numbers (their values do not matter to the time)
+    W1 = np.empty((D, H), np.float32)
+    W1[:] = ((np.arange(H, dtype=np.float32) % 17.0) - 8.0) * np.float32(0.001)
+    W2 = ((torch.rand((H // pool, H), generator=g) - 0.5) * 0.05).numpy()
+    W3 = ((torch.rand((H // pool, O), generator=g) - 0.5) * 0.05).numpy()
+    b1, b2, b3 = np.zeros(H, np.float32), np.zeros(H, np.float32), np.zeros(O, np.float32)
+    onehot = np.zeros((B, O), np.float32)
+    onehot[np.arange(B), np.arange(B) % O] = 1.0
+    t = {}
+
+    def timed(name, fn):
+        t0 = time.perf_counter()
+        r = fn()
+        t[name] = t.get(name, 0.0) + time.perf_counter() - t0
+        return r
+
+    def layer(x, W, b):
+        return oracle.maxout(oracle.add_row_vector(oracle.port_gemm(x, W), b), pool)
+
+    def forward():
+        h1, a1 = layer(X, W1, b1)
+        h2, a2 = layer(h1, W2, b2)
+        return oracle.softmax(oracle.add_row_vector(oracle.port_gemm(h2, W3), b3)), (h1, a1, h2, a2)
+
+    def backward(p, cache):
+        h1, a1, h2, a2 = cache
+        e3 = p - onehot
+        gW3 = oracle.port_gemm(h2, e3, True, False)
+        e2 = oracle.expand_to_maxout_grad(oracle.port_gemm(e3, W3, False, True), a2, pool)
+        gW2 = oracle.port_gemm(h1, e2, True, False)
+        e1 = oracle.expand_to_maxout_grad(oracle.port_gemm(e2, W2, False, True), a1, pool)
+        return oracle.port_gemm(X, e1, True, False), gW2, gW3
+
+    def update(w, grad):
+        prec = oracle.port_absmax(grad.reshape(-1))
+        dec = oracle.port_decompress(oracle.port_compress(grad.reshape(-1), prec), prec)
+        np.multiply(dec, np.float32(rate), out=dec)
+        np.subtract(w.reshape(-1), dec, out=w.reshape(-1))
+
+    oracle.port_gemm(X[:, :1024].copy(), np.ones((1024, 512), np.float32))  # thread pool warm-up
+    p, cache = timed("forward_s", forward)
+    grads = timed("backward_s", lambda: backward(p, cache))
+    for w, grad in zip((W1, W2, W3), grads):
+        timed("codec_and_update_s", lambda: update(w, grad))
+    total = sum(t.values())
+    return dict(t, step_s=total, cores=oracle.num_threads(), kind="port",
+                note="one step, host clock; dense 128 x 100000 batch with 2 % nonzeros, layers 100000 -> 8192 (pool 2) -> 8192 (pool 2) "
+                     "-> 10; products and codec on all threads, helpers and the update on one")
+
+
 def cpu_port_configs():
     """The CPU port on the other configurations, all OpenMP threads: the three products of the 784 -> 1024 layer (batch 128), the
     128 x 40000 round-trip tensor (abs-max, compression, decompression), and decompression of 4096 x 4096 weights followed by the
@@ -659,6 +722,7 @@ def main():
         if not args.no_cpu and args.only is None and "error" not in extra["codec"]:
             extra["codec"]["cpu_port"] = cpu_codec_baseline()
             section("cpu_port_other_configs", cpu_port_configs)
+            section("cpu_port_maxout_step", cpu_port_maxout_step)
     if args.only in (None, "codec"):
         section("layout_100000x8192", lambda: bench_layout(torch, cn, dev))
         torch.cuda.empty_cache()
